@@ -1,0 +1,113 @@
+/*
+ * Stage-level C ABI of libtsnecuda (MI355X / gfx950 build).
+ *
+ * One entry point per stage of the FIt-SNE pipeline, each taking plain DEVICE
+ * pointers and sizes, so that a stage can be driven and checked in isolation on
+ * identical inputs.  Every function returns 0 on success and non-zero on error;
+ * tsne_hip_last_error() then returns a description.  `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream); calls are asynchronous on that
+ * stream unless stated otherwise.
+ *
+ * Layouts (all fp32 / int32):
+ *   points      num_points x num_dims, row-major
+ *   indices     num_points x num_neighbors, row-major, neighbour 0 is the point itself
+ *   sq_dist     same shape, squared L2 distances, ascending per row
+ *   pij         same shape
+ *   embedding   2 * num_points: all x coordinates, then all y coordinates
+ *   forces      same layout as embedding
+ *
+ * Each declaration cites the reference interface it stands in for (paths are
+ * relative to the CannyLab/tsne-cuda checkout).
+ */
+#ifndef TSNECUDA_TSNE_STAGES_H_
+#define TSNECUDA_TSNE_STAGES_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tsne_hip_plan tsne_hip_plan;
+
+/* Description of the last error raised on the calling thread ("" if none). */
+const char *tsne_hip_last_error(void);
+
+/* Exact k nearest neighbours by squared L2 distance, self first with distance
+ * exactly 0, the rest ascending by (distance, index).  Distances are
+ * accumulated in fp32 over ascending dimension with one fused multiply-add per
+ * dimension.  Replaces tsnecuda::util::KNearestNeighbors
+ * (src/util/distance_utils.cu:79-121, include/util/distance_utils.h) together
+ * with PostprocessNeighborIndices (src/util/distance_utils.cu:139-154): indices
+ * are int32 from the start.  num_neighbors must be <= num_points.
+ * Synchronises the stream before returning. */
+int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neighbors, int *indices,
+                 float *sq_dist, void *stream);
+
+/* In-place division of n values by their largest absolute value.
+ * Replaces tsnecuda::util::MaxNormalizeDeviceVector (src/util/math_utils.cu:66-74). */
+int tsne_hip_max_normalize(float *values, int64_t n, void *stream);
+
+/* Per-row search for the Gaussian precision that gives the requested
+ * perplexity; writes row-normalised conditional probabilities.
+ * Replaces tsnecuda::SearchPerplexity (src/kernels/perplexity_search.cu:81-141,
+ * include/kernels/perplexity_search.h).  betas (optional, may be NULL)
+ * receives the precision each row ended with. */
+int tsne_hip_perplexity(const float *sq_dist, int num_points, int num_neighbors, float perplexity,
+                        float epsilon, float *pij, float *betas, void *stream);
+
+/* Pattern-restricted symmetrisation P[i,s] = (p[i,s] + sum_{t: idx[j,t]==i} p[j,t]) / 2N,
+ * j = idx[i,s].  Replaces tsnecuda::util::SymmetrizeMatrixV2
+ * (src/util/math_utils.cu:269-308). */
+int tsne_hip_symmetrize(const float *pij_non_symmetric, const int *indices, int num_points,
+                        int num_neighbors, float *pij, void *stream);
+
+/* Scratch memory and constants for the gradient loop of one problem size.
+ * n_boxes_per_dim is 130 in the reference (src/fit_tsne.cu:246-272); other
+ * values (2..170) exist for testing on reduced grids.  Stands in for the
+ * buffer/plan setup of src/fit_tsne.cu:274-342.  The plan is bound to `device`. */
+int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors, int n_boxes_per_dim,
+                         int device);
+void tsne_hip_plan_destroy(tsne_hip_plan *plan);
+
+/* attr_i = sum_s P[i,s] (y_i - y_j) / (1 + |y_i - y_j|^2), j = idx[i,s].
+ * Replaces tsnecuda::ComputeAttractiveForcesV3 (src/kernels/attr_forces.cu:186-240). */
+int tsne_hip_attractive(tsne_hip_plan *plan, const float *pij, const int *indices, const float *embedding,
+                        float *attractive_forces, void *stream);
+
+/* FFT-interpolated repulsive forces and the normalisation Z = sum_i z_i - N
+ * (written to the device scalar *normalization).  Replaces, for one iteration,
+ * ComputeChargesQij + minmax + PrecomputeFFT2D + NbodyFFT2D +
+ * ComputeRepulsiveForces (src/fit_tsne.cu:425-469, src/kernels/rep_forces.cu,
+ * src/kernels/nbodyfft.cu).  Optional outputs (may be NULL): node_charges and
+ * node_potentials, (3*n_boxes)^2 x 4 floats each; point_potentials, N x 4. */
+int tsne_hip_repulsive(tsne_hip_plan *plan, const float *embedding, float *repulsive_forces,
+                       float *normalization, float *node_charges, float *node_potentials,
+                       float *point_potentials, void *stream);
+
+/* Gains / momentum update of all 2N coordinates; zeroes both force arrays.
+ * normalization is a device scalar.  Replaces tsnecuda::ApplyForces
+ * (src/kernels/apply_forces.cu:59-82). */
+int tsne_hip_update(tsne_hip_plan *plan, float *embedding, float *attractive_forces, float *repulsive_forces,
+                    float *gains, float *old_forces, float eta, const float *normalization, float momentum,
+                    float exaggeration, void *stream);
+
+/* Gradient steps [step_begin, step_end) of the loop at src/fit_tsne.cu:402-580
+ * with no host synchronisation inside: bounds, Z and the schedule switch at
+ * force_magnify_iters stay on the device.  embedding, gains and old_forces are
+ * updated in place.  normalization (device scalar, may be NULL) receives the Z
+ * of the last step. */
+int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, float *embedding, float *gains,
+                     float *old_forces, int step_begin, int step_end, int force_magnify_iters, float eta,
+                     float pre_exaggeration_momentum, float post_exaggeration_momentum,
+                     float early_exaggeration, float *normalization, void *stream);
+
+/* Squared L2 norm of n device floats into the device scalar *out
+ * (tsnecuda::util::L2NormDeviceVector without the root, src/util/math_utils.cu:51-57). */
+int tsne_hip_sum_squares(tsne_hip_plan *plan, const float *values, int64_t n, float *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TSNECUDA_TSNE_STAGES_H_ */

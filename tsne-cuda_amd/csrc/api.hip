@@ -1,0 +1,260 @@
+// Stage-level C ABI: argument checks, plan lifetime, and the fused gradient loop.
+#include <cmath>
+#include <cstdarg>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "../../include/tsnecuda/tsne_stages.h"
+#include "plan.h"
+#include "stages.h"
+
+namespace tsnehip {
+
+namespace {
+thread_local char g_error[512] = "";
+}
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+const char *last_error() { return g_error; }
+
+bool sync_kernels_enabled() {
+    static const bool enabled = []() {
+        const char *v = std::getenv("TSNE_SYNC_KERNELS");
+        return v != nullptr && std::atoi(v) != 0;
+    }();
+    return enabled;
+}
+
+namespace {
+
+LagrangeConsts make_lagrange() {
+    // fp32 arithmetic in the order of src/fit_tsne.cu:303-321.
+    LagrangeConsts lc;
+    const float h = 1 / (float)kInterp;
+    lc.spacing[0] = h / 2;
+    for (int i = 1; i < kInterp; ++i) lc.spacing[i] = lc.spacing[i - 1] + h;
+    for (int i = 0; i < kInterp; ++i) {
+        lc.denom[i] = 1;
+        for (int j = 0; j < kInterp; ++j)
+            if (i != j) lc.denom[i] *= lc.spacing[i] - lc.spacing[j];
+    }
+    return lc;
+}
+
+int check_plan(const tsne_hip_plan *p, const char *who) {
+    if (!p) {
+        set_error("%s: plan is null", who);
+        return 1;
+    }
+    int dev = -1;
+    TSNE_TRY(hipGetDevice(&dev));
+    if (dev != p->device) {
+        set_error("%s: plan belongs to device %d but device %d is current", who, p->device, dev);
+        return 1;
+    }
+    return 0;
+}
+
+#define TSNE_REQUIRE(cond, ...)      \
+    do {                             \
+        if (!(cond)) {               \
+            set_error(__VA_ARGS__);  \
+            return 1;                \
+        }                            \
+    } while (0)
+
+}  // namespace
+}  // namespace tsnehip
+
+using namespace tsnehip;
+
+extern "C" {
+
+const char *tsne_hip_last_error(void) { return last_error(); }
+
+int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neighbors, int *indices,
+                 float *sq_dist, void *stream) {
+    TSNE_REQUIRE(points && indices && sq_dist, "knn: null pointer argument");
+    return run_knn(points, num_points, num_dims, num_neighbors, indices, sq_dist, (hipStream_t)stream);
+}
+
+int tsne_hip_max_normalize(float *values, int64_t n, void *stream) {
+    TSNE_REQUIRE(values && n > 0, "max_normalize: need a non-empty array");
+    hipStream_t s = (hipStream_t)stream;
+    float *scratch = nullptr;
+    TSNE_TRY(hipMalloc(&scratch, sizeof(float)));
+    int rc = launch_max_normalize(values, n, scratch, s);
+    if (!rc && hipStreamSynchronize(s) != hipSuccess) {
+        set_error("max_normalize: stream synchronisation failed");
+        rc = 1;
+    }
+    (void)hipFree(scratch);
+    return rc;
+}
+
+int tsne_hip_perplexity(const float *sq_dist, int num_points, int num_neighbors, float perplexity,
+                        float epsilon, float *pij, float *betas, void *stream) {
+    TSNE_REQUIRE(sq_dist && pij, "perplexity: null pointer argument");
+    TSNE_REQUIRE(num_points > 0 && num_neighbors > 0, "perplexity: empty problem (%d x %d)", num_points,
+                 num_neighbors);
+    TSNE_REQUIRE(perplexity > 0.0f, "perplexity: target must be positive (got %g)", (double)perplexity);
+    return launch_perplexity(sq_dist, num_points, num_neighbors, perplexity, epsilon, pij, betas,
+                             (hipStream_t)stream);
+}
+
+int tsne_hip_symmetrize(const float *pij_non_symmetric, const int *indices, int num_points,
+                        int num_neighbors, float *pij, void *stream) {
+    TSNE_REQUIRE(pij_non_symmetric && indices && pij, "symmetrize: null pointer argument");
+    TSNE_REQUIRE(pij_non_symmetric != pij, "symmetrize: input and output must not alias");
+    TSNE_REQUIRE(num_points > 0 && num_neighbors > 0, "symmetrize: empty problem (%d x %d)", num_points,
+                 num_neighbors);
+    return launch_symmetrize(pij_non_symmetric, indices, num_points, num_neighbors, pij, (hipStream_t)stream);
+}
+
+void tsne_hip_plan_destroy(tsne_hip_plan *p) {
+    if (!p) return;
+    (void)hipFree(p->yxy);
+    (void)hipFree(p->node_charges);
+    (void)hipFree(p->node_potentials);
+    (void)hipFree(p->row_spectra);
+    (void)hipFree(p->col_results);
+    (void)hipFree(p->kernel_rows);
+    (void)hipFree(p->twiddles);
+    (void)hipFree(p->scalars);
+    (void)hipFree(p->attr);
+    (void)hipFree(p->rep);
+    delete p;
+}
+
+int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors, int n_boxes_per_dim,
+                         int device) {
+    TSNE_REQUIRE(plan, "plan_create: null output pointer");
+    *plan = nullptr;
+    TSNE_REQUIRE(num_points > 0, "plan_create: num_points must be positive (got %d)", num_points);
+    TSNE_REQUIRE(num_neighbors > 0, "plan_create: num_neighbors must be positive (got %d)", num_neighbors);
+    TSNE_REQUIRE(n_boxes_per_dim >= 2 && n_boxes_per_dim <= kMaxBoxes,
+                 "plan_create: n_boxes_per_dim must be in [2, %d] (got %d)", kMaxBoxes, n_boxes_per_dim);
+    TSNE_TRY(hipSetDevice(device));
+    tsne_hip_plan *p = new (std::nothrow) tsne_hip_plan();
+    TSNE_REQUIRE(p, "plan_create: out of host memory");
+    p->num_points = num_points;
+    p->num_neighbors = num_neighbors;
+    p->n_boxes = n_boxes_per_dim;
+    p->n_nodes = n_boxes_per_dim * kInterp;
+    p->device = device;
+    p->lagrange = make_lagrange();
+    const size_t G2 = (size_t)p->n_nodes * p->n_nodes;
+    const size_t spec = (size_t)2 * kFft * kNodePad;
+    const size_t N = (size_t)num_points;
+    bool ok = hipMalloc(&p->yxy, sizeof(float2) * N) == hipSuccess &&
+              hipMalloc(&p->node_charges, sizeof(float4) * G2) == hipSuccess &&
+              hipMalloc(&p->node_potentials, sizeof(float4) * G2) == hipSuccess &&
+              hipMalloc(&p->row_spectra, sizeof(float2) * spec) == hipSuccess &&
+              hipMalloc(&p->col_results, sizeof(float2) * spec) == hipSuccess &&
+              hipMalloc(&p->kernel_rows, sizeof(float) * (size_t)(kFft / 2 + 1) * kNodePad) == hipSuccess &&
+              hipMalloc(&p->twiddles, sizeof(float2) * kFft) == hipSuccess &&
+              hipMalloc(&p->scalars, sizeof(LoopScalars)) == hipSuccess &&
+              hipMalloc(&p->attr, sizeof(float) * 2 * N) == hipSuccess &&
+              hipMalloc(&p->rep, sizeof(float) * 2 * N) == hipSuccess;
+    if (ok) {
+        std::vector<float2> tw(kFft);
+        for (int k = 0; k < kFft; ++k) {
+            const double ang = -2.0 * M_PI * (double)k / (double)kFft;
+            tw[k] = make_float2((float)std::cos(ang), (float)std::sin(ang));
+        }
+        ok = hipMemcpy(p->twiddles, tw.data(), sizeof(float2) * kFft, hipMemcpyHostToDevice) == hipSuccess &&
+             hipMemset(p->node_charges, 0, sizeof(float4) * G2) == hipSuccess &&
+             hipMemset(p->row_spectra, 0, sizeof(float2) * spec) == hipSuccess &&
+             hipMemset(p->col_results, 0, sizeof(float2) * spec) == hipSuccess &&
+             hipMemset(p->kernel_rows, 0, sizeof(float) * (size_t)(kFft / 2 + 1) * kNodePad) == hipSuccess &&
+             hipMemset(p->scalars, 0, sizeof(LoopScalars)) == hipSuccess &&
+             hipMemset(p->attr, 0, sizeof(float) * 2 * N) == hipSuccess &&
+             hipMemset(p->rep, 0, sizeof(float) * 2 * N) == hipSuccess;
+    }
+    if (!ok) {
+        set_error("plan_create: device allocation or initialisation failed: %s",
+                  hipGetErrorString(hipGetLastError()));
+        tsne_hip_plan_destroy(p);
+        return 1;
+    }
+    *plan = p;
+    return 0;
+}
+
+int tsne_hip_attractive(tsne_hip_plan *plan, const float *pij, const int *indices, const float *embedding,
+                        float *attractive_forces, void *stream) {
+    if (check_plan(plan, "attractive")) return 1;
+    TSNE_REQUIRE(pij && indices && embedding && attractive_forces, "attractive: null pointer argument");
+    hipStream_t s = (hipStream_t)stream;
+    if (launch_pack_xy(plan, embedding, s)) return 1;
+    return launch_attractive(plan, pij, indices, attractive_forces, s);
+}
+
+int tsne_hip_repulsive(tsne_hip_plan *plan, const float *embedding, float *repulsive_forces,
+                       float *normalization, float *node_charges, float *node_potentials,
+                       float *point_potentials, void *stream) {
+    if (check_plan(plan, "repulsive")) return 1;
+    TSNE_REQUIRE(embedding && repulsive_forces && normalization, "repulsive: null pointer argument");
+    hipStream_t s = (hipStream_t)stream;
+    if (launch_bounds(plan, embedding, 0, s)) return 1;
+    if (launch_repulsive(plan, embedding, 0, repulsive_forces, point_potentials, node_charges, s)) return 1;
+    if (node_potentials)
+        TSNE_TRY(hipMemcpyAsync(node_potentials, plan->node_potentials,
+                                sizeof(float4) * (size_t)plan->n_nodes * plan->n_nodes, hipMemcpyDeviceToDevice,
+                                s));
+    return launch_finish_z(plan, normalization, s);
+}
+
+int tsne_hip_update(tsne_hip_plan *plan, float *embedding, float *attractive_forces, float *repulsive_forces,
+                    float *gains, float *old_forces, float eta, const float *normalization, float momentum,
+                    float exaggeration, void *stream) {
+    if (check_plan(plan, "update")) return 1;
+    TSNE_REQUIRE(embedding && attractive_forces && repulsive_forces && gains && old_forces && normalization,
+                 "update: null pointer argument");
+    return launch_update(plan, embedding, attractive_forces, repulsive_forces, gains, old_forces, eta,
+                         normalization, momentum, exaggeration, -1, (hipStream_t)stream);
+}
+
+int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, float *embedding, float *gains,
+                     float *old_forces, int step_begin, int step_end, int force_magnify_iters, float eta,
+                     float pre_exaggeration_momentum, float post_exaggeration_momentum,
+                     float early_exaggeration, float *normalization, void *stream) {
+    if (check_plan(plan, "iterate")) return 1;
+    TSNE_REQUIRE(pij && indices && embedding && gains && old_forces, "iterate: null pointer argument");
+    TSNE_REQUIRE(step_begin <= step_end, "iterate: step range [%d, %d) is reversed", step_begin, step_end);
+    if (step_begin == step_end) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    // Bounds and the interleaved copy of the starting embedding; from then on
+    // the update kernel keeps both current.
+    int slot = 0;
+    if (launch_bounds(plan, embedding, slot, s)) return 1;
+    if (launch_pack_xy(plan, embedding, s)) return 1;
+    for (int step = step_begin; step < step_end; ++step) {
+        // Schedule of src/fit_tsne.cu:416-420.
+        const bool late = step >= force_magnify_iters;
+        const float momentum = late ? post_exaggeration_momentum : pre_exaggeration_momentum;
+        const float exaggeration = late ? 1.0f : early_exaggeration;
+        if (launch_repulsive(plan, embedding, slot, plan->rep, nullptr, nullptr, s)) return 1;
+        if (launch_attractive(plan, pij, indices, plan->attr, s)) return 1;
+        if (normalization && step == step_end - 1 && launch_finish_z(plan, normalization, s)) return 1;
+        if (launch_update(plan, embedding, plan->attr, plan->rep, gains, old_forces, eta, nullptr, momentum,
+                          exaggeration, slot ^ 1, s))
+            return 1;
+        slot ^= 1;
+    }
+    return 0;
+}
+
+int tsne_hip_sum_squares(tsne_hip_plan *plan, const float *values, int64_t n, float *out, void *stream) {
+    if (check_plan(plan, "sum_squares")) return 1;
+    TSNE_REQUIRE(values && out && n > 0, "sum_squares: need a non-empty array and an output");
+    return launch_sum_squares(values, n, out, (hipStream_t)stream);
+}
+
+}  // extern "C"

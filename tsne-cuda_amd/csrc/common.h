@@ -1,0 +1,86 @@
+// Shared host/device helpers for the gfx950 kernels of libtsnecuda.
+#ifndef TSNE_HIP_COMMON_H_
+#define TSNE_HIP_COMMON_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+namespace tsnehip {
+
+// Error reporting: stage functions return non-zero and leave a message here.
+void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+const char *last_error();
+
+// TSNE_SYNC_KERNELS=1 makes every launch synchronise, as the reference's
+// TSNE_MAYBE_SYNC does (src/include/util/cuda_utils.h:46-70).
+bool sync_kernels_enabled();
+
+#define TSNE_TRY(expr)                                                                              \
+    do {                                                                                            \
+        hipError_t tsne_err_ = (expr);                                                              \
+        if (tsne_err_ != hipSuccess) {                                                              \
+            ::tsnehip::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(tsne_err_),      \
+                                 __FILE__, __LINE__);                                               \
+            return 1;                                                                               \
+        }                                                                                           \
+    } while (0)
+
+// After a kernel launch: surface launch errors; optionally synchronise.
+#define TSNE_LAUNCHED(stream)                                                                       \
+    do {                                                                                            \
+        TSNE_TRY(hipGetLastError());                                                                \
+        if (::tsnehip::sync_kernels_enabled()) TSNE_TRY(hipStreamSynchronize(stream));              \
+    } while (0)
+
+inline int div_up(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+constexpr int kWave = 64;
+
+#ifdef __HIPCC__
+// Order-preserving map between float and uint32 so min/max can use integer atomics.
+__device__ __forceinline__ unsigned int float_to_ordered(float f) {
+    const unsigned int u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float ordered_to_float(unsigned int u) {
+    return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
+}
+
+template <int WIDTH>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int m = WIDTH / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, kWave);
+    return v;
+}
+template <int WIDTH>
+__device__ __forceinline__ float group_min(float v) {
+#pragma unroll
+    for (int m = WIDTH / 2; m > 0; m >>= 1) v = fminf(v, __shfl_xor(v, m, kWave));
+    return v;
+}
+template <int WIDTH>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+    for (int m = WIDTH / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));
+    return v;
+}
+#endif  // __HIPCC__
+
+// Per-iteration device scalars shared by the gradient-loop kernels.
+// Two bound slots alternate between iterations: the update kernel of step s
+// accumulates the bounds that step s+1 reads.
+struct LoopScalars {
+    unsigned int min_enc[2];  // ordered-uint encoding of the smallest coordinate
+    unsigned int max_enc[2];  // ... and of the largest
+    float z_sum;              // sum_i z_i of the current step (Z = z_sum - N)
+    float sumsq;              // scratch for the gradient-norm reduction
+    float vmax;               // scratch for max-normalisation
+    float pad;
+};
+
+}  // namespace tsnehip
+
+#endif  // TSNE_HIP_COMMON_H_

@@ -1,0 +1,193 @@
+// Max-normalisation and per-row perplexity search for gfx950.
+//
+// Semantics: src/util/math_utils.cu:66-74 and
+// src/kernels/perplexity_search.cu:10-141 of the reference.  The reference
+// iterates all rows in lock-step (<= 200 rounds of: exponentiate nnz values,
+// two cuBLAS row reductions, an entropy transform, a per-row update kernel and
+// a host-side "all found" reduction).  Rows never interact, so here a group of
+// lanes owns a row, keeps its distances in registers and runs the whole
+// bisection privately: the distances are read once and the probabilities
+// written once.
+#include "plan.h"
+
+#include <algorithm>
+#include <cfloat>
+
+namespace tsnehip {
+
+namespace {
+
+__global__ __launch_bounds__(256) void abs_max_kernel(const float *__restrict__ v, int64_t n, float *out) {
+    float m = 0.0f;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (int64_t)gridDim.x * blockDim.x)
+        m = fmaxf(m, fabsf(v[t]));
+    m = group_max<kWave>(m);
+    // Non-negative floats order like their bit patterns.
+    if ((threadIdx.x & (kWave - 1)) == 0) atomicMax(reinterpret_cast<unsigned int *>(out), __float_as_uint(m));
+}
+
+__global__ __launch_bounds__(256) void divide_kernel(float *__restrict__ v, int64_t n, const float *denom) {
+    const float d = *denom;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (int64_t)gridDim.x * blockDim.x)
+        v[t] = v[t] / d;
+}
+
+__global__ void zero_scalar_kernel(float *p) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *p = 0.0f;
+}
+
+// thrust_transform_functions.h:32-37: x*log(x) with NaN/Inf mapped to 0.
+__device__ __forceinline__ float entropy_term(float v) {
+    const float e = v * logf(v);
+    return (e != e || isinf(e)) ? 0.0f : e;
+}
+
+// One row per LANES-lane group, VPL values per lane held in registers.
+template <int LANES, int VPL>
+__global__ __launch_bounds__(256) void perplexity_kernel(const float *__restrict__ sq_dist, int N, int K,
+                                                         float log_target, float eps, float *__restrict__ pij,
+                                                         float *__restrict__ betas) {
+#pragma clang fp contract(off)
+    constexpr int kRowsPerBlock = 256 / LANES;
+    const int row = blockIdx.x * kRowsPerBlock + threadIdx.x / LANES;
+    const int lane = threadIdx.x % LANES;
+    const bool live = row < N;
+    const size_t base = (size_t)(live ? row : 0) * K;
+
+    float d[VPL];
+    bool self[VPL];
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+        const int s = lane + v * LANES;
+        d[v] = (live && s < K) ? sq_dist[base + s] : 0.0f;
+        // perplexity_search.cu:32: neighbour 0 at distance 0 is the point itself.
+        self[v] = (s == 0 && d[v] == 0.0f);
+    }
+
+    float beta = 1.0f, lo = -FLT_MAX, hi = FLT_MAX;
+    float p[VPL];
+    float sum = 1.0f;
+    bool done = !live;
+    for (int it = 0; it < 200; ++it) {
+        if (!done) {
+            float ls = 0.0f, le = 0.0f;
+#pragma unroll
+            for (int v = 0; v < VPL; ++v) {
+                const int s = lane + v * LANES;
+                float pv = 0.0f;
+                if (s < K && !self[v]) pv = expf(-beta * d[v]);
+                p[v] = pv;
+                ls += pv;
+                if (s < K) le += entropy_term(pv);
+            }
+            sum = group_sum<LANES>(ls);
+            const float ent = group_sum<LANES>(le);
+            const float H = (-ent / sum) + logf(sum);
+            const float diff = H - log_target;
+            const bool found = (diff < eps && -diff < eps);
+            if (found || it == 199) {
+                done = true;
+            } else if (diff > 0) {
+                lo = beta;
+                beta = (hi == FLT_MAX || hi == -FLT_MAX) ? beta * 2.0f : (beta + hi) / 2.0f;
+            } else {
+                hi = beta;
+                beta = (lo == -FLT_MAX || lo == FLT_MAX) ? beta / 2.0f : (beta + lo) / 2.0f;
+            }
+        }
+        if (__all(done)) break;
+    }
+    if (live) {
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            const int s = lane + v * LANES;
+            if (s < K) pij[base + s] = p[v] / sum;
+        }
+        if (betas && lane == 0) betas[row] = beta;
+    }
+}
+
+// Any K: one wave per row, distances re-read from memory every round.
+__global__ __launch_bounds__(256) void perplexity_generic_kernel(const float *__restrict__ sq_dist, int N, int K,
+                                                                 float log_target, float eps,
+                                                                 float *__restrict__ pij,
+                                                                 float *__restrict__ betas) {
+#pragma clang fp contract(off)
+    const int row = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    if (row >= N) return;
+    const size_t base = (size_t)row * K;
+    float beta = 1.0f, lo = -FLT_MAX, hi = FLT_MAX, sum = 1.0f;
+    for (int it = 0; it < 200; ++it) {
+        float ls = 0.0f, le = 0.0f;
+        for (int s = lane; s < K; s += kWave) {
+            const float dv = sq_dist[base + s];
+            const float pv = (s == 0 && dv == 0.0f) ? 0.0f : expf(-beta * dv);
+            ls += pv;
+            le += entropy_term(pv);
+        }
+        sum = group_sum<kWave>(ls);
+        const float ent = group_sum<kWave>(le);
+        const float H = (-ent / sum) + logf(sum);
+        const float diff = H - log_target;
+        const bool found = (diff < eps && -diff < eps);
+        if (found || it == 199) break;
+        if (diff > 0) {
+            lo = beta;
+            beta = (hi == FLT_MAX || hi == -FLT_MAX) ? beta * 2.0f : (beta + hi) / 2.0f;
+        } else {
+            hi = beta;
+            beta = (lo == -FLT_MAX || lo == FLT_MAX) ? beta / 2.0f : (beta + lo) / 2.0f;
+        }
+    }
+    for (int s = lane; s < K; s += kWave) {
+        const float dv = sq_dist[base + s];
+        const float pv = (s == 0 && dv == 0.0f) ? 0.0f : expf(-beta * dv);
+        pij[base + s] = pv / sum;
+    }
+    if (betas && lane == 0) betas[row] = beta;
+}
+
+}  // namespace
+
+// scratch: one device float.
+int launch_max_normalize(float *values, int64_t n, float *scratch, hipStream_t s) {
+    zero_scalar_kernel<<<1, 64, 0, s>>>(scratch);
+    TSNE_LAUNCHED(s);
+    const int blocks = std::max(1, (int)std::min<int64_t>(div_up(n, 256 * 4), 4096));
+    abs_max_kernel<<<blocks, 256, 0, s>>>(values, n, scratch);
+    TSNE_LAUNCHED(s);
+    divide_kernel<<<blocks, 256, 0, s>>>(values, n, scratch);
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+int launch_perplexity(const float *sq_dist, int N, int K, float perplexity, float eps, float *pij, float *betas,
+                      hipStream_t s) {
+    const float log_target = logf(perplexity);
+#define TSNE_PERP(LANES, VPL)                                                                                  \
+    perplexity_kernel<LANES, VPL><<<div_up(N, 256 / LANES), 256, 0, s>>>(sq_dist, N, K, log_target, eps, pij, \
+                                                                         betas)
+    if (K <= 32) {
+        TSNE_PERP(16, 2);
+    } else if (K <= 64) {
+        TSNE_PERP(32, 2);
+    } else if (K <= 96) {
+        TSNE_PERP(32, 3);
+    } else if (K <= 128) {
+        TSNE_PERP(64, 2);
+    } else if (K <= 256) {
+        TSNE_PERP(64, 4);
+    } else if (K <= 512) {
+        TSNE_PERP(64, 8);
+    } else if (K <= 1024) {
+        TSNE_PERP(64, 16);
+    } else {
+        perplexity_generic_kernel<<<div_up(N, 256 / kWave), 256, 0, s>>>(sq_dist, N, K, log_target, eps, pij, betas);
+    }
+#undef TSNE_PERP
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+}  // namespace tsnehip

@@ -1,0 +1,63 @@
+// Scratch memory and constants of the gradient loop (internal).
+#ifndef TSNE_HIP_PLAN_H_
+#define TSNE_HIP_PLAN_H_
+
+#include "common.h"
+
+namespace tsnehip {
+
+constexpr int kInterp = 3;        // interpolation nodes per box and dimension (src/fit_tsne.cu:248)
+constexpr int kTerms = 4;         // charges per point (src/fit_tsne.cu:254)
+constexpr int kFft = 1024;        // padded transform length, >= 2 * 3 * n_boxes - 1
+constexpr int kNodePad = 512;     // leading dimension of the transposed spectra (>= nodes per dim)
+constexpr int kMaxBoxes = 170;    // 3 * 170 = 510 nodes <= kNodePad
+
+// Lagrange node positions inside a box and the basis denominators, formed in
+// fp32 exactly as the reference does on the host (src/fit_tsne.cu:303-321).
+struct LagrangeConsts {
+    float spacing[kInterp];
+    float denom[kInterp];
+};
+
+}  // namespace tsnehip
+
+struct tsne_hip_plan {
+    int num_points = 0;
+    int num_neighbors = 0;
+    int n_boxes = 0;
+    int n_nodes = 0;  // n_boxes * kInterp
+    int device = 0;
+    tsnehip::LagrangeConsts lagrange;
+
+    float2 *yxy = nullptr;         // N interleaved (x, y) pairs for the neighbour gathers
+    float4 *node_charges = nullptr;     // n_nodes^2, one float4 (4 terms) per node
+    float4 *node_potentials = nullptr;  // n_nodes^2
+    float2 *row_spectra = nullptr;      // 2 plane pairs x kFft x kNodePad (transposed)
+    float2 *col_results = nullptr;      // same shape
+    float *kernel_rows = nullptr;       // (kFft/2+1) x kNodePad: row spectra of the Cauchy kernel
+    float2 *twiddles = nullptr;         // kFft roots of unity
+    tsnehip::LoopScalars *scalars = nullptr;
+    float *attr = nullptr;  // 2N, used by tsne_hip_iterate
+    float *rep = nullptr;   // 2N
+};
+
+namespace tsnehip {
+
+// Stage launchers shared between the stage-level ABI and the fused loop.
+// `slot` selects which pair of bounds in LoopScalars the launch reads.
+int launch_bounds_reset(tsne_hip_plan *p, int slot, hipStream_t s);
+int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s);
+int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *rep, float *point_potentials,
+                     float *charges_out, hipStream_t s);
+// Writes Z = z_sum - N to the device scalar *normalization.
+int launch_finish_z(tsne_hip_plan *p, float *normalization, hipStream_t s);
+int launch_pack_xy(tsne_hip_plan *p, const float *embedding, hipStream_t s);
+int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, float *attr, hipStream_t s);
+int launch_sum_squares(const float *values, int64_t n, float *out, hipStream_t s);
+int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, float *gains, float *old_forces,
+                  float eta, const float *normalization, float momentum, float exaggeration, int next_slot,
+                  hipStream_t s);
+
+}  // namespace tsnehip
+
+#endif  // TSNE_HIP_PLAN_H_

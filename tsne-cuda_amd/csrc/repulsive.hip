@@ -1,0 +1,504 @@
+// FFT-interpolated repulsive forces for gfx950.
+//
+// One gradient step evaluates, for every point i and the four charge terms
+// q_j = (1, x_j, y_j, x_j^2 + y_j^2),
+//     phi_i[t] = sum_j q_j[t] / (1 + |y_i - y_j|^2)^2
+// by (1) spreading the charges onto an n_nodes x n_nodes grid of equispaced
+// interpolation nodes with 3x3 Lagrange weights, (2) convolving the grid with
+// the squared-Cauchy kernel, (3) interpolating the node potentials back.
+// Semantics follow src/kernels/nbodyfft.cu and src/kernels/rep_forces.cu of the
+// reference; the structure does not:
+//   * bounds, box width and Z never leave the device;
+//   * charges, box indices and Lagrange weights are recomputed in registers
+//     instead of being stored (src/kernels/nbodyfft.cu:43-105,
+//     src/kernels/rep_forces.cu:57-76);
+//   * the convolution zero-pads to 1024 and runs as in-place radix-4 FFTs in
+//     LDS: a decimation-in-frequency forward transform leaves its output in
+//     base-4 digit-reversed order, the decimation-in-time inverse consumes that
+//     order, so nothing is ever permuted.  Two real charge planes ride in one
+//     complex transform; the kernel is real and even, so its spectrum is real
+//     and the planes never mix.  fp32 round-off does leak between the two
+//     planes of a pair in proportion to the larger one, so planes of like
+//     magnitude are paired: (1, r^2 / m^2) and (x, y), with m the largest
+//     absolute coordinate.
+#include "plan.h"
+
+#include <algorithm>
+
+namespace tsnehip {
+
+namespace {
+
+constexpr int kLog2Fft = 10;
+
+__device__ __forceinline__ int rev4(int x) {
+    // Reverse the five base-4 digits of a 10-bit index.
+    const unsigned int y = __brev((unsigned int)x) >> (32 - kLog2Fft);
+    return (int)(((y & 0x155u) << 1) | ((y >> 1) & 0x155u));
+}
+
+__device__ __forceinline__ float2 cmul(float2 a, float2 b) {
+    return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x);
+}
+__device__ __forceinline__ float2 cmul_conj(float2 a, float2 b) {  // a * conj(b)
+    return make_float2(a.x * b.x + a.y * b.y, a.y * b.x - a.x * b.y);
+}
+__device__ __forceinline__ float2 cadd(float2 a, float2 b) { return make_float2(a.x + b.x, a.y + b.y); }
+__device__ __forceinline__ float2 csub(float2 a, float2 b) { return make_float2(a.x - b.x, a.y - b.y); }
+
+// One radix-4 stage over `nfft` transforms of length 1024 stored back to back
+// in LDS.  L is the sub-transform length of the stage.  Forward stages run
+// L = 1024, 256, 64, 16, 4; inverse stages run the same butterflies backwards
+// with L = 4, 16, 64, 256, 1024.
+template <bool INVERSE>
+__device__ __forceinline__ void radix4_stage(float2 *s, int nfft, int log2L, const float2 *tw, int tid,
+                                             int nthreads) {
+    const int L = 1 << log2L;
+    const int q4 = L >> 2;
+    const int log2q4 = log2L - 2;
+    const int stride = kFft >> log2L;
+    for (int id = tid; id < nfft * (kFft / 4); id += nthreads) {
+        const int f = id >> 8;
+        const int q = id & 255;
+        const int k = q & (q4 - 1);
+        const int b = q >> log2q4;
+        float2 *a = s + f * kFft + b * L + k;
+        const float2 w1 = tw[k * stride];
+        const float2 w2 = tw[2 * k * stride];
+        const float2 w3 = tw[3 * k * stride];
+        float2 a0 = a[0], a1 = a[q4], a2 = a[2 * q4], a3 = a[3 * q4];
+        if (!INVERSE) {
+            const float2 t0 = cadd(a0, a2), t1 = csub(a0, a2), t2 = cadd(a1, a3), t3 = csub(a1, a3);
+            a[0] = cadd(t0, t2);
+            a[q4] = cmul(make_float2(t1.x + t3.y, t1.y - t3.x), w1);
+            a[2 * q4] = cmul(csub(t0, t2), w2);
+            a[3 * q4] = cmul(make_float2(t1.x - t3.y, t1.y + t3.x), w3);
+        } else {
+            a1 = cmul_conj(a1, w1);
+            a2 = cmul_conj(a2, w2);
+            a3 = cmul_conj(a3, w3);
+            const float2 u0 = cadd(a0, a2), u1 = csub(a0, a2), u2 = cadd(a1, a3), u3 = csub(a1, a3);
+            a[0] = cadd(u0, u2);
+            a[q4] = make_float2(u1.x - u3.y, u1.y + u3.x);
+            a[2 * q4] = csub(u0, u2);
+            a[3 * q4] = make_float2(u1.x + u3.y, u1.y - u3.x);
+        }
+    }
+}
+
+__device__ __forceinline__ void fft_forward(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+#pragma unroll
+    for (int l = kLog2Fft; l >= 2; l -= 2) {
+        radix4_stage<false>(s, nfft, l, tw, tid, nthreads);
+        __syncthreads();
+    }
+}
+__device__ __forceinline__ void fft_inverse(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+#pragma unroll
+    for (int l = 2; l <= kLog2Fft; l += 2) {
+        radix4_stage<true>(s, nfft, l, tw, tid, nthreads);
+        __syncthreads();
+    }
+}
+
+struct Bounds {
+    float lo, box_width, h;
+};
+__device__ __forceinline__ Bounds load_bounds(const LoopScalars *sc, int slot, int n_boxes) {
+#pragma clang fp contract(off)
+    Bounds b;
+    b.lo = ordered_to_float(sc->min_enc[slot]);
+    const float hi = ordered_to_float(sc->max_enc[slot]);
+    b.box_width = (hi - b.lo) / (float)n_boxes;  // src/fit_tsne.cu:442
+    b.h = b.box_width / (float)kInterp;          // src/kernels/nbodyfft.cu:270
+    return b;
+}
+
+// 1 / m^2 with m the largest absolute coordinate: brings the r^2 charge plane
+// to the magnitude of the unit charge plane it shares a transform with.
+__device__ __forceinline__ float r2_plane_scale(const LoopScalars *sc, int slot) {
+    const float lo = ordered_to_float(sc->min_enc[slot]);
+    const float hi = ordered_to_float(sc->max_enc[slot]);
+    const float m2 = fmaxf(lo * lo, hi * hi);
+    return m2 > 0.0f ? 1.0f / m2 : 1.0f;
+}
+
+// Box index (clamped), in-box coordinate and the three Lagrange basis values of
+// one coordinate (src/kernels/nbodyfft.cu:43-105,205-227), with the fp32
+// operations kept in the reference's order and never contracted.
+__device__ __forceinline__ void bin_and_weights(float v, const Bounds &bd, int n_boxes, const LagrangeConsts &lc,
+                                                int &box, float *L) {
+#pragma clang fp contract(off)
+    int b = (int)((v - bd.lo) / bd.box_width);
+    b = max(0, b);
+    b = min(n_boxes - 1, b);
+    box = b;
+    const float lower = b * bd.box_width + bd.lo;
+    const float t = (v - lower) / bd.box_width;
+    const float d0 = t - lc.spacing[0], d1 = t - lc.spacing[1], d2 = t - lc.spacing[2];
+    L[0] = (d1 * d2) / lc.denom[0];
+    L[1] = (d0 * d2) / lc.denom[1];
+    L[2] = (d0 * d1) / lc.denom[2];
+}
+
+// ---------------------------------------------------------------------------
+// Bounds of the embedding: one scalar min and max over all 2N coordinates
+// (src/fit_tsne.cu:430-432), kept on the device in an order-preserving integer
+// encoding so that blocks can combine with integer atomics.
+// ---------------------------------------------------------------------------
+__global__ void bounds_reset_kernel(LoopScalars *sc, int slot) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        sc->min_enc[slot] = 0xffffffffu;
+        sc->max_enc[slot] = 0u;
+    }
+}
+
+__global__ __launch_bounds__(256) void bounds_kernel(const float *__restrict__ v, int64_t n, LoopScalars *sc,
+                                                     int slot) {
+    float lo = INFINITY, hi = -INFINITY;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (int64_t)gridDim.x * blockDim.x) {
+        const float x = v[t];
+        lo = fminf(lo, x);
+        hi = fmaxf(hi, x);
+    }
+    lo = group_min<kWave>(lo);
+    hi = group_max<kWave>(hi);
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        atomicMin(&sc->min_enc[slot], float_to_ordered(lo));
+        atomicMax(&sc->max_enc[slot], float_to_ordered(hi));
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Step prologue: clears Z and the bounds slot the coming update will fill.
+// ---------------------------------------------------------------------------
+__global__ void step_prologue_kernel(LoopScalars *sc, int next_slot) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        sc->z_sum = 0.0f;
+        if (next_slot >= 0) {
+            sc->min_enc[next_slot] = 0xffffffffu;
+            sc->max_enc[next_slot] = 0u;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Spread: w[node][t] += Lx_a * Ly_b * q[t] (src/kernels/nbodyfft.cu:107-139).
+// The row index of the node grid is the x node.  One thread per point, 36
+// hardware fp32 atomics into the L2-resident 2.4 MB grid.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void spread_kernel(const float *__restrict__ emb, int N, const LoopScalars *sc,
+                                                     int slot, int n_boxes, LagrangeConsts lc,
+                                                     float *__restrict__ w) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= N) return;
+    const Bounds bd = load_bounds(sc, slot, n_boxes);
+    const float x = emb[i], y = emb[N + i];
+    int bx, by;
+    float Lx[kInterp], Ly[kInterp];
+    bin_and_weights(x, bd, n_boxes, lc, bx, Lx);
+    bin_and_weights(y, bd, n_boxes, lc, by, Ly);
+    const int G = n_boxes * kInterp;
+    const float q3 = x * x + y * y;
+#pragma unroll
+    for (int a = 0; a < kInterp; ++a) {
+#pragma unroll
+        for (int b = 0; b < kInterp; ++b) {
+            const float lw = Lx[a] * Ly[b];
+            float *dst = w + ((size_t)(bx * kInterp + a) * G + (by * kInterp + b)) * kTerms;
+            atomicAdd(dst + 0, lw);
+            atomicAdd(dst + 1, lw * x);
+            atomicAdd(dst + 2, lw * y);
+            atomicAdd(dst + 3, lw * q3);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Kernel rows: for node offsets a in [0, G) transform the even sequence
+// b -> k(a, |b|) = (1 + (a h)^2 + (b h)^2)^-2 (src/kernels/nbodyfft.cu:175-203)
+// along b.  Two rows share one complex transform (both spectra are real).
+// Output kernel_rows[v][a] for frequencies v in [0, 512].
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float kernel_value(float lo, float h, int a, int b) {
+#pragma clang fp contract(off)
+    const float base = lo + h / 2;
+    const float ya = base + a * h;
+    const float xb = base + b * h;
+    const float da = base - ya;
+    const float db = base - xb;
+    const double s = 1.0 + (double)da * (double)da + (double)db * (double)db;
+    return (float)(1.0 / (s * s));
+}
+
+__global__ __launch_bounds__(256) void kernel_rows_kernel(const LoopScalars *sc, int slot, int n_boxes,
+                                                          const float2 *__restrict__ twiddles,
+                                                          float *__restrict__ kernel_rows) {
+    __shared__ float2 tw[kFft];
+    __shared__ float2 s[2][kFft];
+    const int tid = threadIdx.x;
+    const int G = n_boxes * kInterp;
+    const Bounds bd = load_bounds(sc, slot, n_boxes);
+    const int a0 = blockIdx.x * 4;
+    for (int e = tid; e < kFft; e += 256) tw[e] = twiddles[e];
+    for (int e = tid; e < 2 * kFft; e += 256) {
+        const int f = e >> kLog2Fft, m = e & (kFft - 1);
+        const int b = m < kFft / 2 ? m : kFft - m;
+        const int ra = a0 + 2 * f;
+        float2 v = make_float2(0.f, 0.f);
+        if (b < G) {
+            if (ra < G) v.x = kernel_value(bd.lo, bd.h, ra, b);
+            if (ra + 1 < G) v.y = kernel_value(bd.lo, bd.h, ra + 1, b);
+        }
+        s[f][m] = v;
+    }
+    __syncthreads();
+    fft_forward(&s[0][0], 2, tw, tid, 256);
+    for (int e = tid; e < 2 * kFft; e += 256) {
+        const int f = e >> kLog2Fft, pos = e & (kFft - 1);
+        const int v = rev4(pos);
+        if (v <= kFft / 2) {
+            const int ra = a0 + 2 * f;
+            const float2 val = s[f][pos];
+            *reinterpret_cast<float2 *>(kernel_rows + (size_t)v * kNodePad + ra) = val;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Row pass: transforms two grid rows (x nodes m0, m0+1), both plane pairs,
+// along the y-node axis; clears the charges it consumed so that the next step
+// starts from zero without a memset.  Output is transposed:
+// row_spectra[pair][pos][m], pos = digit-reversed frequency position.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void conv_rows_forward_kernel(float4 *__restrict__ w, int G,
+                                                                const LoopScalars *sc, int slot,
+                                                                const float2 *__restrict__ twiddles,
+                                                                float2 *__restrict__ row_spectra) {
+    __shared__ float2 tw[kFft];
+    __shared__ float2 s[4][kFft];  // [row * 2 + pair]
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.x * 2;
+    const float s3 = r2_plane_scale(sc, slot);
+    for (int e = tid; e < kFft; e += 256) tw[e] = twiddles[e];
+    for (int e = tid; e < 2 * kFft; e += 256) {
+        const int r = e >> kLog2Fft, n = e & (kFft - 1);
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (n < G && m0 + r < G) {
+            float4 *src = w + (size_t)(m0 + r) * G + n;
+            v = *src;
+            *src = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        s[r * 2 + 0][n] = make_float2(v.x, v.w * s3);  // planes 1 and r^2 / m^2
+        s[r * 2 + 1][n] = make_float2(v.y, v.z);       // planes x and y
+    }
+    __syncthreads();
+    fft_forward(&s[0][0], 4, tw, tid, 256);
+    for (int e = tid; e < 2 * kFft; e += 256) {
+        const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
+        const float2 r0 = s[0 + pair][pos], r1 = s[2 + pair][pos];
+        float4 *dst = reinterpret_cast<float4 *>(row_spectra + ((size_t)pair * kFft + pos) * kNodePad + m0);
+        *dst = make_float4(r0.x, r0.y, r1.x, r1.y);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Column pass for two spectrum positions: forward transform along the x-node
+// axis, multiply by the kernel spectrum, inverse transform.  The kernel
+// spectrum column of each position is produced here from kernel_rows (one more
+// packed transform) so it never travels through memory.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restrict__ row_spectra, int G,
+                                                           const float *__restrict__ kernel_rows,
+                                                           const float2 *__restrict__ twiddles,
+                                                           float2 *__restrict__ col_results) {
+    __shared__ float2 tw[kFft];
+    __shared__ float2 s[5][kFft];  // [col * 2 + pair], then the kernel columns
+    const int tid = threadIdx.x;
+    const int c0 = blockIdx.x * 2;
+    for (int e = tid; e < kFft; e += 512) tw[e] = twiddles[e];
+    for (int e = tid; e < 4 * kFft; e += 512) {
+        const int f = e >> kLog2Fft, m = e & (kFft - 1);
+        const int col = f >> 1, pair = f & 1;
+        float2 v = make_float2(0.f, 0.f);
+        if (m < G) v = row_spectra[((size_t)pair * kFft + c0 + col) * kNodePad + m];
+        s[f][m] = v;
+    }
+    {
+        int v0 = rev4(c0), v1 = rev4(c0 + 1);
+        v0 = min(v0, kFft - v0);
+        v1 = min(v1, kFft - v1);
+        for (int m = tid; m < kFft; m += 512) {
+            const int a = m < kFft / 2 ? m : kFft - m;
+            float2 v = make_float2(0.f, 0.f);
+            if (a < G) {
+                v.x = kernel_rows[(size_t)v0 * kNodePad + a];
+                v.y = kernel_rows[(size_t)v1 * kNodePad + a];
+            }
+            s[4][m] = v;
+        }
+    }
+    __syncthreads();
+    fft_forward(&s[0][0], 5, tw, tid, 512);
+    for (int e = tid; e < 4 * kFft; e += 512) {
+        const int f = e >> kLog2Fft, m = e & (kFft - 1);
+        const float2 kk = s[4][m];
+        const float kv = (f >> 1) ? kk.y : kk.x;
+        float2 v = s[f][m];
+        v.x *= kv;
+        v.y *= kv;
+        s[f][m] = v;
+    }
+    __syncthreads();
+    fft_inverse(&s[0][0], 4, tw, tid, 512);
+    for (int e = tid; e < 4 * kFft; e += 512) {
+        const int f = e >> kLog2Fft, m = e & (kFft - 1);
+        const int col = f >> 1, pair = f & 1;
+        if (m < G) col_results[((size_t)pair * kFft + c0 + col) * kNodePad + m] = s[f][m];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Inverse row pass for x nodes m0, m0+1: consumes digit-reversed positions,
+// produces node potentials in natural order, scaled by 1/1024^2.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void conv_rows_inverse_kernel(const float2 *__restrict__ col_results, int G,
+                                                                const LoopScalars *sc, int slot,
+                                                                const float2 *__restrict__ twiddles,
+                                                                float4 *__restrict__ node_potentials) {
+    __shared__ float2 tw[kFft];
+    __shared__ float2 s[4][kFft];  // [row * 2 + pair]
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.x * 2;
+    for (int e = tid; e < kFft; e += 256) tw[e] = twiddles[e];
+    for (int e = tid; e < 2 * kFft; e += 256) {
+        const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
+        const float4 v =
+            *reinterpret_cast<const float4 *>(col_results + ((size_t)pair * kFft + pos) * kNodePad + m0);
+        s[0 + pair][pos] = make_float2(v.x, v.y);
+        s[2 + pair][pos] = make_float2(v.z, v.w);
+    }
+    __syncthreads();
+    fft_inverse(&s[0][0], 4, tw, tid, 256);
+    const float scale = 1.0f / ((float)kFft * (float)kFft);
+    const float scale3 = scale / r2_plane_scale(sc, slot);
+    for (int e = tid; e < 2 * kFft; e += 256) {
+        const int r = e >> kLog2Fft, n = e & (kFft - 1);
+        if (n < G && m0 + r < G) {
+            const float2 p0 = s[r * 2 + 0][n], p1 = s[r * 2 + 1][n];
+            node_potentials[(size_t)(m0 + r) * G + n] =
+                make_float4(p0.x * scale, p1.x * scale, p1.y * scale, p0.y * scale3);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Gather + force assembly: phi_i = sum_{a,b} Lx_a Ly_b y~[node] then
+// rep = (x phi1 - phi2, y phi1 - phi3), z_i = (1+x^2+y^2) phi1 - 2(x phi2 + y phi3) + phi4
+// (src/kernels/nbodyfft.cu:141-173, src/kernels/rep_forces.cu:3-31).  Block
+// partial sums of z_i go to the device scalar with one atomic per block.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gather_forces_kernel(const float *__restrict__ emb, int N,
+                                                            const LoopScalars *sc_in, int slot, int n_boxes,
+                                                            LagrangeConsts lc,
+                                                            const float4 *__restrict__ node_potentials,
+                                                            float *__restrict__ rep, float *__restrict__ phi_out,
+                                                            LoopScalars *sc) {
+    __shared__ float partial[256 / kWave];
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    float z = 0.0f;
+    if (i < N) {
+        const Bounds bd = load_bounds(sc_in, slot, n_boxes);
+        const float x = emb[i], y = emb[N + i];
+        int bx, by;
+        float Lx[kInterp], Ly[kInterp];
+        bin_and_weights(x, bd, n_boxes, lc, bx, Lx);
+        bin_and_weights(y, bd, n_boxes, lc, by, Ly);
+        const int G = n_boxes * kInterp;
+        float4 phi = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int a = 0; a < kInterp; ++a) {
+#pragma unroll
+            for (int b = 0; b < kInterp; ++b) {
+                const float lw = Lx[a] * Ly[b];
+                const float4 yt = node_potentials[(size_t)(bx * kInterp + a) * G + (by * kInterp + b)];
+                phi.x += lw * yt.x;
+                phi.y += lw * yt.y;
+                phi.z += lw * yt.z;
+                phi.w += lw * yt.w;
+            }
+        }
+        z = (1 + x * x + y * y) * phi.x - 2 * (x * phi.y + y * phi.z) + phi.w;
+        rep[i] = x * phi.x - phi.y;
+        rep[N + i] = y * phi.x - phi.z;
+        if (phi_out) reinterpret_cast<float4 *>(phi_out)[i] = phi;
+    }
+    z = group_sum<kWave>(z);
+    if ((threadIdx.x & (kWave - 1)) == 0) partial[threadIdx.x / kWave] = z;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 256 / kWave; ++k) t += partial[k];
+        atomicAdd(&sc->z_sum, t);
+    }
+}
+
+__global__ void finish_z_kernel(const LoopScalars *sc, int N, float *out) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *out = sc->z_sum - (float)N;  // src/kernels/rep_forces.cu:54
+}
+
+}  // namespace
+
+int launch_finish_z(tsne_hip_plan *p, float *normalization, hipStream_t s) {
+    finish_z_kernel<<<1, 64, 0, s>>>(p->scalars, p->num_points, normalization);
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+int launch_bounds_reset(tsne_hip_plan *p, int slot, hipStream_t s) {
+    bounds_reset_kernel<<<1, 64, 0, s>>>(p->scalars, slot);
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s) {
+    if (launch_bounds_reset(p, slot, s)) return 1;
+    const int64_t n = 2 * (int64_t)p->num_points;
+    const int blocks = (int)std::min<int64_t>(div_up(n, 256 * 4), 2048);
+    bounds_kernel<<<blocks, 256, 0, s>>>(embedding, n, p->scalars, slot);
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+// All kernels of one repulsive-force evaluation.  Expects the bounds of
+// `embedding` in `slot`; leaves sum_i z_i in scalars->z_sum and resets the other
+// bounds slot.  charges_out (optional) receives a copy of the node charges.
+int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *rep, float *point_potentials,
+                     float *charges_out, hipStream_t s) {
+    const int N = p->num_points, G = p->n_nodes, nb = p->n_boxes;
+    step_prologue_kernel<<<1, 64, 0, s>>>(p->scalars, slot ^ 1);
+    TSNE_LAUNCHED(s);
+    kernel_rows_kernel<<<div_up(G, 4), 256, 0, s>>>(p->scalars, slot, nb, p->twiddles, p->kernel_rows);
+    TSNE_LAUNCHED(s);
+    spread_kernel<<<div_up(N, 256), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
+                                                 reinterpret_cast<float *>(p->node_charges));
+    TSNE_LAUNCHED(s);
+    if (charges_out)
+        TSNE_TRY(hipMemcpyAsync(charges_out, p->node_charges, sizeof(float4) * (size_t)G * G,
+                                hipMemcpyDeviceToDevice, s));
+    conv_rows_forward_kernel<<<div_up(G, 2), 256, 0, s>>>(p->node_charges, G, p->scalars, slot, p->twiddles,
+                                                          p->row_spectra);
+    TSNE_LAUNCHED(s);
+    conv_columns_kernel<<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
+    TSNE_LAUNCHED(s);
+    conv_rows_inverse_kernel<<<div_up(G, 2), 256, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
+                                                          p->node_potentials);
+    TSNE_LAUNCHED(s);
+    gather_forces_kernel<<<div_up(N, 256), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
+                                                        p->node_potentials, rep, point_potentials, p->scalars);
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+}  // namespace tsnehip

@@ -1,0 +1,123 @@
+// Gains / momentum update of the embedding for gfx950.
+//
+// Semantics: src/kernels/apply_forces.cu:11-57 of the reference (no factor 4,
+// no re-centring, sign test through signbit, gain constants in double).  In the
+// fused loop the same pass also refreshes the interleaved (x, y) copy used by
+// the neighbour gathers and accumulates the bounds of the new embedding, which
+// replaces the reference's per-step host-synchronising minmax_element
+// (src/fit_tsne.cu:430-432).
+#include "plan.h"
+
+#include <algorithm>
+
+namespace tsnehip {
+
+namespace {
+
+__device__ __forceinline__ float step_coordinate(float &gain, float &u, float attr, float rep, float exaggeration,
+                                                 float normalization, float momentum, float eta) {
+#pragma clang fp contract(off)
+    const float d = exaggeration * attr - (rep / normalization);
+    float g = gain;
+    g = (signbit(d) != signbit(u)) ? (float)((double)g + 0.2) : (float)((double)g * 0.8);
+    g = ((double)g < 0.01) ? (float)0.01 : g;
+    u = momentum * u - eta * g * d;
+    gain = g;
+    return u;
+}
+
+template <bool FUSED>
+__global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, float *__restrict__ attr,
+                                                     float *__restrict__ rep, float *__restrict__ gains,
+                                                     float *__restrict__ old, int N, float eta,
+                                                     const float *__restrict__ z_ptr, float z_offset, float momentum,
+                                                     float exaggeration, float2 *__restrict__ yxy, LoopScalars *sc,
+                                                     int next_slot) {
+    const float normalization = *z_ptr - z_offset;
+    float lo = INFINITY, hi = -INFINITY;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
+        float gx = gains[i], gy = gains[N + i];
+        float ux = old[i], uy = old[N + i];
+        step_coordinate(gx, ux, attr[i], rep[i], exaggeration, normalization, momentum, eta);
+        step_coordinate(gy, uy, attr[N + i], rep[N + i], exaggeration, normalization, momentum, eta);
+        const float x = emb[i] + ux;
+        const float y = emb[N + i] + uy;
+        emb[i] = x;
+        emb[N + i] = y;
+        attr[i] = 0.0f;
+        attr[N + i] = 0.0f;
+        rep[i] = 0.0f;
+        rep[N + i] = 0.0f;
+        old[i] = ux;
+        old[N + i] = uy;
+        gains[i] = gx;
+        gains[N + i] = gy;
+        if (FUSED) {
+            yxy[i] = make_float2(x, y);
+            lo = fminf(lo, fminf(x, y));
+            hi = fmaxf(hi, fmaxf(x, y));
+        }
+    }
+    if (FUSED) {
+        lo = group_min<kWave>(lo);
+        hi = group_max<kWave>(hi);
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            atomicMin(&sc->min_enc[next_slot], float_to_ordered(lo));
+            atomicMax(&sc->max_enc[next_slot], float_to_ordered(hi));
+        }
+    }
+}
+
+__global__ void clear_scalar_kernel(float *p) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *p = 0.0f;
+}
+
+__global__ __launch_bounds__(256) void sum_squares_kernel(const float *__restrict__ v, int64_t n, float *out) {
+    __shared__ float partial[256 / kWave];
+    float acc = 0.0f;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (int64_t)gridDim.x * blockDim.x) {
+        const float x = v[t];
+        acc += x * x;
+    }
+    acc = group_sum<kWave>(acc);
+    if ((threadIdx.x & (kWave - 1)) == 0) partial[threadIdx.x / kWave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.0f;
+        for (int k = 0; k < 256 / kWave; ++k) t += partial[k];
+        atomicAdd(out, t);
+    }
+}
+
+}  // namespace
+
+// normalization == nullptr: Z is taken from the loop scalars (z_sum - N).
+// next_slot >= 0: also refresh the (x, y) copy and accumulate the new bounds.
+int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, float *gains, float *old_forces,
+                  float eta, const float *normalization, float momentum, float exaggeration, int next_slot,
+                  hipStream_t s) {
+    const int N = p->num_points;
+    const float *z_ptr = normalization ? normalization : &p->scalars->z_sum;
+    const float z_offset = normalization ? 0.0f : (float)N;
+    const int blocks = div_up(N, 256);
+    if (next_slot >= 0) {
+        update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_offset,
+                                                   momentum, exaggeration, p->yxy, p->scalars, next_slot);
+    } else {
+        update_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_offset,
+                                                    momentum, exaggeration, nullptr, nullptr, 0);
+    }
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+int launch_sum_squares(const float *values, int64_t n, float *out, hipStream_t s) {
+    clear_scalar_kernel<<<1, 64, 0, s>>>(out);  // a kernel, not a memset node, so the call can be graph-captured
+    TSNE_LAUNCHED(s);
+    const int blocks = (int)std::min<int64_t>(div_up(n, 256 * 4), 2048);
+    sum_squares_kernel<<<std::max(blocks, 1), 256, 0, s>>>(values, n, out);
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+}  // namespace tsnehip

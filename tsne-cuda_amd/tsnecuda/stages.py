@@ -1,0 +1,153 @@
+"""ctypes bindings of the stage-level C ABI (``include/tsnecuda/tsne_stages.h``).
+
+Arguments are torch CUDA tensors; only their device pointers and sizes cross
+the boundary.  Every call runs on torch's current stream, so torch events and
+synchronisation see the work.  Raises ``RuntimeError`` with the library's
+message when a call fails.
+"""
+import ctypes
+import os
+
+import torch
+
+_lib = None
+_vp = ctypes.c_void_p
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtsnecuda.so")
+        if not os.path.exists(path):
+            raise OSError("%s not found: build it with `make -C tsne-cuda_amd` first" % path)
+        L = ctypes.CDLL(path)
+        L.tsne_hip_last_error.restype = ctypes.c_char_p
+        c_int, c_float, c_i64 = ctypes.c_int, ctypes.c_float, ctypes.c_int64
+        L.tsne_hip_knn.argtypes = [_vp, c_int, c_int, c_int, _vp, _vp, _vp]
+        L.tsne_hip_max_normalize.argtypes = [_vp, c_i64, _vp]
+        L.tsne_hip_perplexity.argtypes = [_vp, c_int, c_int, c_float, c_float, _vp, _vp, _vp]
+        L.tsne_hip_symmetrize.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
+        L.tsne_hip_plan_create.argtypes = [ctypes.POINTER(_vp), c_int, c_int, c_int, c_int]
+        L.tsne_hip_plan_destroy.argtypes = [_vp]
+        L.tsne_hip_plan_destroy.restype = None
+        L.tsne_hip_attractive.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp]
+        L.tsne_hip_repulsive.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]
+        L.tsne_hip_update.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, c_float, _vp, c_float, c_float, _vp]
+        L.tsne_hip_iterate.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, c_int, c_int, c_int, c_float, c_float,
+                                       c_float, c_float, _vp, _vp]
+        L.tsne_hip_sum_squares.argtypes = [_vp, _vp, c_i64, _vp, _vp]
+        for name in ("knn", "max_normalize", "perplexity", "symmetrize", "plan_create", "attractive",
+                     "repulsive", "update", "iterate", "sum_squares"):
+            getattr(L, "tsne_hip_" + name).restype = c_int
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise RuntimeError(lib().tsne_hip_last_error().decode())
+
+
+def _ptr(t):
+    return None if t is None else _vp(t.data_ptr())
+
+
+def _stream():
+    return _vp(torch.cuda.current_stream().cuda_stream)
+
+
+def _f32(t):
+    assert t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()
+    return t
+
+
+def knn(points, num_neighbors):
+    points = _f32(points)
+    n, d = points.shape
+    idx = torch.empty((n, num_neighbors), dtype=torch.int32, device=points.device)
+    dist = torch.empty((n, num_neighbors), dtype=torch.float32, device=points.device)
+    _check(lib().tsne_hip_knn(_ptr(points), n, d, num_neighbors, _ptr(idx), _ptr(dist), _stream()))
+    return idx, dist
+
+
+def max_normalize_(values):
+    _check(lib().tsne_hip_max_normalize(_ptr(_f32(values)), values.numel(), _stream()))
+    return values
+
+
+def perplexity(sq_dist, perplexity, epsilon, return_betas=False):
+    sq_dist = _f32(sq_dist)
+    n, k = sq_dist.shape
+    pij = torch.empty_like(sq_dist)
+    betas = torch.empty(n, dtype=torch.float32, device=sq_dist.device) if return_betas else None
+    _check(lib().tsne_hip_perplexity(_ptr(sq_dist), n, k, perplexity, epsilon, _ptr(pij), _ptr(betas), _stream()))
+    return (pij, betas) if return_betas else pij
+
+
+def symmetrize(pij, idx):
+    pij = _f32(pij)
+    n, k = pij.shape
+    out = torch.empty_like(pij)
+    _check(lib().tsne_hip_symmetrize(_ptr(pij), _ptr(idx), n, k, _ptr(out), _stream()))
+    return out
+
+
+class Plan(object):
+    """Scratch memory of the gradient loop for one problem size."""
+
+    def __init__(self, num_points, num_neighbors, n_boxes_per_dim=130, device=0):
+        self._h = _vp()
+        self.num_points, self.num_neighbors, self.n_boxes = num_points, num_neighbors, n_boxes_per_dim
+        self.n_nodes = 3 * n_boxes_per_dim
+        self.device = torch.device("cuda", device)
+        _check(lib().tsne_hip_plan_create(ctypes.byref(self._h), num_points, num_neighbors, n_boxes_per_dim,
+                                          device))
+
+    def close(self):
+        if self._h:
+            lib().tsne_hip_plan_destroy(self._h)
+            self._h = _vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def attractive(self, pij, idx, embedding):
+        out = torch.empty(2 * self.num_points, dtype=torch.float32, device=self.device)
+        _check(lib().tsne_hip_attractive(self._h, _ptr(_f32(pij)), _ptr(idx), _ptr(_f32(embedding)), _ptr(out),
+                                         _stream()))
+        return out
+
+    def repulsive(self, embedding, details=False):
+        n, g = self.num_points, self.n_nodes
+        rep = torch.empty(2 * n, dtype=torch.float32, device=self.device)
+        z = torch.empty(1, dtype=torch.float32, device=self.device)
+        w = yt = phi = None
+        if details:
+            w = torch.empty((g, g, 4), dtype=torch.float32, device=self.device)
+            yt = torch.empty((g, g, 4), dtype=torch.float32, device=self.device)
+            phi = torch.empty((n, 4), dtype=torch.float32, device=self.device)
+        _check(lib().tsne_hip_repulsive(self._h, _ptr(_f32(embedding)), _ptr(rep), _ptr(z), _ptr(w), _ptr(yt),
+                                        _ptr(phi), _stream()))
+        return (rep, z, w, yt, phi) if details else (rep, z)
+
+    def update_(self, embedding, attr, rep, gains, old_forces, eta, normalization, momentum, exaggeration):
+        _check(lib().tsne_hip_update(self._h, _ptr(_f32(embedding)), _ptr(_f32(attr)), _ptr(_f32(rep)),
+                                     _ptr(_f32(gains)), _ptr(_f32(old_forces)), eta, _ptr(_f32(normalization)),
+                                     momentum, exaggeration, _stream()))
+
+    def iterate_(self, pij, idx, embedding, gains, old_forces, step_begin, step_end, force_magnify_iters=250,
+                 eta=200.0, pre_momentum=0.5, post_momentum=0.8, early_exaggeration=12.0):
+        z = torch.zeros(1, dtype=torch.float32, device=self.device)
+        _check(lib().tsne_hip_iterate(self._h, _ptr(_f32(pij)), _ptr(idx), _ptr(_f32(embedding)),
+                                      _ptr(_f32(gains)), _ptr(_f32(old_forces)), step_begin, step_end,
+                                      force_magnify_iters, eta, pre_momentum, post_momentum, early_exaggeration,
+                                      _ptr(z), _stream()))
+        return z
+
+    def sum_squares(self, values):
+        out = torch.empty(1, dtype=torch.float32, device=self.device)
+        _check(lib().tsne_hip_sum_squares(self._h, _ptr(_f32(values)), values.numel(), _ptr(out), _stream()))
+        return out
