@@ -1,0 +1,157 @@
+#!/usr/bin/env python3
+"""Benchmark of the FIt-SNE gradient pipeline on one MI355X.
+
+A "step" is one gradient iteration (repulsive + attractive forces + update) of
+the 1,000,000 x 50 configuration (config c3) with the inputs resident in HBM.
+Prints ONE JSON line: gradient iterations per second, plus per-phase times of
+the one-shot stages, the end-to-end fit time through the drop-in entry point,
+the roofline of the dominant kernel (attractive forces, HBM-bound) and the CPU
+baseline (the oracle's gradient loop on the host cores, bounded sample).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--points N]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "tsne-cuda_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default="c3")
+    ap.add_argument("--points", type=int, default=None, help="override the point count of the workload")
+    ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end fit through pymodule_tsne")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cpu-steps", type=int, default=20, help="gradient steps of the CPU baseline sample")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run 10 plain 256 MiB device copies (known traffic, to scale rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build is single-GPU (one MI355X per process, no collectives); run with --gpus 1")
+
+    import numpy as np
+    import torch
+    from tsnecuda import TSNE, stages, synthetic
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    torch.cuda.set_device(0)
+    stages.lib()  # fails loudly if libtsnecuda.so is missing
+
+    t0 = time.time()
+    X, fit = synthetic.make_config(args.workload, n=args.points)
+    n, d = X.shape
+    k = min(fit["num_neighbors"], n)
+    Y0 = synthetic.initial_embedding(n)
+    y0 = np.concatenate([Y0[:, 0], Y0[:, 1]])
+    gen_s = time.time() - t0
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        a = time.perf_counter()
+        out = fn()
+        torch.cuda.synchronize()
+        return out, time.perf_counter() - a
+
+    # ---- one-shot stages, inputs resident in HBM -------------------------
+    dX = torch.from_numpy(X).cuda()
+    (idx, d2), knn_s = timed(lambda: stages.knn(dX, k))
+    del dX
+    _, norm_s = timed(lambda: stages.max_normalize_(d2))
+    cond, perp_s = timed(lambda: stages.perplexity(d2, fit["perplexity"], 1e-4))
+    P, sym_s = timed(lambda: stages.symmetrize(cond, idx))
+    del cond, d2
+
+    # ---- gradient loop ----------------------------------------------------
+    plan = stages.Plan(n, k)
+    y = torch.from_numpy(y0).cuda()
+    gains, old = torch.ones_like(y), torch.zeros_like(y)
+    eta = fit["learning_rate"]
+    _, warm_s = timed(lambda: plan.iterate_(P, idx, y, gains, old, 0, args.warmup, eta=eta))
+    z, loop_s = timed(lambda: plan.iterate_(P, idx, y, gains, old, args.warmup, args.warmup + args.steps, eta=eta))
+    ms_per_step = loop_s * 1e3 / args.steps
+    iters_per_s = args.steps / loop_s
+
+    # ---- per-kernel durations: HIP events on the loop's stream, recorded by
+    # the library around every kernel of a further stretch of the same loop ----
+    prof_steps = min(args.steps, 200)
+    plan.profile_begin()
+    plan.iterate_(P, idx, y, gains, old, args.warmup + args.steps, args.warmup + args.steps + prof_steps, eta=eta)
+    prof = plan.profile_end()
+    kernels_us = {name: 1e3 * ms / max(cnt, 1) for name, (ms, cnt) in prof.items()}
+    attr_ms = kernels_us["attractive_kernel"] * 1e-3
+    attr_bytes = 8.0 * n * k + 16.0 * n  # P and index streams; read positions, write forces
+    achieved = attr_bytes / (attr_ms * 1e-3) / 1e9
+
+    if args.calibrate:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    # ---- end-to-end fit through the drop-in entry point (host buffers) ----
+    fit_s = None
+    if not args.no_fit:
+        model = TSNE(perplexity=fit["perplexity"], num_neighbors=k, learning_rate=eta, n_iter=1000,
+                     perplexity_epsilon=1e-4)
+        a = time.perf_counter()
+        emb = model.fit_transform(X, y=Y0)
+        fit_s = time.perf_counter() - a
+        assert np.isfinite(emb).all()
+
+    # ---- CPU baseline: the oracle's gradient loop on the host cores -------
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+        P_h, idx_h = P.cpu().numpy(), idx.cpu().numpy()
+        a = time.perf_counter()
+        oracle.iterate(P_h, idx_h, y0, args.cpu_steps, eta=eta)
+        cpu_s = time.perf_counter() - a
+        cpu = {"value": args.cpu_steps / cpu_s, "unit": "iter/s", "cores": oracle.num_threads(), "kind": "port",
+               "sample": "%d gradient steps of the same %d x %d workload (P and neighbours from the GPU stages), "
+                         "C++/OpenMP restatement" % (args.cpu_steps, n, k)}
+
+    out = {
+        "metric": "gradient_iters_per_sec",
+        "value": iters_per_s,
+        "unit": "iter/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "%s: %d x %d fp32, perplexity %g, K=%d, lr %g; step = one gradient iteration"
+                               % (args.workload, n, d, fit["perplexity"], k, eta)},
+        "fit_seconds": fit_s,
+        "phases_s": {"knn": knn_s, "max_normalize": norm_s, "perplexity": perp_s, "symmetrize": sym_s,
+                     "gradient_loop_%d_steps" % args.steps: loop_s, "data_generation_host": gen_s},
+        "roofline": {"bound": "hbm", "kernel": "attractive_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "bytes_per_launch": attr_bytes, "ms_per_launch": attr_ms},
+        "kernels_us": kernels_us,
+        "cpu_baseline": cpu,
+        "final_Z": float(z.item()),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -106,6 +106,16 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
  * (tsnecuda::util::L2NormDeviceVector without the root, src/util/math_utils.cu:51-57). */
 int tsne_hip_sum_squares(tsne_hip_plan *plan, const float *values, int64_t n, float *out, void *stream);
 
+/* Per-kernel timing of tsne_hip_iterate with HIP events on the loop's own
+ * stream (the measured counterpart of the reference's _time_* phase timers,
+ * src/fit_tsne.cu:8-14,586-601).  Between profile_begin and profile_end every
+ * kernel launch of tsne_hip_iterate is bracketed by events; profile_end waits
+ * for them and fills total_ms[k] / launches[k] for k < tsne_hip_profile_kernel_count(). */
+int tsne_hip_profile_kernel_count(void);
+const char *tsne_hip_profile_kernel_name(int id);
+int tsne_hip_profile_begin(tsne_hip_plan *plan);
+int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches);
+
 #ifdef __cplusplus
 }
 #endif

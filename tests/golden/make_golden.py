@@ -1,0 +1,71 @@
+#!/usr/bin/env python3
+"""Regenerates the fixtures in this directory from the CPU oracle.
+
+The reference's own tests hold no golden vectors for this path (its test
+sources do not compile), so the fixtures are the oracle's outputs on small
+seeded inputs; the oracle itself is pinned by the closed-form / brute-force
+checks in tests/test_oracle.py.
+
+  small256.npz   256 x 16 points, K = 16: neighbours, P, forces and one update
+                 step from a fixed embedding (a few hundred KB at most)
+  c0_fit.json    config c0 (5000 x 50, K = 90, perplexity 30): objective value
+                 of the oracle's 1000-step fit from the seeded initial embedding
+
+Run from the repository root:  python tests/golden/make_golden.py
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tsne-cuda_amd"))
+
+import oracle  # noqa: E402
+from tsnecuda import synthetic  # noqa: E402
+
+
+def small_case():
+    n, d, k, perp = 256, 16, 16, 5.0
+    X = synthetic.gaussian_clusters(n, d=d, clusters=3, center_scale=4.0, seed=7)
+    idx, d2 = oracle.knn(X, k)
+    dn, dmax = oracle.max_normalize(d2)
+    p, beta, iters = oracle.perplexity(dn, perp, 1e-4, return_search=True)
+    P = oracle.symmetrize(p, idx)
+    Y0 = synthetic.initial_embedding(n, seed=8, scale=1.0)  # unit-scale embedding: non-trivial forces
+    y = np.concatenate([Y0[:, 0], Y0[:, 1]]).astype(np.float32)
+    attr = oracle.attractive(P, idx, y)
+    rep, z = oracle.repulsive(y)
+    gains = np.ones_like(y)
+    old = np.zeros_like(y)
+    y1, g1, u1 = oracle.update(y, attr, rep, gains, old, 200.0, z, 0.5, 12.0)
+    np.savez_compressed(os.path.join(HERE, "small256.npz"), X=X, idx=idx, d2=d2, dn=dn, p=p, beta=beta,
+                        iters=iters, P=P, y=y, attr=attr, rep=rep, z=np.float32(z), y1=y1, g1=g1, u1=u1,
+                        perplexity=np.float32(perp))
+
+
+def c0_fit():
+    X, fit = synthetic.make_config("c0")
+    Y0 = synthetic.initial_embedding(X.shape[0])
+    y0 = np.concatenate([Y0[:, 0], Y0[:, 1]])
+    y, z, idx, P = oracle.fit(X, y0, fit["num_neighbors"], fit["perplexity"], eps=1e-4, iterations=1000,
+                              eta=fit["learning_rate"])
+    out = {
+        "config": "c0: 5000 x 50, K=90, perplexity 30, lr 200, 1000 steps, exaggeration 12 for 250, VECTOR init seed 1",
+        "kl_exact_z": oracle.kl(P, idx, y),
+        "kl_initial": oracle.kl(P, idx, y0),
+        "z_final_interpolated": z,
+        "extent": [float(y.min()), float(y.max())],
+        "p_sum": float(P.astype(np.float64).sum()),
+    }
+    with open(os.path.join(HERE, "c0_fit.json"), "w") as f:
+        json.dump(out, f, indent=1)
+    print(out)
+
+
+if __name__ == "__main__":
+    small_case()
+    c0_fit()

@@ -176,3 +176,111 @@ def test_iterate_short(stages, c0_problem, start, steps):
     assert rel_l2(dy.cpu().numpy(), y_o) <= 1e-4
     assert abs(float(z.item()) - z_o) <= 1e-4 * abs(z_o)
     plan.close()
+
+
+@pytest.mark.parametrize("n,d,k,perp", [
+    (2, 2, 2, 1.5),         # smallest problem: self plus one neighbour
+    (50, 3, 50, 10.0),      # K == N, fewer points than one candidate tile
+    (333, 130, 17, 5.0),    # ragged sizes, more dimensions than one staging chunk
+    (1000, 7, 300, 60.0),   # wide rows: 64 lanes x 8 values in the perplexity search
+    (700, 5, 1, 1.0),       # K == 1: only self
+    (1300, 20, 1100, 300.0),  # K > 1024: generic row kernels
+])
+def test_one_shot_stages_edge_shapes(stages, n, d, k, perp):
+    from tsnecuda import synthetic
+    X = synthetic.gaussian_clusters(n, d=d, clusters=2, center_scale=2.0, seed=n)
+    idx_o, d2_o = oracle.knn(X, k)
+    idx, d2 = stages.knn(dev(X), k)
+    assert np.array_equal(idx.cpu().numpy(), idx_o)
+    assert np.array_equal(d2.cpu().numpy(), d2_o)
+    if k == 1:
+        return
+    dn_o, _ = oracle.max_normalize(d2_o)
+    dn = stages.max_normalize_(d2)
+    assert np.array_equal(dn.cpu().numpy(), dn_o)
+    p_o, beta_o, _ = oracle.perplexity(dn_o, perp, 1e-4, return_search=True)
+    p, beta = stages.perplexity(dn, perp, 1e-4, return_betas=True)
+    same = beta.cpu().numpy() == beta_o
+    assert same.mean() >= 0.9
+    np.testing.assert_allclose(p.cpu().numpy()[same], p_o[same], rtol=2e-5, atol=1e-30)
+    P_o = oracle.symmetrize(p_o, idx_o)
+    P = stages.symmetrize(dev(p_o), dev(idx_o)).cpu().numpy()
+    np.testing.assert_allclose(P, P_o, rtol=1e-6, atol=0)
+    # gradient stages on the same pattern
+    rng = np.random.default_rng(n)
+    y = (rng.standard_normal(2 * n) * 5.0).astype(np.float32)
+    plan = stages.Plan(n, k)
+    got = plan.attractive(dev(P_o), dev(idx_o), dev(y)).cpu().numpy()
+    assert rel_l2(got, oracle.attractive(P_o, idx_o, y)) <= 1e-4
+    rep, z = plan.repulsive(dev(y))
+    rep_o, z_o, _, _, phi_o = oracle.repulsive(y, details=True)
+    # rep = x*phi1 - phi2 cancels; with a handful of far-apart points the two
+    # terms are orders of magnitude larger than their difference, so the fp32
+    # noise of the transforms (~1e-6 of the terms) is what bounds the error.
+    terms = np.concatenate([y[:n] * phi_o[:, 0], phi_o[:, 1], y[n:] * phi_o[:, 0], phi_o[:, 2]])
+    cond = np.linalg.norm(terms) / np.linalg.norm(rep_o)
+    assert rel_l2(rep.cpu().numpy(), rep_o) <= max(1e-4, 2e-6 * cond)
+    # Z = sum_i z_i - N: the subtraction cancels when there are only a few far-apart points.
+    assert abs(float(z.item()) - z_o) <= 1e-4 * (abs(z_o) + n)
+    plan.close()
+
+
+def test_knn_duplicates_and_ties(stages):
+    # Exact duplicates: ties broken by lower index, self still first.
+    X = np.zeros((300, 4), np.float32)
+    X[100:] = 1.0
+    X[200:] = np.float32(2.5)
+    idx_o, d2_o = oracle.knn(X, 120)
+    idx, d2 = stages.knn(dev(X), 120)
+    assert np.array_equal(idx.cpu().numpy(), idx_o)
+    assert np.array_equal(d2.cpu().numpy(), d2_o)
+
+
+@pytest.mark.parametrize("nb", [4, 7, 33])
+def test_repulsive_reduced_grids(stages, nb):
+    """Other grid sizes than the reference's 130 boxes, against the oracle's
+    direct (no FFT) node-to-node sums where those are affordable."""
+    rng = np.random.default_rng(nb)
+    n = 900
+    y = (rng.standard_normal(2 * n) * 2.0).astype(np.float32)
+    plan = stages.Plan(n, 8, n_boxes_per_dim=nb)
+    rep, z, w, yt, phi = plan.repulsive(dev(y), details=True)
+    rep_o, z_o, w_o, yt_o, phi_o = oracle.repulsive(y, nb=nb, direct=(nb <= 7), details=True)
+    assert rel_l2(w.cpu().numpy(), w_o) <= 1e-5
+    assert rel_l2(yt.cpu().numpy(), yt_o) <= 2e-5
+    assert rel_l2(rep.cpu().numpy(), rep_o) <= 1e-4
+    assert abs(float(z.item()) - z_o) <= 1e-5 * abs(z_o)
+    plan.close()
+
+
+def test_golden_small256(stages):
+    """The committed 256-point fixture, stage by stage through the C ABI."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "small256.npz"))
+    k = g["idx"].shape[1]
+    idx, d2 = stages.knn(dev(g["X"]), k)
+    assert np.array_equal(idx.cpu().numpy(), g["idx"]) and np.array_equal(d2.cpu().numpy(), g["d2"])
+    p, beta = stages.perplexity(stages.max_normalize_(d2), float(g["perplexity"]), 1e-4, return_betas=True)
+    same = beta.cpu().numpy() == g["beta"]
+    assert same.mean() >= 0.95
+    np.testing.assert_allclose(p.cpu().numpy()[same], g["p"][same], rtol=1e-5, atol=1e-30)
+    np.testing.assert_allclose(stages.symmetrize(dev(g["p"]), dev(g["idx"])).cpu().numpy(), g["P"], rtol=1e-6)
+    plan = stages.Plan(256, k)
+    dy = dev(g["y"])
+    attr = plan.attractive(dev(g["P"]), dev(g["idx"]), dy)
+    rep, z = plan.repulsive(dy)
+    assert rel_l2(attr.cpu().numpy(), g["attr"]) <= 1e-4
+    assert rel_l2(rep.cpu().numpy(), g["rep"]) <= 1e-4
+    assert abs(float(z.item()) - float(g["z"])) <= 1e-5 * float(g["z"])
+    gains, old = torch.ones_like(dy), torch.zeros_like(dy)
+    plan.update_(dy, dev(g["attr"]), dev(g["rep"]), gains, old, 200.0, dev(np.array([g["z"]], np.float32)), 0.5, 12.0)
+    np.testing.assert_allclose(dy.cpu().numpy(), g["y1"], rtol=1e-6, atol=1e-9)
+    assert np.array_equal(gains.cpu().numpy(), g["g1"])
+    plan.close()
+
+
+def test_errors_are_reported(stages):
+    with pytest.raises(RuntimeError, match="exceeds num_points"):
+        stages.knn(dev(np.zeros((5, 2), np.float32)), 9)
+    with pytest.raises(RuntimeError, match="n_boxes_per_dim"):
+        stages.Plan(100, 5, n_boxes_per_dim=1000)

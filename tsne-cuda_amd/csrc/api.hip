@@ -31,7 +31,26 @@ bool sync_kernels_enabled() {
     return enabled;
 }
 
+int profile_mark(tsne_hip_plan *p, int id, hipStream_t s) {
+    if (!p->profiling) return 0;
+    if (p->events_used == p->events.size()) {
+        hipEvent_t e;
+        TSNE_TRY(hipEventCreate(&e));
+        p->events.push_back(e);
+    }
+    TSNE_TRY(hipEventRecord(p->events[p->events_used], s));
+    if (p->event_kernel.size() <= p->events_used) p->event_kernel.resize(p->events_used + 1);
+    p->event_kernel[p->events_used] = id;
+    p->events_used += 1;
+    return 0;
+}
+
 namespace {
+
+const char *const kLoopKernelNames[kKernelCount] = {
+    "step_prologue_kernel",     "kernel_rows_kernel",  "tile_count_kernel",        "tile_scan_kernel",
+    "tile_scatter_kernel",      "spread_kernel",       "conv_rows_forward_kernel", "conv_columns_kernel",
+    "conv_rows_inverse_kernel", "gather_forces_kernel", "attractive_kernel",       "update_kernel"};
 
 LagrangeConsts make_lagrange() {
     // fp32 arithmetic in the order of src/fit_tsne.cu:303-321.
@@ -119,7 +138,13 @@ int tsne_hip_symmetrize(const float *pij_non_symmetric, const int *indices, int 
 
 void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     if (!p) return;
+    for (hipEvent_t e : p->events) (void)hipEventDestroy(e);
     (void)hipFree(p->yxy);
+    (void)hipFree(p->tile_xy);
+    (void)hipFree(p->tile_count);
+    (void)hipFree(p->tile_cursor);
+    (void)hipFree(p->chunks);
+    (void)hipFree(p->num_chunks);
     (void)hipFree(p->node_charges);
     (void)hipFree(p->node_potentials);
     (void)hipFree(p->row_spectra);
@@ -152,7 +177,13 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
     const size_t G2 = (size_t)p->n_nodes * p->n_nodes;
     const size_t spec = (size_t)2 * kFft * kNodePad;
     const size_t N = (size_t)num_points;
+    p->max_chunks = (int)(N / kChunkPoints) + kMaxTiles + 1;
     bool ok = hipMalloc(&p->yxy, sizeof(float2) * N) == hipSuccess &&
+              hipMalloc(&p->tile_xy, sizeof(float2) * N) == hipSuccess &&
+              hipMalloc(&p->tile_count, sizeof(int) * kMaxTiles) == hipSuccess &&
+              hipMalloc(&p->tile_cursor, sizeof(int) * kMaxTiles) == hipSuccess &&
+              hipMalloc(&p->chunks, sizeof(int4) * p->max_chunks) == hipSuccess &&
+              hipMalloc(&p->num_chunks, sizeof(int)) == hipSuccess &&
               hipMalloc(&p->node_charges, sizeof(float4) * G2) == hipSuccess &&
               hipMalloc(&p->node_potentials, sizeof(float4) * G2) == hipSuccess &&
               hipMalloc(&p->row_spectra, sizeof(float2) * spec) == hipSuccess &&
@@ -170,6 +201,8 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
         }
         ok = hipMemcpy(p->twiddles, tw.data(), sizeof(float2) * kFft, hipMemcpyHostToDevice) == hipSuccess &&
              hipMemset(p->node_charges, 0, sizeof(float4) * G2) == hipSuccess &&
+             hipMemset(p->tile_count, 0, sizeof(int) * kMaxTiles) == hipSuccess &&
+             hipMemset(p->num_chunks, 0, sizeof(int)) == hipSuccess &&
              hipMemset(p->row_spectra, 0, sizeof(float2) * spec) == hipSuccess &&
              hipMemset(p->col_results, 0, sizeof(float2) * spec) == hipSuccess &&
              hipMemset(p->kernel_rows, 0, sizeof(float) * (size_t)(kFft / 2 + 1) * kNodePad) == hipSuccess &&
@@ -248,6 +281,41 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
             return 1;
         slot ^= 1;
     }
+    return profile_mark(plan, -1, s);
+}
+
+int tsne_hip_profile_kernel_count(void) { return kKernelCount; }
+
+const char *tsne_hip_profile_kernel_name(int id) {
+    return (id >= 0 && id < kKernelCount) ? kLoopKernelNames[id] : "";
+}
+
+int tsne_hip_profile_begin(tsne_hip_plan *plan) {
+    if (check_plan(plan, "profile_begin")) return 1;
+    plan->profiling = true;
+    plan->events_used = 0;
+    return 0;
+}
+
+int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches) {
+    if (check_plan(plan, "profile_end")) return 1;
+    TSNE_REQUIRE(total_ms && launches, "profile_end: null output");
+    plan->profiling = false;
+    for (int k = 0; k < kKernelCount; ++k) {
+        total_ms[k] = 0.0;
+        launches[k] = 0;
+    }
+    if (plan->events_used == 0) return 0;
+    TSNE_TRY(hipEventSynchronize(plan->events[plan->events_used - 1]));
+    for (size_t e = 0; e + 1 < plan->events_used; ++e) {
+        const int id = plan->event_kernel[e];
+        if (id < 0) continue;
+        float ms = 0.0f;
+        TSNE_TRY(hipEventElapsedTime(&ms, plan->events[e], plan->events[e + 1]));
+        total_ms[id] += ms;
+        launches[id] += 1;
+    }
+    plan->events_used = 0;
     return 0;
 }
 

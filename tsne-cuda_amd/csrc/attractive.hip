@@ -14,10 +14,67 @@ namespace tsnehip {
 
 namespace {
 
-template <int LANES>
+// A group of LANES lanes owns ROWS consecutive rows and covers each with SLOTS
+// strided slots (LANES * SLOTS >= K).  All index and probability loads of the
+// ROWS rows are issued before the first gather, and all gathers before the
+// arithmetic, so a wave keeps ROWS * SLOTS independent loads per lane in flight
+// instead of living for two short dependent round trips.
+template <int LANES, int SLOTS, int ROWS>
 __global__ __launch_bounds__(256) void attractive_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
                                                          const float2 *__restrict__ yxy, float *__restrict__ attr,
                                                          int N, int K) {
+    constexpr int kGroups = 256 / LANES;
+    const int lane = threadIdx.x % LANES;
+    const int row0 = (blockIdx.x * kGroups + threadIdx.x / LANES) * ROWS;
+    int j[ROWS][SLOTS];
+    float pv[ROWS][SLOTS];
+    float2 yi[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const int row = row0 + r;
+        const bool live = row < N;
+        const size_t base = (size_t)(live ? row : 0) * K;
+        yi[r] = yxy[live ? row : 0];
+#pragma unroll
+        for (int t = 0; t < SLOTS; ++t) {
+            const int s = lane + t * LANES;
+            const bool ok = live && s < K;
+            j[r][t] = ok ? idx[base + s] : 0;
+            pv[r][t] = ok ? pij[base + s] : 0.0f;  // zero weight for padding slots
+        }
+    }
+    float2 yj[ROWS][SLOTS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+        for (int t = 0; t < SLOTS; ++t) yj[r][t] = yxy[j[r][t]];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        float ax = 0.0f, ay = 0.0f;
+#pragma unroll
+        for (int t = 0; t < SLOTS; ++t) {
+            const float dx = yi[r].x - yj[r][t].x;
+            const float dy = yi[r].y - yj[r][t].y;
+            const float w = pv[r][t] * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
+            ax += w * dx;
+            ay += w * dy;
+        }
+        ax = group_sum<LANES>(ax);
+        ay = group_sum<LANES>(ay);
+        const int row = row0 + r;
+        if (lane == 0 && row < N) {
+            attr[row] = ax;
+            attr[N + row] = ay;
+        }
+    }
+}
+
+// Any K: LANES lanes per row, strided loop.
+template <int LANES>
+__global__ __launch_bounds__(256) void attractive_generic_kernel(const float *__restrict__ pij,
+                                                                 const int *__restrict__ idx,
+                                                                 const float2 *__restrict__ yxy,
+                                                                 float *__restrict__ attr, int N, int K) {
     constexpr int kRowsPerBlock = 256 / LANES;
     const int row = blockIdx.x * kRowsPerBlock + threadIdx.x / LANES;
     const int lane = threadIdx.x % LANES;
@@ -27,9 +84,9 @@ __global__ __launch_bounds__(256) void attractive_kernel(const float *__restrict
         const size_t base = (size_t)row * K;
 #pragma unroll 4
         for (int s = lane; s < K; s += LANES) {
-            const int j = idx[base + s];
+            const int jj = idx[base + s];
             const float pv = pij[base + s];
-            const float2 yj = yxy[j];
+            const float2 yj = yxy[jj];
             const float dx = yi.x - yj.x;
             const float dy = yi.y - yj.y;
             const float w = pv * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
@@ -62,13 +119,26 @@ int launch_pack_xy(tsne_hip_plan *p, const float *embedding, hipStream_t s) {
 // Expects plan->yxy to hold the current embedding as (x, y) pairs.
 int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, float *attr, hipStream_t s) {
     const int N = p->num_points, K = p->num_neighbors;
+    if (profile_mark(p, kKernelAttractive, s)) return 1;
+#define TSNE_ATTR(LANES, SLOTS, ROWS)                                                              \
+    attractive_kernel<LANES, SLOTS, ROWS><<<div_up(N, (256 / LANES) * ROWS), 256, 0, s>>>(pij, indices, p->yxy, \
+                                                                                          attr, N, K)
     if (K <= 16) {
-        attractive_kernel<16><<<div_up(N, 256 / 16), 256, 0, s>>>(pij, indices, p->yxy, attr, N, K);
+        TSNE_ATTR(16, 1, 8);
+    } else if (K <= 32) {
+        TSNE_ATTR(16, 2, 4);
+    } else if (K <= 64) {
+        TSNE_ATTR(32, 2, 4);
     } else if (K <= 96) {
-        attractive_kernel<32><<<div_up(N, 256 / 32), 256, 0, s>>>(pij, indices, p->yxy, attr, N, K);
+        TSNE_ATTR(32, 3, 4);
+    } else if (K <= 128) {
+        TSNE_ATTR(64, 2, 4);
+    } else if (K <= 256) {
+        TSNE_ATTR(64, 4, 2);
     } else {
-        attractive_kernel<64><<<div_up(N, 256 / 64), 256, 0, s>>>(pij, indices, p->yxy, attr, N, K);
+        attractive_generic_kernel<64><<<div_up(N, 256 / 64), 256, 0, s>>>(pij, indices, p->yxy, attr, N, K);
     }
+#undef TSNE_ATTR
     TSNE_LAUNCHED(s);
     return 0;
 }

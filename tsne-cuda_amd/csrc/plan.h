@@ -2,6 +2,8 @@
 #ifndef TSNE_HIP_PLAN_H_
 #define TSNE_HIP_PLAN_H_
 
+#include <vector>
+
 #include "common.h"
 
 namespace tsnehip {
@@ -11,12 +13,32 @@ constexpr int kTerms = 4;         // charges per point (src/fit_tsne.cu:254)
 constexpr int kFft = 1024;        // padded transform length, >= 2 * 3 * n_boxes - 1
 constexpr int kNodePad = 512;     // leading dimension of the transposed spectra (>= nodes per dim)
 constexpr int kMaxBoxes = 170;    // 3 * 170 = 510 nodes <= kNodePad
+constexpr int kTileBoxes = 10;    // boxes per side of a spreading tile (30 x 30 nodes, 14.4 KB in LDS)
+constexpr int kMaxTiles = 17 * 17;  // ceil(kMaxBoxes / kTileBoxes)^2
+constexpr int kChunkPoints = 2048;  // points one workgroup spreads into its private LDS tile
 
 // Lagrange node positions inside a box and the basis denominators, formed in
 // fp32 exactly as the reference does on the host (src/fit_tsne.cu:303-321).
 struct LagrangeConsts {
     float spacing[kInterp];
     float denom[kInterp];
+};
+
+// Kernels of one gradient step, in launch order (profiling slots).
+enum LoopKernel {
+    kKernelPrologue = 0,
+    kKernelKernelRows,
+    kKernelTileCount,
+    kKernelTileScan,
+    kKernelTileScatter,
+    kKernelSpread,
+    kKernelConvRowsForward,
+    kKernelConvColumns,
+    kKernelConvRowsInverse,
+    kKernelGather,
+    kKernelAttractive,
+    kKernelUpdate,
+    kKernelCount
 };
 
 }  // namespace tsnehip
@@ -30,6 +52,12 @@ struct tsne_hip_plan {
     tsnehip::LagrangeConsts lagrange;
 
     float2 *yxy = nullptr;         // N interleaved (x, y) pairs for the neighbour gathers
+    float2 *tile_xy = nullptr;     // N positions grouped by spreading tile (rebuilt every step)
+    int *tile_count = nullptr;     // points per tile
+    int *tile_cursor = nullptr;    // running write position per tile during the scatter
+    int4 *chunks = nullptr;        // (tile, first point, count, -) per spreading workgroup
+    int *num_chunks = nullptr;
+    int max_chunks = 0;
     float4 *node_charges = nullptr;     // n_nodes^2, one float4 (4 terms) per node
     float4 *node_potentials = nullptr;  // n_nodes^2
     float2 *row_spectra = nullptr;      // 2 plane pairs x kFft x kNodePad (transposed)
@@ -39,9 +67,20 @@ struct tsne_hip_plan {
     tsnehip::LoopScalars *scalars = nullptr;
     float *attr = nullptr;  // 2N, used by tsne_hip_iterate
     float *rep = nullptr;   // 2N
+
+    // Optional per-kernel timing: an event is recorded before every kernel of
+    // the loop and one after the last; a kernel's time is the gap to the next
+    // event on the same in-order stream.
+    bool profiling = false;
+    std::vector<hipEvent_t> events;
+    std::vector<int> event_kernel;  // kernel id per recorded event, -1 = end marker
+    size_t events_used = 0;
 };
 
 namespace tsnehip {
+
+// Records a profiling event for kernel `id` (no-op unless profiling is on).
+int profile_mark(tsne_hip_plan *p, int id, hipStream_t s);
 
 // Stage launchers shared between the stage-level ABI and the fused loop.
 // `slot` selects which pair of bounds in LoopScalars the launch reads.

@@ -161,9 +161,19 @@ __global__ __launch_bounds__(256) void bounds_kernel(const float *__restrict__ v
         lo = fminf(lo, x);
         hi = fmaxf(hi, x);
     }
+    __shared__ float wlo[256 / kWave], whi[256 / kWave];
     lo = group_min<kWave>(lo);
     hi = group_max<kWave>(hi);
     if ((threadIdx.x & (kWave - 1)) == 0) {
+        wlo[threadIdx.x / kWave] = lo;
+        whi[threadIdx.x / kWave] = hi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 1; k < 256 / kWave; ++k) {
+            lo = fminf(lo, wlo[k]);
+            hi = fmaxf(hi, whi[k]);
+        }
         atomicMin(&sc->min_enc[slot], float_to_ordered(lo));
         atomicMax(&sc->max_enc[slot], float_to_ordered(hi));
     }
@@ -172,8 +182,9 @@ __global__ __launch_bounds__(256) void bounds_kernel(const float *__restrict__ v
 // ---------------------------------------------------------------------------
 // Step prologue: clears Z and the bounds slot the coming update will fill.
 // ---------------------------------------------------------------------------
-__global__ void step_prologue_kernel(LoopScalars *sc, int next_slot) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
+__global__ void step_prologue_kernel(LoopScalars *sc, int next_slot, int *tile_count) {
+    if (threadIdx.x < kMaxTiles) tile_count[threadIdx.x] = 0;
+    if (threadIdx.x == 0) {
         sc->z_sum = 0.0f;
         if (next_slot >= 0) {
             sc->min_enc[next_slot] = 0xffffffffu;
@@ -184,32 +195,147 @@ __global__ void step_prologue_kernel(LoopScalars *sc, int next_slot) {
 
 // ---------------------------------------------------------------------------
 // Spread: w[node][t] += Lx_a * Ly_b * q[t] (src/kernels/nbodyfft.cu:107-139).
-// The row index of the node grid is the x node.  One thread per point, 36
-// hardware fp32 atomics into the L2-resident 2.4 MB grid.
+// The row index of the node grid is the x node.
+//
+// The reference issues 36 global atomics per point.  Nodes belong to exactly
+// one box, so here the points are first grouped by 10 x 10-box tile with a
+// counting sort (count, scan, scatter: positions only, the P matrix keeps its
+// order); then a workgroup takes up to 2048 points of one tile, accumulates
+// them into a private 30 x 30-node tile in LDS with LDS atomics, and adds the
+// non-zero nodes of its tile to the grid with one global atomic each.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void spread_kernel(const float *__restrict__ emb, int N, const LoopScalars *sc,
+__device__ __forceinline__ int box_of(float v, const Bounds &bd, int n_boxes) {
+#pragma clang fp contract(off)
+    int b = (int)((v - bd.lo) / bd.box_width);  // same expression as bin_and_weights
+    b = max(0, b);
+    return min(n_boxes - 1, b);
+}
+
+__device__ __forceinline__ int tile_of(float x, float y, const Bounds &bd, int n_boxes, int tiles_per_dim) {
+    return (box_of(y, bd, n_boxes) / kTileBoxes) * tiles_per_dim + box_of(x, bd, n_boxes) / kTileBoxes;
+}
+
+__global__ __launch_bounds__(256) void tile_count_kernel(const float *__restrict__ emb, int N, const LoopScalars *sc,
+                                                         int slot, int n_boxes, int *__restrict__ tile_count) {
+    __shared__ int hist[kMaxTiles];
+    const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
+    const int n_tiles = tiles_per_dim * tiles_per_dim;
+    for (int b = threadIdx.x; b < n_tiles; b += 256) hist[b] = 0;
+    __syncthreads();
+    const Bounds bd = load_bounds(sc, slot, n_boxes);
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < N; i += gridDim.x * 256)
+        atomicAdd(&hist[tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim)], 1);
+    __syncthreads();
+    for (int b = threadIdx.x; b < n_tiles; b += 256)
+        if (hist[b]) atomicAdd(&tile_count[b], hist[b]);
+}
+
+// One workgroup: exclusive scan of the tile counts and of the chunk counts,
+// write cursors, cut every tile into chunks of at most kChunkPoints points.
+__global__ __launch_bounds__(512) void tile_scan_kernel(const int *__restrict__ tile_count, int n_tiles,
+                                                        int *__restrict__ tile_cursor, int4 *__restrict__ chunks,
+                                                        int *__restrict__ num_chunks) {
+    __shared__ int pts[512], chk[512];
+    const int t = threadIdx.x;
+    const int cnt = t < n_tiles ? tile_count[t] : 0;
+    const int nchunk = (cnt + kChunkPoints - 1) / kChunkPoints;
+    pts[t] = cnt;
+    chk[t] = nchunk;
+    __syncthreads();
+    // Hillis-Steele inclusive scans over 512 slots.
+    for (int off = 1; off < 512; off <<= 1) {
+        const int a = t >= off ? pts[t - off] : 0;
+        const int b = t >= off ? chk[t - off] : 0;
+        __syncthreads();
+        pts[t] += a;
+        chk[t] += b;
+        __syncthreads();
+    }
+    const int first_point = pts[t] - cnt, first_chunk = chk[t] - nchunk;
+    if (t < n_tiles) {
+        tile_cursor[t] = first_point;
+        for (int c = 0; c < nchunk; ++c)
+            chunks[first_chunk + c] =
+                make_int4(t, first_point + c * kChunkPoints, min(kChunkPoints, cnt - c * kChunkPoints), 0);
+    }
+    if (t == 511) *num_chunks = chk[t];
+}
+
+// Same point-to-workgroup assignment as tile_count_kernel: the workgroup
+// reserves a run per tile with one global atomic, then ranks its points inside
+// the run with LDS atomics.
+__global__ __launch_bounds__(256) void tile_scatter_kernel(const float *__restrict__ emb, int N,
+                                                           const LoopScalars *sc, int slot, int n_boxes,
+                                                           int *__restrict__ tile_cursor,
+                                                           float2 *__restrict__ tile_xy) {
+    __shared__ int hist[kMaxTiles];
+    __shared__ int base[kMaxTiles];
+    const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
+    const int n_tiles = tiles_per_dim * tiles_per_dim;
+    for (int b = threadIdx.x; b < n_tiles; b += 256) hist[b] = 0;
+    __syncthreads();
+    const Bounds bd = load_bounds(sc, slot, n_boxes);
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < N; i += gridDim.x * 256)
+        atomicAdd(&hist[tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim)], 1);
+    __syncthreads();
+    for (int b = threadIdx.x; b < n_tiles; b += 256) {
+        base[b] = hist[b] ? atomicAdd(&tile_cursor[b], hist[b]) : 0;
+        hist[b] = 0;
+    }
+    __syncthreads();
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < N; i += gridDim.x * 256) {
+        const float x = emb[i], y = emb[N + i];
+        const int t = tile_of(x, y, bd, n_boxes, tiles_per_dim);
+        const int r = atomicAdd(&hist[t], 1);
+        tile_xy[base[t] + r] = make_float2(x, y);
+    }
+}
+
+__global__ __launch_bounds__(256) void spread_kernel(const float2 *__restrict__ tile_xy,
+                                                     const int4 *__restrict__ chunks,
+                                                     const int *__restrict__ num_chunks, const LoopScalars *sc,
                                                      int slot, int n_boxes, LagrangeConsts lc,
                                                      float *__restrict__ w) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= N) return;
+    constexpr int kTileNodes = kTileBoxes * kInterp;  // 30
+    __shared__ float acc[kTileNodes * kTileNodes * kTerms];
+    if ((int)blockIdx.x >= *num_chunks) return;
+    const int4 ch = chunks[blockIdx.x];
+    const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
+    const int bx0 = (ch.x % tiles_per_dim) * kTileBoxes;
+    const int by0 = (ch.x / tiles_per_dim) * kTileBoxes;
+    for (int e = threadIdx.x; e < kTileNodes * kTileNodes * kTerms; e += 256) acc[e] = 0.0f;
+    __syncthreads();
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    const float x = emb[i], y = emb[N + i];
-    int bx, by;
-    float Lx[kInterp], Ly[kInterp];
-    bin_and_weights(x, bd, n_boxes, lc, bx, Lx);
-    bin_and_weights(y, bd, n_boxes, lc, by, Ly);
+    for (int p = threadIdx.x; p < ch.z; p += 256) {
+        const float2 pt = tile_xy[ch.y + p];
+        const float x = pt.x, y = pt.y;
+        int bx, by;
+        float Lx[kInterp], Ly[kInterp];
+        bin_and_weights(x, bd, n_boxes, lc, bx, Lx);
+        bin_and_weights(y, bd, n_boxes, lc, by, Ly);
+        const float q3 = x * x + y * y;
+        const int nx = (bx - bx0) * kInterp, ny = (by - by0) * kInterp;
+#pragma unroll
+        for (int a = 0; a < kInterp; ++a) {
+#pragma unroll
+            for (int b = 0; b < kInterp; ++b) {
+                const float lw = Lx[a] * Ly[b];
+                float *dst = acc + ((nx + a) * kTileNodes + (ny + b)) * kTerms;
+                atomicAdd(dst + 0, lw);
+                atomicAdd(dst + 1, lw * x);
+                atomicAdd(dst + 2, lw * y);
+                atomicAdd(dst + 3, lw * q3);
+            }
+        }
+    }
+    __syncthreads();
     const int G = n_boxes * kInterp;
-    const float q3 = x * x + y * y;
-#pragma unroll
-    for (int a = 0; a < kInterp; ++a) {
-#pragma unroll
-        for (int b = 0; b < kInterp; ++b) {
-            const float lw = Lx[a] * Ly[b];
-            float *dst = w + ((size_t)(bx * kInterp + a) * G + (by * kInterp + b)) * kTerms;
-            atomicAdd(dst + 0, lw);
-            atomicAdd(dst + 1, lw * x);
-            atomicAdd(dst + 2, lw * y);
-            atomicAdd(dst + 3, lw * q3);
+    for (int e = threadIdx.x; e < kTileNodes * kTileNodes * kTerms; e += 256) {
+        const float v = acc[e];
+        if (v != 0.0f) {
+            const int node = e / kTerms, t = e % kTerms;
+            const int gx = bx0 * kInterp + node / kTileNodes, gy = by0 * kInterp + node % kTileNodes;
+            if (gx < G && gy < G) atomicAdd(w + ((size_t)gx * G + gy) * kTerms + t, v);
         }
     }
 }
@@ -477,24 +603,45 @@ int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_
 int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *rep, float *point_potentials,
                      float *charges_out, hipStream_t s) {
     const int N = p->num_points, G = p->n_nodes, nb = p->n_boxes;
-    step_prologue_kernel<<<1, 64, 0, s>>>(p->scalars, slot ^ 1);
+    if (profile_mark(p, kKernelPrologue, s)) return 1;
+    step_prologue_kernel<<<1, 320, 0, s>>>(p->scalars, slot ^ 1, p->tile_count);
     TSNE_LAUNCHED(s);
+    if (profile_mark(p, kKernelKernelRows, s)) return 1;
     kernel_rows_kernel<<<div_up(G, 4), 256, 0, s>>>(p->scalars, slot, nb, p->twiddles, p->kernel_rows);
     TSNE_LAUNCHED(s);
-    spread_kernel<<<div_up(N, 256), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
-                                                 reinterpret_cast<float *>(p->node_charges));
+    const int tiles_per_dim = (nb + kTileBoxes - 1) / kTileBoxes;
+    const int sort_blocks = std::min(div_up(N, 256 * 4), 1024);
+    if (profile_mark(p, kKernelTileCount, s)) return 1;
+    tile_count_kernel<<<sort_blocks, 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_count);
+    TSNE_LAUNCHED(s);
+    if (profile_mark(p, kKernelTileScan, s)) return 1;
+    tile_scan_kernel<<<1, 512, 0, s>>>(p->tile_count, tiles_per_dim * tiles_per_dim, p->tile_cursor, p->chunks,
+                                      p->num_chunks);
+    TSNE_LAUNCHED(s);
+    if (profile_mark(p, kKernelTileScatter, s)) return 1;
+    tile_scatter_kernel<<<sort_blocks, 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_cursor, p->tile_xy);
+    TSNE_LAUNCHED(s);
+    if (profile_mark(p, kKernelSpread, s)) return 1;
+    // Upper bound on the number of chunks; surplus workgroups exit at once.
+    const int spread_blocks = N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1;
+    spread_kernel<<<spread_blocks, 256, 0, s>>>(p->tile_xy, p->chunks, p->num_chunks, p->scalars, slot, nb,
+                                                p->lagrange, reinterpret_cast<float *>(p->node_charges));
     TSNE_LAUNCHED(s);
     if (charges_out)
         TSNE_TRY(hipMemcpyAsync(charges_out, p->node_charges, sizeof(float4) * (size_t)G * G,
                                 hipMemcpyDeviceToDevice, s));
+    if (profile_mark(p, kKernelConvRowsForward, s)) return 1;
     conv_rows_forward_kernel<<<div_up(G, 2), 256, 0, s>>>(p->node_charges, G, p->scalars, slot, p->twiddles,
                                                           p->row_spectra);
     TSNE_LAUNCHED(s);
+    if (profile_mark(p, kKernelConvColumns, s)) return 1;
     conv_columns_kernel<<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
     TSNE_LAUNCHED(s);
+    if (profile_mark(p, kKernelConvRowsInverse, s)) return 1;
     conv_rows_inverse_kernel<<<div_up(G, 2), 256, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
                                                           p->node_potentials);
     TSNE_LAUNCHED(s);
+    if (profile_mark(p, kKernelGather, s)) return 1;
     gather_forces_kernel<<<div_up(N, 256), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
                                                         p->node_potentials, rep, point_potentials, p->scalars);
     TSNE_LAUNCHED(s);

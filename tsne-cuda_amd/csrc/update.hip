@@ -59,9 +59,21 @@ __global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, fl
         }
     }
     if (FUSED) {
+        // One pair of atomics per workgroup: same-address atomics serialise.
+        __shared__ float wlo[256 / kWave], whi[256 / kWave];
         lo = group_min<kWave>(lo);
         hi = group_max<kWave>(hi);
         if ((threadIdx.x & (kWave - 1)) == 0) {
+            wlo[threadIdx.x / kWave] = lo;
+            whi[threadIdx.x / kWave] = hi;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int k = 1; k < 256 / kWave; ++k) {
+                lo = fminf(lo, wlo[k]);
+                hi = fmaxf(hi, whi[k]);
+            }
             atomicMin(&sc->min_enc[next_slot], float_to_ordered(lo));
             atomicMax(&sc->max_enc[next_slot], float_to_ordered(hi));
         }
@@ -99,7 +111,8 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
     const int N = p->num_points;
     const float *z_ptr = normalization ? normalization : &p->scalars->z_sum;
     const float z_offset = normalization ? 0.0f : (float)N;
-    const int blocks = div_up(N, 256);
+    const int blocks = std::min(div_up(N, 256), 2048);
+    if (profile_mark(p, kKernelUpdate, s)) return 1;
     if (next_slot >= 0) {
         update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_offset,
                                                    momentum, exaggeration, p->yxy, p->scalars, next_slot);

@@ -36,6 +36,12 @@ def lib():
         L.tsne_hip_iterate.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, c_int, c_int, c_int, c_float, c_float,
                                        c_float, c_float, _vp, _vp]
         L.tsne_hip_sum_squares.argtypes = [_vp, _vp, c_i64, _vp, _vp]
+        L.tsne_hip_profile_kernel_name.argtypes = [c_int]
+        L.tsne_hip_profile_kernel_name.restype = ctypes.c_char_p
+        L.tsne_hip_profile_begin.argtypes = [_vp]
+        L.tsne_hip_profile_end.argtypes = [_vp, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_int)]
+        for name in ("profile_begin", "profile_end", "profile_kernel_count"):
+            getattr(L, "tsne_hip_" + name).restype = c_int
         for name in ("knn", "max_normalize", "perplexity", "symmetrize", "plan_create", "attractive",
                      "repulsive", "update", "iterate", "sum_squares"):
             getattr(L, "tsne_hip_" + name).restype = c_int
@@ -146,6 +152,17 @@ class Plan(object):
                                       force_magnify_iters, eta, pre_momentum, post_momentum, early_exaggeration,
                                       _ptr(z), _stream()))
         return z
+
+    def profile_begin(self):
+        _check(lib().tsne_hip_profile_begin(self._h))
+
+    def profile_end(self):
+        """{kernel name: (total ms, launches)} of the iterate_ calls since profile_begin."""
+        n = lib().tsne_hip_profile_kernel_count()
+        ms = (ctypes.c_double * n)()
+        cnt = (ctypes.c_int * n)()
+        _check(lib().tsne_hip_profile_end(self._h, ms, cnt))
+        return {lib().tsne_hip_profile_kernel_name(i).decode(): (ms[i], cnt[i]) for i in range(n)}
 
     def sum_squares(self, values):
         out = torch.empty(1, dtype=torch.float32, device=self.device)
