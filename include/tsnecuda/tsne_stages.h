@@ -70,8 +70,18 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
                          int device);
 void tsne_hip_plan_destroy(tsne_hip_plan *plan);
 
+/* Re-blocks the fixed sparse pattern (pij, indices) once into the plan: entries
+ * grouped by (row strip, column partition) so that the attractive kernel can
+ * stage neighbour positions in LDS.  Costs 8 bytes per non-zero of device
+ * memory; pij and indices are not referenced after the call has completed on
+ * the stream.  Afterwards tsne_hip_attractive and tsne_hip_iterate accept
+ * pij = indices = NULL and use the re-blocked copy.  Has no counterpart in the
+ * reference (its P matrix stays in N x K order, src/fit_tsne.cu:153). */
+int tsne_hip_attractive_prepare(tsne_hip_plan *plan, const float *pij, const int *indices, void *stream);
+
 /* attr_i = sum_s P[i,s] (y_i - y_j) / (1 + |y_i - y_j|^2), j = idx[i,s].
- * Replaces tsnecuda::ComputeAttractiveForcesV3 (src/kernels/attr_forces.cu:186-240). */
+ * Replaces tsnecuda::ComputeAttractiveForcesV3 (src/kernels/attr_forces.cu:186-240).
+ * pij = indices = NULL: use the pattern given to tsne_hip_attractive_prepare. */
 int tsne_hip_attractive(tsne_hip_plan *plan, const float *pij, const int *indices, const float *embedding,
                         float *attractive_forces, void *stream);
 
@@ -96,7 +106,8 @@ int tsne_hip_update(tsne_hip_plan *plan, float *embedding, float *attractive_for
  * with no host synchronisation inside: bounds, Z and the schedule switch at
  * force_magnify_iters stay on the device.  embedding, gains and old_forces are
  * updated in place.  normalization (device scalar, may be NULL) receives the Z
- * of the last step. */
+ * of the last step.  pij = indices = NULL: use the pattern given to
+ * tsne_hip_attractive_prepare. */
 int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, float *embedding, float *gains,
                      float *old_forces, int step_begin, int step_end, int force_magnify_iters, float eta,
                      float pre_exaggeration_momentum, float post_exaggeration_momentum,

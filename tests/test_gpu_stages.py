@@ -284,3 +284,41 @@ def test_errors_are_reported(stages):
         stages.knn(dev(np.zeros((5, 2), np.float32)), 9)
     with pytest.raises(RuntimeError, match="n_boxes_per_dim"):
         stages.Plan(100, 5, n_boxes_per_dim=1000)
+
+
+@pytest.mark.parametrize("n,k", [(5000, 90), (20000, 30), (9000, 7), (300, 300)])
+def test_attractive_blocked_pattern(stages, n, k):
+    """The re-blocked (row strip x column partition) copy of the pattern gives
+    the same forces as the oracle; 20000 and 9000 points span several column
+    partitions, 300 x 300 is a dense pattern in a single bucket."""
+    rng = np.random.default_rng(n + k)
+    idx = np.stack([rng.permutation(n)[:k] for _ in range(n)]).astype(np.int32)
+    idx[:, 0] = np.arange(n)
+    P = (rng.random((n, k)) * 1e-5).astype(np.float32)
+    P[:, 0] = 0.0
+    y = (rng.standard_normal(2 * n) * 8.0).astype(np.float32)
+    want = oracle.attractive(P, idx, y)
+    plan = stages.Plan(n, k)
+    plan.prepare_attractive(dev(P), dev(idx))
+    got = plan.attractive(None, None, dev(y)).cpu().numpy()
+    assert rel_l2(got, want) <= 1e-4
+    # integer accumulation: the result does not depend on the order of the additions
+    again = plan.attractive(None, None, dev(y)).cpu().numpy()
+    assert np.array_equal(got, again)
+    plan.close()
+
+
+def test_iterate_with_prepared_pattern(stages, c0_problem):
+    c = c0_problem
+    n = c["X"].shape[0]
+    y_o, z_o = oracle.iterate(c["P"], c["idx"], c["y0"], 5)
+    plan = stages.Plan(n, c["K"])
+    plan.prepare_attractive(dev(c["P"]), dev(c["idx"]))
+    dy = dev(c["y0"])
+    gains, old = torch.ones_like(dy), torch.zeros_like(dy)
+    z = plan.iterate_(None, None, dy, gains, old, 0, 5)
+    assert rel_l2(dy.cpu().numpy(), y_o) <= 1e-4
+    assert abs(float(z.item()) - z_o) <= 1e-4 * abs(z_o)
+    plan.close()
+    with pytest.raises(RuntimeError, match="none prepared"):
+        stages.Plan(n, c["K"]).iterate_(None, None, dy, gains, old, 0, 1)

@@ -139,6 +139,7 @@ int tsne_hip_symmetrize(const float *pij_non_symmetric, const int *indices, int 
 void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     if (!p) return;
     for (hipEvent_t e : p->events) (void)hipEventDestroy(e);
+    release_blocked(p);
     (void)hipFree(p->yxy);
     (void)hipFree(p->tile_xy);
     (void)hipFree(p->tile_count);
@@ -178,7 +179,8 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
     const size_t spec = (size_t)2 * kFft * kNodePad;
     const size_t N = (size_t)num_points;
     p->max_chunks = (int)(N / kChunkPoints) + kMaxTiles + 1;
-    bool ok = hipMalloc(&p->yxy, sizeof(float2) * N) == hipSuccess &&
+    // yxy carries one spare pair so that two-point (float4) loads may straddle the end.
+    bool ok = hipMalloc(&p->yxy, sizeof(float2) * (N + 2)) == hipSuccess &&
               hipMalloc(&p->tile_xy, sizeof(float2) * N) == hipSuccess &&
               hipMalloc(&p->tile_count, sizeof(int) * kMaxTiles) == hipSuccess &&
               hipMalloc(&p->tile_cursor, sizeof(int) * kMaxTiles) == hipSuccess &&
@@ -200,6 +202,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
             tw[k] = make_float2((float)std::cos(ang), (float)std::sin(ang));
         }
         ok = hipMemcpy(p->twiddles, tw.data(), sizeof(float2) * kFft, hipMemcpyHostToDevice) == hipSuccess &&
+             hipMemset(p->yxy, 0, sizeof(float2) * (N + 2)) == hipSuccess &&
              hipMemset(p->node_charges, 0, sizeof(float4) * G2) == hipSuccess &&
              hipMemset(p->tile_count, 0, sizeof(int) * kMaxTiles) == hipSuccess &&
              hipMemset(p->num_chunks, 0, sizeof(int)) == hipSuccess &&
@@ -223,10 +226,18 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
 int tsne_hip_attractive(tsne_hip_plan *plan, const float *pij, const int *indices, const float *embedding,
                         float *attractive_forces, void *stream) {
     if (check_plan(plan, "attractive")) return 1;
-    TSNE_REQUIRE(pij && indices && embedding && attractive_forces, "attractive: null pointer argument");
+    TSNE_REQUIRE(embedding && attractive_forces, "attractive: null pointer argument");
+    TSNE_REQUIRE((pij == nullptr) == (indices == nullptr), "attractive: pij and indices must both be given or both be null");
     hipStream_t s = (hipStream_t)stream;
     if (launch_pack_xy(plan, embedding, s)) return 1;
+    if (!pij) return launch_attractive_blocked(plan, attractive_forces, s);
     return launch_attractive(plan, pij, indices, attractive_forces, s);
+}
+
+int tsne_hip_attractive_prepare(tsne_hip_plan *plan, const float *pij, const int *indices, void *stream) {
+    if (check_plan(plan, "attractive_prepare")) return 1;
+    TSNE_REQUIRE(pij && indices, "attractive_prepare: null pointer argument");
+    return prepare_blocked(plan, pij, indices, (hipStream_t)stream);
 }
 
 int tsne_hip_repulsive(tsne_hip_plan *plan, const float *embedding, float *repulsive_forces,
@@ -259,7 +270,9 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
                      float pre_exaggeration_momentum, float post_exaggeration_momentum,
                      float early_exaggeration, float *normalization, void *stream) {
     if (check_plan(plan, "iterate")) return 1;
-    TSNE_REQUIRE(pij && indices && embedding && gains && old_forces, "iterate: null pointer argument");
+    TSNE_REQUIRE(embedding && gains && old_forces, "iterate: null pointer argument");
+    TSNE_REQUIRE((pij == nullptr) == (indices == nullptr), "iterate: pij and indices must both be given or both be null");
+    TSNE_REQUIRE(pij || plan->blocked_ready, "iterate: no pattern given and none prepared");
     TSNE_REQUIRE(step_begin <= step_end, "iterate: step range [%d, %d) is reversed", step_begin, step_end);
     if (step_begin == step_end) return 0;
     hipStream_t s = (hipStream_t)stream;
@@ -274,7 +287,8 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
         const float momentum = late ? post_exaggeration_momentum : pre_exaggeration_momentum;
         const float exaggeration = late ? 1.0f : early_exaggeration;
         if (launch_repulsive(plan, embedding, slot, plan->rep, nullptr, nullptr, s)) return 1;
-        if (launch_attractive(plan, pij, indices, plan->attr, s)) return 1;
+        if (pij ? launch_attractive(plan, pij, indices, plan->attr, s) : launch_attractive_blocked(plan, plan->attr, s))
+            return 1;
         if (normalization && step == step_end - 1 && launch_finish_z(plan, normalization, s)) return 1;
         if (launch_update(plan, embedding, plan->attr, plan->rep, gains, old_forces, eta, nullptr, momentum,
                           exaggeration, slot ^ 1, s))

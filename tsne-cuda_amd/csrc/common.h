@@ -77,7 +77,7 @@ struct LoopScalars {
     unsigned int max_enc[2];  // ... and of the largest
     float z_sum;              // sum_i z_i of the current step (Z = z_sum - N)
     float sumsq;              // scratch for the gradient-norm reduction
-    float vmax;               // scratch for max-normalisation
+    float vmax;               // largest probability of the re-blocked pattern (fixed-point scale)
     float pad;
 };
 

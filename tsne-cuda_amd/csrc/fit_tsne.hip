@@ -201,6 +201,14 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     const int n_boxes_per_dim = 130;  // 125 rounded up in the reference's allowed list
     tsne_hip_plan *plan = nullptr;
     TSNE_OR_DIE(tsne_hip_plan_create(&plan, N, K, n_boxes_per_dim, gpu_opt.device), "plan creation");
+    // Re-block the sparse pattern for the LDS-staged attractive kernel; shapes it
+    // cannot hold (very large K or N) keep the row-ordered kernel.
+    const bool blocked = tsnehip::prepare_blocked(plan, d_pij.as<float>(), d_idx.as<int>(), stream) == 0;
+    if (blocked) {
+        hip_or_die(hipStreamSynchronize(stream), "pattern re-blocking");
+        d_pij.release();
+        d_idx.release();
+    }
 
     std::ofstream dump_file;
     if (opt.get_dump_points()) {
@@ -244,7 +252,8 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         TSNE_OR_DIE(tsnehip::launch_repulsive(plan, d_emb.as<float>(), slot, plan->rep, nullptr, nullptr, stream),
                     "repulsive forces");
         if (timing) hip_or_die(hipEventRecord(ev[1], stream), "event");
-        TSNE_OR_DIE(tsnehip::launch_attractive(plan, d_pij.as<float>(), d_idx.as<int>(), plan->attr, stream),
+        TSNE_OR_DIE(blocked ? tsnehip::launch_attractive_blocked(plan, plan->attr, stream)
+                            : tsnehip::launch_attractive(plan, d_pij.as<float>(), d_idx.as<int>(), plan->attr, stream),
                     "attractive forces");
         if (timing) hip_or_die(hipEventRecord(ev[2], stream), "event");
         if (step + 1 == iterations || want_stop)

@@ -68,6 +68,13 @@ struct tsne_hip_plan {
     float *attr = nullptr;  // 2N, used by tsne_hip_iterate
     float *rep = nullptr;   // 2N
 
+    // Re-blocked copy of the sparse pattern for the LDS-staged attractive kernel.
+    float *ent_p = nullptr;         // nnz probabilities, grouped by (row strip, column partition)
+    unsigned int *ent_c = nullptr;  // nnz packed (column within partition | row within strip << 14)
+    unsigned int *seg = nullptr;    // n_strips x (n_parts + 1) bucket offsets inside a strip
+    int strip_rows = 0, n_strips = 0, n_parts = 0;
+    bool blocked_ready = false;
+
     // Optional per-kernel timing: an event is recorded before every kernel of
     // the loop and one after the last; a kernel's time is the gap to the next
     // event on the same in-order stream.
@@ -92,6 +99,9 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
 int launch_finish_z(tsne_hip_plan *p, float *normalization, hipStream_t s);
 int launch_pack_xy(tsne_hip_plan *p, const float *embedding, hipStream_t s);
 int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, float *attr, hipStream_t s);
+int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s);
+void release_blocked(tsne_hip_plan *p);
+int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s);
 int launch_sum_squares(const float *values, int64_t n, float *out, hipStream_t s);
 int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, float *gains, float *old_forces,
                   float eta, const float *normalization, float momentum, float exaggeration, int next_slot,

@@ -31,6 +31,8 @@ def lib():
         L.tsne_hip_plan_destroy.argtypes = [_vp]
         L.tsne_hip_plan_destroy.restype = None
         L.tsne_hip_attractive.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp]
+        L.tsne_hip_attractive_prepare.argtypes = [_vp, _vp, _vp, _vp]
+        L.tsne_hip_attractive_prepare.restype = c_int
         L.tsne_hip_repulsive.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]
         L.tsne_hip_update.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, c_float, _vp, c_float, c_float, _vp]
         L.tsne_hip_iterate.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, c_int, c_int, c_int, c_float, c_float,
@@ -120,10 +122,15 @@ class Plan(object):
         except Exception:
             pass
 
+    def prepare_attractive(self, pij, idx):
+        """Re-blocks (pij, idx) into the plan; afterwards attractive() and
+        iterate_() may be called with pij = idx = None."""
+        _check(lib().tsne_hip_attractive_prepare(self._h, _ptr(_f32(pij)), _ptr(idx), _stream()))
+
     def attractive(self, pij, idx, embedding):
         out = torch.empty(2 * self.num_points, dtype=torch.float32, device=self.device)
-        _check(lib().tsne_hip_attractive(self._h, _ptr(_f32(pij)), _ptr(idx), _ptr(_f32(embedding)), _ptr(out),
-                                         _stream()))
+        _check(lib().tsne_hip_attractive(self._h, _ptr(None if pij is None else _f32(pij)), _ptr(idx),
+                                         _ptr(_f32(embedding)), _ptr(out), _stream()))
         return out
 
     def repulsive(self, embedding, details=False):
@@ -147,7 +154,8 @@ class Plan(object):
     def iterate_(self, pij, idx, embedding, gains, old_forces, step_begin, step_end, force_magnify_iters=250,
                  eta=200.0, pre_momentum=0.5, post_momentum=0.8, early_exaggeration=12.0):
         z = torch.zeros(1, dtype=torch.float32, device=self.device)
-        _check(lib().tsne_hip_iterate(self._h, _ptr(_f32(pij)), _ptr(idx), _ptr(_f32(embedding)),
+        _check(lib().tsne_hip_iterate(self._h, _ptr(None if pij is None else _f32(pij)), _ptr(idx),
+                                      _ptr(_f32(embedding)),
                                       _ptr(_f32(gains)), _ptr(_f32(old_forces)), step_begin, step_end,
                                       force_magnify_iters, eta, pre_momentum, post_momentum, early_exaggeration,
                                       _ptr(z), _stream()))
