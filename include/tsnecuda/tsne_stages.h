@@ -44,6 +44,16 @@ const char *tsne_hip_last_error(void);
 int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neighbors, int *indices,
                  float *sq_dist, void *stream);
 
+/* tsne_hip_knn with an explicit choice of the distance sweep: 0 = choose by
+ * shape (what tsne_hip_knn does), 1 = vector-ALU sweep, 2 = matrix-instruction
+ * (MFMA) candidate sweep followed by an exact re-rank and verification (at most
+ * 126 dimensions).  Results are identical whichever sweep runs.  stats (host
+ * pointer to two ints, may be NULL): [0] = 1 if the matrix sweep ran,
+ * [1] = queries the verification sent back to the vector sweep.  Same
+ * reference counterpart as tsne_hip_knn. */
+int tsne_hip_knn_select(const float *points, int num_points, int num_dims, int num_neighbors, int *indices,
+                        float *sq_dist, void *stream, int sweep, int *stats);
+
 /* In-place division of n values by their largest absolute value.
  * Replaces tsnecuda::util::MaxNormalizeDeviceVector (src/util/math_utils.cu:66-74). */
 int tsne_hip_max_normalize(float *values, int64_t n, void *stream);

@@ -322,3 +322,40 @@ def test_iterate_with_prepared_pattern(stages, c0_problem):
     plan.close()
     with pytest.raises(RuntimeError, match="none prepared"):
         stages.Plan(n, c["K"]).iterate_(None, None, dy, gains, old, 0, 1)
+
+
+@pytest.mark.parametrize("n,d,k", [
+    (3000, 50, 90),    # the benchmark's shape at small N
+    (700, 7, 20),      # odd dimension count, fewer candidates than the K' margin wants
+    (1500, 126, 33),   # the largest dimension count the matrix sweep takes
+    (40, 3, 40),       # K == N, a single partial tile
+    (2500, 33, 300),   # wide neighbour lists
+])
+def test_knn_matrix_sweep_is_exact(stages, n, d, k):
+    """The MFMA candidate sweep + exact re-rank gives the oracle's neighbours bit
+    for bit, and agrees with the vector sweep."""
+    from tsnecuda import synthetic
+    X = synthetic.gaussian_clusters(n, d=d, clusters=3, center_scale=6.0, seed=n + d)
+    idx_o, d2_o = oracle.knn(X, k)
+    idx, d2, stats = stages.knn_select(dev(X), k, 2)
+    assert stats[0] == 1
+    assert np.array_equal(idx.cpu().numpy(), idx_o)
+    assert np.array_equal(d2.cpu().numpy(), d2_o)
+    idx_v, d2_v, stats_v = stages.knn_select(dev(X), k, 1)
+    assert stats_v[0] == 0
+    assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
+
+
+def test_knn_matrix_sweep_verification_falls_back(stages):
+    """Points far from the origin with tiny mutual distances: the approximate
+    |c|^2 - 2 q.c distances cannot separate them, the verification must notice
+    and the vector sweep must repair every such query; duplicates tie on index."""
+    rng = np.random.default_rng(3)
+    base = rng.standard_normal((1, 16)).astype(np.float32) * 300.0
+    X = (base + rng.standard_normal((2000, 16)).astype(np.float32) * 1e-2).astype(np.float32)
+    X[1000:1100] = X[0:100]  # exact duplicates
+    idx_o, d2_o = oracle.knn(X, 25)
+    idx, d2, stats = stages.knn_select(dev(X), 25, 2)
+    assert stats[0] == 1 and stats[1] > 0
+    assert np.array_equal(idx.cpu().numpy(), idx_o)
+    assert np.array_equal(d2.cpu().numpy(), d2_o)

@@ -103,6 +103,14 @@ int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neig
     return run_knn(points, num_points, num_dims, num_neighbors, indices, sq_dist, (hipStream_t)stream);
 }
 
+int tsne_hip_knn_select(const float *points, int num_points, int num_dims, int num_neighbors, int *indices,
+                        float *sq_dist, void *stream, int sweep, int *stats) {
+    TSNE_REQUIRE(points && indices && sq_dist, "knn: null pointer argument");
+    TSNE_REQUIRE(sweep >= 0 && sweep <= 2, "knn: sweep must be 0 (choose), 1 (vector) or 2 (matrix), got %d", sweep);
+    return run_knn_mode(points, num_points, num_dims, num_neighbors, indices, sq_dist, (hipStream_t)stream, sweep,
+                        stats);
+}
+
 int tsne_hip_max_normalize(float *values, int64_t n, void *stream) {
     TSNE_REQUIRE(values && n > 0, "max_normalize: need a non-empty array");
     hipStream_t s = (hipStream_t)stream;

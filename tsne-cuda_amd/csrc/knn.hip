@@ -3,37 +3,59 @@
 // Stands in for the FAISS IVF-Flat search of the reference
 // (src/util/distance_utils.cu:79-121), which is approximate; this one is exact
 // and reproducible: the squared distance of a pair is accumulated in fp32 over
-// ascending dimension with one fused multiply-add per dimension, neighbours are
-// ordered by (distance, index), and the point itself is forced into slot 0 with
-// distance exactly 0 (the perplexity search depends on that,
-// src/kernels/perplexity_search.cu:30-32).
+// ascending dimension with one fused multiply-add per dimension ("canonical"
+// distance), neighbours are ordered by (distance, index), and the point itself
+// is forced into slot 0 with distance exactly 0 (the perplexity search depends
+// on that, src/kernels/perplexity_search.cu:30-32).
 //
-// Layout: the points are transposed once to [dim][point] so that a tile of
-// candidates is a run of contiguous floats per dimension.  A workgroup owns 64
-// queries and sweeps all candidates in tiles of 128; each thread keeps a 4 x 8
-// block of running distances in registers.  Selection is a filter against the
-// query's current k-th best (almost every candidate dies on one 64-bit
-// compare); survivors are appended to a per-query list that is compacted with
-// an LDS bitonic sort whenever a further tile might overflow it.
+// Two sweeps share the selection machinery (a per-query candidate list filtered
+// against the query's current k-th best and compacted by an LDS bitonic sort):
+//
+//  * VALU sweep: canonical distances directly, 64 queries x 128-candidate tiles,
+//    4 x 8 register block per thread.  Exact by construction; any dimension.
+//
+//  * MFMA sweep (up to 126 dimensions): v_mfma_f32_32x32x2f32 evaluates
+//    |c|^2 - 2 q.c for 32 candidates x 32 queries at a time.  The queries are
+//    the B operand and stay in registers for the whole sweep (scaled by -2,
+//    with one extra dimension that multiplies the candidate's |c|^2 by 1); the
+//    candidates stream through LDS in the A operand's lane layout.  A lane owns
+//    one query column of the 32 x 32 result, so filtering is a min over its 16
+//    accumulators against one threshold register.  These distances are only
+//    approximate (cancellation), so the sweep keeps K' > K candidates; a second
+//    kernel recomputes their canonical distances, sorts, and proves that nothing
+//    outside the list can belong to the top K: every discarded candidate has an
+//    approximate distance >= tau (the K'-th best), hence a canonical distance
+//    >= tau - g for a rigorous rounding bound g, and the query passes when its
+//    K-th canonical distance is below that.  Queries that do not pass are redone
+//    by the VALU sweep, so the result is exact either way.
 #include "common.h"
 
 #include <algorithm>
 #include <climits>
+#include <cmath>
+#include <vector>
 
 namespace tsnehip {
 
 namespace {
 
-constexpr int kQT = 64;   // queries per workgroup
-constexpr int kCT = 128;  // candidates per tile
-constexpr int kDC = 32;   // dimensions staged per chunk
-
 typedef unsigned long long u64;
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kQT = 64;   // VALU sweep: queries per workgroup
+constexpr int kCT = 128;  // candidates per tile (both sweeps)
+constexpr int kDC = 32;   // VALU sweep: dimensions staged per chunk
+constexpr int kMQ = 128;  // MFMA sweep: queries per workgroup (4 waves x 32)
+constexpr int kMfmaMaxSteps = 64;  // k-steps of 2 dimensions: up to 126 dimensions + 2 augmented
+static_assert(kMQ == kCT, "query tiles and candidate tiles share the packed layout");
 
 __device__ __forceinline__ u64 pack_key(float d, int j) {
     return ((u64)float_to_ordered(d) << 32) | (unsigned int)j;
 }
+__device__ __forceinline__ float key_distance(u64 key) { return ordered_to_float((unsigned int)(key >> 32)); }
+__device__ __forceinline__ int key_index(u64 key) { return (int)(unsigned int)(key & 0xffffffffu); }
 
+// Transposed copy of the points, [dim][point], padded to Npad points (vector sweep).
 __global__ __launch_bounds__(256) void transpose_points_kernel(const float *__restrict__ X, int N, int D, int Npad,
                                                                float *__restrict__ Xt) {
     __shared__ float tile[32][33];
@@ -48,6 +70,50 @@ __global__ __launch_bounds__(256) void transpose_points_kernel(const float *__re
         const int d = d0 + r, i = i0 + tx;
         if (d < D && i < Npad) Xt[(size_t)d * Npad + i] = tile[tx][r];
     }
+}
+
+// |x|^2 of every point (fp32, one fma per dimension) and the largest of them.
+__global__ __launch_bounds__(256) void norms_kernel(const float *__restrict__ X, int N, int D, int Npad,
+                                                    float *__restrict__ norms, float *__restrict__ max_norm) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    float nrm = 0.0f;
+    if (i < N) {
+        const float *x = X + (size_t)i * D;
+        for (int d = 0; d < D; ++d) nrm = fmaf(x[d], x[d], nrm);
+    }
+    if (i < Npad) norms[i] = nrm;
+    nrm = group_max<kWave>(nrm);
+    if ((threadIdx.x & (kWave - 1)) == 0) atomicMax(reinterpret_cast<unsigned int *>(max_norm), __float_as_uint(nrm));
+}
+
+// Points in the A-operand layout of v_mfma_f32_32x32x2f32, tile by tile, so that
+// a 128-candidate tile is one contiguous run of float4:
+//   Xp[tile][block of 32 points (4)][group of 4 k-steps (S4)][lane (64)] float4
+// where lane = (dimension % 2) * 32 + point % 32 and component = k-step % 4,
+// k-step = dimension / 2.  Dimension Dnorm carries |x|^2, padding is zero.
+__global__ __launch_bounds__(256) void pack_points_kernel(const float *__restrict__ X,
+                                                          const float *__restrict__ norms, int N, int D, int Dnorm,
+                                                          int S4, int Npad, float4 *__restrict__ Xp) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // one float4 of Xp per thread
+    const int64_t total = (int64_t)Npad * S4 * 2;
+    if (t >= total) return;
+    const int lane = (int)(t & 63);
+    const int64_t rest = t >> 6;
+    const int s4 = (int)(rest % S4);
+    const int64_t blk = rest / S4;  // tile * 4 + block
+    const int i = (int)(blk * 32 + (lane & 31));
+    const int h = lane >> 5;
+    float v[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int d = 2 * (4 * s4 + c) + h;
+        v[c] = 0.0f;
+        if (i < N) {
+            if (d < D) v[c] = X[(size_t)i * D + d];
+            else if (d == Dnorm) v[c] = norms[i];
+        }
+    }
+    Xp[t] = make_float4(v[0], v[1], v[2], v[3]);
 }
 
 // Sorts sortbuf[0..cap) ascending (cap a power of two), all 256 threads.
@@ -85,13 +151,18 @@ __device__ __forceinline__ void compact_query(u64 *list, int cap, int want, int 
     __syncthreads();
 }
 
+// ---------------------------------------------------------------------------
+// VALU sweep.  qlist == nullptr: queries are 0..N-1; otherwise the nq listed ones.
+// ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict__ Xt, int N, int Npad, int D, int K,
                                                         int cap, u64 *__restrict__ lists, int num_qtiles,
+                                                        const int *__restrict__ qlist, int nq,
                                                         int *__restrict__ out_idx, float *__restrict__ out_d) {
     __shared__ __attribute__((aligned(16))) float xq[kDC][kQT];
     __shared__ __attribute__((aligned(16))) float xc[kDC][kCT];
     __shared__ u64 thr[kQT];
     __shared__ int cnt[kQT];
+    __shared__ int qid[kQT];
     extern __shared__ u64 sortbuf[];
 
     const int tid = threadIdx.x;
@@ -100,10 +171,11 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
     u64 *list = lists + (size_t)blockIdx.x * kQT * cap;
 
     for (int qt = blockIdx.x; qt < num_qtiles; qt += gridDim.x) {
-        const int q0 = qt * kQT;
         if (tid < kQT) {
+            const int slot = qt * kQT + tid;
             thr[tid] = ~0ull;
             cnt[tid] = 0;
+            qid[tid] = slot < nq ? (qlist ? qlist[slot] : slot) : -1;
         }
         __syncthreads();
         for (int c0 = 0; c0 < N; c0 += kCT) {
@@ -115,10 +187,10 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
             for (int d0 = 0; d0 < D; d0 += kDC) {
                 const int dn = min(kDC, D - d0);
                 __syncthreads();
-                for (int e = tid; e < dn * (kQT / 4); e += 256) {
-                    const int dd = e / (kQT / 4), v = e % (kQT / 4);
-                    *reinterpret_cast<float4 *>(&xq[dd][v * 4]) =
-                        *reinterpret_cast<const float4 *>(Xt + (size_t)(d0 + dd) * Npad + q0 + v * 4);
+                for (int e = tid; e < dn * kQT; e += 256) {
+                    const int dd = e / kQT, ql = e % kQT;
+                    const int q = qid[ql];
+                    xq[dd][ql] = q >= 0 ? Xt[(size_t)(d0 + dd) * Npad + q] : 0.0f;
                 }
                 for (int e = tid; e < dn * (kCT / 4); e += 256) {
                     const int dd = e / (kCT / 4), v = e % (kCT / 4);
@@ -145,13 +217,13 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 const int ql = tq * 4 + a;
-                const int q = q0 + ql;
+                const int q = qid[ql];
                 const u64 limit = thr[ql];
 #pragma unroll
                 for (int b = 0; b < 8; ++b) {
                     const int j = c0 + tc * 8 + b;
                     const u64 key = pack_key(acc[a][b], j);
-                    if (j < N && q < N && j != q && key < limit) {
+                    if (j < N && q >= 0 && j != q && key < limit) {
                         const int slot = atomicAdd(&cnt[ql], 1);
                         list[(size_t)ql * cap + slot] = key;
                     }
@@ -166,22 +238,245 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
         }
         // Final ordering and output: self first, then the K-1 best others.
         for (int ql = 0; ql < kQT; ++ql) {
-            const int q = q0 + ql;
-            if (q >= N) break;
+            const int q = qid[ql];
+            if (q < 0) break;
             compact_query(list, cap, want, cnt, thr, ql, sortbuf, tid);
             for (int e = tid; e < K; e += 256) {
                 int j = q;
                 float d = 0.0f;
                 if (e > 0) {
                     const u64 key = sortbuf[e - 1];
-                    j = (int)(unsigned int)(key & 0xffffffffu);
-                    d = ordered_to_float((unsigned int)(key >> 32));
+                    j = key_index(key);
+                    d = key_distance(key);
                 }
                 out_idx[(size_t)q * K + e] = j;
                 out_d[(size_t)q * K + e] = d;
             }
             __syncthreads();
         }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// MFMA sweep.  KSTEPS = Daug / 2 k-steps of v_mfma_f32_32x32x2f32.
+// Dynamic LDS: two candidate tiles, copied verbatim from the packed points
+//   a[buf][cand block (4)][step group (S4)][lane (64)] float4   (4 steps per float4)
+// followed by the sort buffer (cap keys).
+// Output per query: the `want` best candidates by approximate distance
+// (cand, -1 padded) and tau = the approximate distance of the last one kept
+// (+inf when fewer than `want` candidates exist), both without the |q|^2 term.
+// ---------------------------------------------------------------------------
+template <int KSTEPS>
+__global__ __launch_bounds__(256) void knn_mfma_sweep_kernel(const float4 *__restrict__ Xp, int N, int D, int Dnorm,
+                                                             int want, int cap, u64 *__restrict__ lists,
+                                                             int num_qtiles, int *__restrict__ cand,
+                                                             float *__restrict__ tau) {
+    constexpr int S4 = (KSTEPS + 3) / 4;
+    constexpr int kTileFloat4 = 4 * S4 * 64;              // float4 per candidate tile
+    constexpr int kLoadsPerThread = kTileFloat4 / 256;    // == S4
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    float4 *a_lds = reinterpret_cast<float4 *>(lds_raw);
+    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + 2 * kTileFloat4);
+    __shared__ u64 thr[kMQ];
+    __shared__ int cnt[kMQ];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int qn = lane & 31, kh = lane >> 5;
+    u64 *list = lists + (size_t)blockIdx.x * kMQ * cap;
+
+    // One candidate tile: global -> registers (in flight during the matrix instructions) -> LDS.
+    float4 stage[kLoadsPerThread];
+    auto fetch = [&](int tile) {
+        const float4 *src = Xp + (size_t)tile * kTileFloat4 + tid;
+#pragma unroll
+        for (int r = 0; r < kLoadsPerThread; ++r) stage[r] = src[r * 256];
+    };
+    auto stash = [&](int buf) {
+        float4 *dst = a_lds + buf * kTileFloat4 + tid;
+#pragma unroll
+        for (int r = 0; r < kLoadsPerThread; ++r) dst[r * 256] = stage[r];
+    };
+    const int num_ctiles = (N + kCT - 1) / kCT;
+
+    for (int qt = blockIdx.x; qt < num_qtiles; qt += gridDim.x) {
+        const int q0 = qt * kMQ;
+        const int q = q0 + wave * 32 + qn;  // this lane's query (>= N in the last tile: padded zeros)
+        if (tid < kMQ) {
+            thr[tid] = ~0ull;
+            cnt[tid] = 0;
+        }
+        // B operand from the same packed layout (query tiles and candidate tiles coincide: kMQ == kCT):
+        // -2 q_d for the real dimensions, 1 for the |c|^2 row, 0 elsewhere.
+        float bq[4 * S4];
+        {
+            const float4 *src = Xp + (size_t)qt * kTileFloat4 + (size_t)wave * S4 * 64 + lane;
+#pragma unroll
+            for (int s4 = 0; s4 < S4; ++s4) {
+                const float4 v = src[s4 * 64];
+                const float c[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int d = 2 * (4 * s4 + k) + kh;
+                    bq[4 * s4 + k] = d < D ? -2.0f * c[k] : (d == Dnorm ? 1.0f : 0.0f);
+                }
+            }
+        }
+        fetch(0);
+        __syncthreads();
+        stash(0);
+        __syncthreads();
+        int buf = 0;
+        for (int ct = 0; ct < num_ctiles; ++ct) {
+            const int c0 = ct * kCT;
+            const bool more = ct + 1 < num_ctiles;
+            if (more) fetch(ct + 1);
+            const u64 limit = thr[wave * 32 + qn];
+            // ~0 is "no threshold yet": its distance field does not decode to a number.
+            const float limit_d = limit == ~0ull ? INFINITY : key_distance(limit);
+            // Two candidate blocks at a time: two independent accumulator chains keep the matrix pipe busy.
+#pragma unroll
+            for (int cb = 0; cb < 4; cb += 2) {
+                v16f acc0 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                v16f acc1 = acc0;
+                const float4 *a0 = a_lds + (size_t)(buf * 4 + cb) * S4 * 64 + lane;
+                const float4 *a1 = a0 + S4 * 64;
+#pragma unroll
+                for (int s4 = 0; s4 < S4; ++s4) {
+                    const float4 x = a0[s4 * 64], y = a1[s4 * 64];
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, bq[4 * s4], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.x, bq[4 * s4], acc1, 0, 0, 0);
+                    if (4 * s4 + 1 < KSTEPS) {
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, bq[4 * s4 + 1], acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.y, bq[4 * s4 + 1], acc1, 0, 0, 0);
+                    }
+                    if (4 * s4 + 2 < KSTEPS) {
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, bq[4 * s4 + 2], acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.z, bq[4 * s4 + 2], acc1, 0, 0, 0);
+                    }
+                    if (4 * s4 + 3 < KSTEPS) {
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, bq[4 * s4 + 3], acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.w, bq[4 * s4 + 3], acc1, 0, 0, 0);
+                    }
+                }
+                // Register v of lane l holds candidate row 8*(v/4) + 4*(l/32) + v%4 of the block, query column l%32.
+                float best = fminf(acc0[0], acc1[0]);
+#pragma unroll
+                for (int v = 1; v < 16; ++v) best = fminf(best, fminf(acc0[v], acc1[v]));
+                if (best <= limit_d) {
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const float dist = half ? acc1[v] : acc0[v];
+                            const int j = c0 + (cb + half) * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
+                            const u64 key = pack_key(dist, j);
+                            if (key < limit && j < N && j != q && q < N) {
+                                const int slot = atomicAdd(&cnt[wave * 32 + qn], 1);
+                                list[(size_t)(wave * 32 + qn) * cap + slot] = key;
+                            }
+                        }
+                    }
+                }
+            }
+            __syncthreads();  // all waves are done with tile `buf`; counters are final for this tile
+            const int crowded = (tid < kMQ) && (cnt[tid] > cap - kCT);
+            if (__syncthreads_or(crowded)) {
+                for (int ql = 0; ql < kMQ; ++ql)
+                    if (cnt[ql] > cap - kCT) compact_query(list, cap, want, cnt, thr, ql, sortbuf, tid);
+            }
+            if (more) {
+                stash(buf ^ 1);
+                __syncthreads();
+                buf ^= 1;
+            }
+        }
+        for (int ql = 0; ql < kMQ; ++ql) {
+            const int qq = q0 + ql;
+            if (qq >= N) break;
+            const int n = cnt[ql];
+            __syncthreads();
+            compact_query(list, cap, want, cnt, thr, ql, sortbuf, tid);
+            for (int e = tid; e < want; e += 256) cand[(size_t)qq * want + e] = e < n ? key_index(sortbuf[e]) : -1;
+            if (tid == 0) tau[qq] = n >= want ? key_distance(sortbuf[want - 1]) : INFINITY;
+            __syncthreads();
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Re-rank: canonical distances of a query's candidates, sort by (distance,
+// index), verify, write.  One wave per query, four queries per workgroup.
+// Dynamic LDS: 4 x sort_n keys.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void knn_rerank_kernel(const float *__restrict__ X,
+                                                         const float *__restrict__ norms, int N, int D, int K,
+                                                         int want, int sort_n, const int *__restrict__ cand,
+                                                         const float *__restrict__ tau,
+                                                         const float *__restrict__ max_norm,
+                                                         int *__restrict__ out_idx, float *__restrict__ out_d,
+                                                         int *__restrict__ fail_count, int *__restrict__ fail_list) {
+    extern __shared__ u64 keys_all[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int q = blockIdx.x * 4 + wave;
+    u64 *keys = keys_all + (size_t)wave * sort_n;
+    const bool live = q < N;
+    const float *xq = X + (size_t)(live ? q : 0) * D;
+    for (int c = lane; c < sort_n; c += kWave) {
+        u64 key = ~0ull;
+        if (live && c < want) {
+            const int j = cand[(size_t)q * want + c];
+            if (j >= 0) {
+                const float *xj = X + (size_t)j * D;
+                float acc = 0.0f;
+                for (int d = 0; d < D; ++d) {
+                    const float df = xq[d] - xj[d];
+                    acc = fmaf(df, df, acc);
+                }
+                key = pack_key(acc, j);
+            }
+        }
+        keys[c] = key;
+    }
+    __syncthreads();
+    // Bitonic sort of each wave's keys; all four waves run the same schedule.
+    for (int k = 2; k <= sort_n; k <<= 1) {
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int t = lane; t < sort_n / 2; t += kWave) {
+                const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+                const int hi = lo | j;
+                const bool up = (lo & k) == 0;
+                const u64 a = keys[lo], b = keys[hi];
+                if ((a > b) == up) {
+                    keys[lo] = b;
+                    keys[hi] = a;
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (!live) return;
+    // Every candidate outside the list has an approximate distance >= tau (without |q|^2), so its
+    // canonical distance is >= tau + |q|^2 - g.  g bounds |approximate - canonical|: both are sums of
+    // at most D + 3 rounded terms of magnitude <= (|q| + |c|)^2, and the canonical distance carries
+    // a relative error of (D + 2) 2^-24 of itself; a factor of four covers the matrix unit's
+    // accumulation order and the rounding of the stored norms.
+    const float kth = key_distance(keys[K - 2]);
+    const float t = tau[q];
+    bool pass = isinf(t) && t > 0.0f;
+    if (!pass) {
+        const double nq = norms[q], nmax = *max_norm;
+        const double eps = 5.9604644775390625e-08;  // 2^-24
+        const double g = 4.0 * (D + 4) * eps * (nq + nmax + 2.0 * sqrt(nq * nmax)) + (D + 4) * eps * (double)kth;
+        pass = (double)kth < (double)t + nq - g;
+    }
+    if (pass) {
+        for (int e = lane; e < K; e += kWave) {
+            out_idx[(size_t)q * K + e] = e == 0 ? q : key_index(keys[e - 1]);
+            out_d[(size_t)q * K + e] = e == 0 ? 0.0f : key_distance(keys[e - 1]);
+        }
+    } else if (lane == 0) {
+        fail_list[atomicAdd(fail_count, 1)] = q;
     }
 }
 
@@ -194,9 +489,89 @@ __global__ __launch_bounds__(256) void knn_self_only_kernel(int N, int *__restri
     }
 }
 
+struct DeviceMem {
+    void *p = nullptr;
+    ~DeviceMem() {
+        if (p) (void)hipFree(p);
+    }
+    bool alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 1) == hipSuccess; }
+    template <typename T>
+    T *as() const {
+        return static_cast<T *>(p);
+    }
+};
+
+int next_pow2(int v) {
+    int n = 1;
+    while (n < v) n <<= 1;
+    return n;
+}
+
+template <int KSTEPS>
+int launch_mfma_sweep(const float4 *Xp, int N, int D, int Dnorm, int want, int cap, u64 *lists, int num_qtiles,
+                      int grid, int *cand, float *tau, hipStream_t s) {
+    constexpr int S4 = (KSTEPS + 3) / 4;
+    const size_t lds = sizeof(float4) * 2 * 4 * S4 * 64 + sizeof(u64) * cap;
+    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_sweep_kernel<KSTEPS>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    knn_mfma_sweep_kernel<KSTEPS><<<grid, 256, lds, s>>>(Xp, N, D, Dnorm, want, cap, lists, num_qtiles, cand, tau);
+    TSNE_TRY(hipGetLastError());
+    return 0;
+}
+
+// Instantiated step counts: every count up to 32 (62 dimensions), then multiples of 4.
+int dispatch_mfma_sweep(int ksteps, const float4 *Xp, int N, int D, int Dnorm, int want, int cap, u64 *lists,
+                        int num_qtiles, int grid, int *cand, float *tau, hipStream_t s) {
+#define TSNE_MFMA_CASE(KS) \
+    case KS:               \
+        return launch_mfma_sweep<KS>(Xp, N, D, Dnorm, want, cap, lists, num_qtiles, grid, cand, tau, s);
+    switch (ksteps) {
+        TSNE_MFMA_CASE(2) TSNE_MFMA_CASE(3) TSNE_MFMA_CASE(4) TSNE_MFMA_CASE(5) TSNE_MFMA_CASE(6)
+        TSNE_MFMA_CASE(7) TSNE_MFMA_CASE(8) TSNE_MFMA_CASE(9) TSNE_MFMA_CASE(10) TSNE_MFMA_CASE(11)
+        TSNE_MFMA_CASE(12) TSNE_MFMA_CASE(13) TSNE_MFMA_CASE(14) TSNE_MFMA_CASE(15) TSNE_MFMA_CASE(16)
+        TSNE_MFMA_CASE(17) TSNE_MFMA_CASE(18) TSNE_MFMA_CASE(19) TSNE_MFMA_CASE(20) TSNE_MFMA_CASE(21)
+        TSNE_MFMA_CASE(22) TSNE_MFMA_CASE(23) TSNE_MFMA_CASE(24) TSNE_MFMA_CASE(25) TSNE_MFMA_CASE(26)
+        TSNE_MFMA_CASE(27) TSNE_MFMA_CASE(28) TSNE_MFMA_CASE(29) TSNE_MFMA_CASE(30) TSNE_MFMA_CASE(31)
+        TSNE_MFMA_CASE(32) TSNE_MFMA_CASE(36) TSNE_MFMA_CASE(40) TSNE_MFMA_CASE(44) TSNE_MFMA_CASE(48)
+        TSNE_MFMA_CASE(52) TSNE_MFMA_CASE(56) TSNE_MFMA_CASE(60) TSNE_MFMA_CASE(64)
+        default:
+            set_error("knn: no matrix-instruction sweep for %d steps", ksteps);
+            return 1;
+    }
+#undef TSNE_MFMA_CASE
+}
+
+int valu_cap(int K) {
+    int cap = 256;
+    while (cap < K - 1 + kCT) cap <<= 1;
+    return cap;
+}
+
+// VALU sweep over all points (qlist == nullptr) or over the nq listed queries.
+int run_valu_sweep(const float *Xt, int N, int Npad, int D, int K, const int *qlist, int nq, int cus, int *indices,
+                   float *sq_dist, hipStream_t s) {
+    const int cap = valu_cap(K);
+    const int num_qtiles = div_up(nq, kQT);
+    const int grid = std::min(num_qtiles, cus * 3);
+    DeviceMem lists;
+    if (!lists.alloc(sizeof(u64) * (size_t)grid * kQT * cap)) {
+        set_error("knn: out of device memory for the candidate lists");
+        return 1;
+    }
+    knn_sweep_kernel<<<grid, 256, sizeof(u64) * cap, s>>>(Xt, N, Npad, D, K, cap, lists.as<u64>(), num_qtiles, qlist,
+                                                          nq, indices, sq_dist);
+    TSNE_TRY(hipGetLastError());
+    TSNE_TRY(hipStreamSynchronize(s));
+    return 0;
+}
+
 }  // namespace
 
-int run_knn(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s) {
+// mode: 0 = choose, 1 = VALU sweep only, 2 = matrix-instruction sweep (error if the shape does not fit).
+// stats (optional, 2 ints): [0] = 1 if the matrix-instruction sweep ran, [1] = queries redone by the VALU sweep.
+int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s, int mode,
+                 int *stats) {
+    if (stats) stats[0] = stats[1] = 0;
     if (N <= 0 || D <= 0 || K <= 0) {
         set_error("knn: num_points, num_dims and num_neighbors must be positive (got %d, %d, %d)", N, D, K);
         return 1;
@@ -211,41 +586,87 @@ int run_knn(const float *points, int N, int D, int K, int *indices, float *sq_di
         TSNE_TRY(hipStreamSynchronize(s));
         return 0;
     }
-    int cap = 256;
-    while (cap < K - 1 + kCT) cap <<= 1;
-    if (cap > 4096) {
+    if (valu_cap(K) > 4096) {
         set_error("knn: num_neighbors = %d is not supported (limit %d)", K, 4096 - kCT + 1);
         return 1;
     }
-    const int Npad = div_up(N, kCT) * kCT;
-    const int num_qtiles = div_up(N, kQT);
     int device = 0, cus = 256;
     TSNE_TRY(hipGetDevice(&device));
     TSNE_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
-    const int grid = std::min(num_qtiles, cus * 3);
 
-    float *Xt = nullptr;
-    u64 *lists = nullptr;
-    TSNE_TRY(hipMalloc(&Xt, sizeof(float) * (size_t)D * Npad));
-    if (hipMalloc(&lists, sizeof(u64) * (size_t)grid * kQT * cap) != hipSuccess) {
-        (void)hipFree(Xt);
-        set_error("knn: out of device memory for the candidate lists");
+    // Matrix-instruction sweep geometry.
+    const int Dnorm = (D + 1) & ~1;        // |x|^2 row: first even row after the real dimensions
+    int ksteps = (Dnorm + 2) / 2;          // k-steps incl. the augmented pair
+    if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
+    const int want = std::min(N - 1, (K - 1) + std::max(32, (K - 1) / 2));  // K' candidates kept per query
+    const int mcap = next_pow2(want + kCT) < 256 ? 256 : next_pow2(want + kCT);
+    const size_t mfma_lds = sizeof(float4) * 2 * 4 * ((ksteps + 3) / 4) * 64 + sizeof(u64) * mcap;
+    const bool mfma_fits = ksteps <= kMfmaMaxSteps && mcap <= 4096 && mfma_lds <= 150 * 1024;
+    bool use_mfma = mode == 2 || (mode == 0 && mfma_fits && N >= 8192);
+    if (mode == 2 && !mfma_fits) {
+        set_error("knn: the matrix-instruction sweep does not fit %d dimensions / %d neighbours", D, K);
         return 1;
     }
-    int rc = 0;
-    do {
+
+    const int Npad = div_up(N, kCT) * kCT;
+    // Transposed points for the vector sweep (built only when that sweep runs).
+    DeviceMem Xt;
+    auto build_transposed = [&]() -> int {
+        if (!Xt.alloc(sizeof(float) * (size_t)D * Npad)) {
+            set_error("knn: out of device memory for the transposed points");
+            return 1;
+        }
         dim3 tgrid(div_up(Npad, 32), div_up(D, 32));
-        transpose_points_kernel<<<tgrid, 256, 0, s>>>(points, N, D, Npad, Xt);
-        if (hipGetLastError() != hipSuccess) { rc = 1; break; }
-        knn_sweep_kernel<<<grid, 256, sizeof(u64) * cap, s>>>(Xt, N, Npad, D, K, cap, lists, num_qtiles, indices,
-                                                              sq_dist);
-        if (hipGetLastError() != hipSuccess) { rc = 1; break; }
-        if (hipStreamSynchronize(s) != hipSuccess) { rc = 1; break; }
-    } while (0);
-    if (rc) set_error("knn: kernel launch or execution failed: %s", hipGetErrorString(hipGetLastError()));
-    (void)hipFree(Xt);
-    (void)hipFree(lists);
-    return rc;
+        transpose_points_kernel<<<tgrid, 256, 0, s>>>(points, N, D, Npad, Xt.as<float>());
+        TSNE_TRY(hipGetLastError());
+        return 0;
+    };
+    if (!use_mfma) {
+        if (build_transposed()) return 1;
+        return run_valu_sweep(Xt.as<float>(), N, Npad, D, K, nullptr, N, cus, indices, sq_dist, s);
+    }
+
+    const int S4 = (ksteps + 3) / 4;
+    DeviceMem Xp, norms, lists, cand, tau, scal, fail_list;
+    const int num_qtiles = div_up(N, kMQ);
+    const int grid = std::min(num_qtiles, cus * 2);
+    if (!Xp.alloc(sizeof(float4) * (size_t)Npad * S4 * 2) || !norms.alloc(sizeof(float) * Npad) ||
+        !lists.alloc(sizeof(u64) * (size_t)grid * kMQ * mcap) || !cand.alloc(sizeof(int) * (size_t)N * want) ||
+        !tau.alloc(sizeof(float) * N) || !scal.alloc(2 * sizeof(int)) || !fail_list.alloc(sizeof(int) * N)) {
+        set_error("knn: out of device memory for the candidate buffers");
+        return 1;
+    }
+    TSNE_TRY(hipMemsetAsync(scal.p, 0, 2 * sizeof(int), s));  // [0] max |x|^2 (float bits), [1] fail count
+    norms_kernel<<<div_up(Npad, 256), 256, 0, s>>>(points, N, D, Npad, norms.as<float>(), scal.as<float>());
+    TSNE_TRY(hipGetLastError());
+    pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm, S4,
+                                                                          Npad, Xp.as<float4>());
+    TSNE_TRY(hipGetLastError());
+    if (dispatch_mfma_sweep(ksteps, Xp.as<float4>(), N, D, Dnorm, want, mcap, lists.as<u64>(), num_qtiles, grid,
+                            cand.as<int>(), tau.as<float>(), s))
+        return 1;
+    const int sort_n = next_pow2(want) < 64 ? 64 : next_pow2(want);
+    knn_rerank_kernel<<<div_up(N, 4), 256, sizeof(u64) * 4 * sort_n, s>>>(
+        points, norms.as<float>(), N, D, K, want, sort_n, cand.as<int>(), tau.as<float>(), scal.as<float>(), indices,
+        sq_dist, scal.as<int>() + 1, fail_list.as<int>());
+    TSNE_TRY(hipGetLastError());
+    int host_scal[2] = {0, 0};
+    TSNE_TRY(hipMemcpyAsync(host_scal, scal.p, sizeof(host_scal), hipMemcpyDeviceToHost, s));
+    TSNE_TRY(hipStreamSynchronize(s));
+    const int failed = host_scal[1];
+    if (stats) {
+        stats[0] = 1;
+        stats[1] = failed;
+    }
+    if (failed > 0) {
+        if (build_transposed()) return 1;
+        return run_valu_sweep(Xt.as<float>(), N, Npad, D, K, fail_list.as<int>(), failed, cus, indices, sq_dist, s);
+    }
+    return 0;
+}
+
+int run_knn(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s) {
+    return run_knn_mode(points, N, D, K, indices, sq_dist, s, 0, nullptr);
 }
 
 }  // namespace tsnehip

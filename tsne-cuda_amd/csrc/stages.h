@@ -7,6 +7,8 @@
 namespace tsnehip {
 
 int run_knn(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s);
+int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s, int mode,
+                 int *stats);
 int launch_max_normalize(float *values, int64_t n, float *scratch, hipStream_t s);
 int launch_perplexity(const float *sq_dist, int N, int K, float perplexity, float eps, float *pij, float *betas,
                       hipStream_t s);

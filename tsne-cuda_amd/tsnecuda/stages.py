@@ -24,6 +24,8 @@ def lib():
         L.tsne_hip_last_error.restype = ctypes.c_char_p
         c_int, c_float, c_i64 = ctypes.c_int, ctypes.c_float, ctypes.c_int64
         L.tsne_hip_knn.argtypes = [_vp, c_int, c_int, c_int, _vp, _vp, _vp]
+        L.tsne_hip_knn_select.argtypes = [_vp, c_int, c_int, c_int, _vp, _vp, _vp, c_int, ctypes.POINTER(c_int)]
+        L.tsne_hip_knn_select.restype = c_int
         L.tsne_hip_max_normalize.argtypes = [_vp, c_i64, _vp]
         L.tsne_hip_perplexity.argtypes = [_vp, c_int, c_int, c_float, c_float, _vp, _vp, _vp]
         L.tsne_hip_symmetrize.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
@@ -76,6 +78,19 @@ def knn(points, num_neighbors):
     dist = torch.empty((n, num_neighbors), dtype=torch.float32, device=points.device)
     _check(lib().tsne_hip_knn(_ptr(points), n, d, num_neighbors, _ptr(idx), _ptr(dist), _stream()))
     return idx, dist
+
+
+def knn_select(points, num_neighbors, sweep):
+    """knn() with an explicit sweep (1 = vector ALU, 2 = matrix instructions).
+    Returns (indices, sq_dist, stats) with stats = (matrix sweep ran, queries redone)."""
+    points = _f32(points)
+    n, d = points.shape
+    idx = torch.empty((n, num_neighbors), dtype=torch.int32, device=points.device)
+    dist = torch.empty((n, num_neighbors), dtype=torch.float32, device=points.device)
+    stats = (ctypes.c_int * 2)()
+    _check(lib().tsne_hip_knn_select(_ptr(points), n, d, num_neighbors, _ptr(idx), _ptr(dist), _stream(), sweep,
+                                     stats))
+    return idx, dist, (int(stats[0]), int(stats[1]))
 
 
 def max_normalize_(values):
