@@ -41,6 +41,7 @@ namespace {
 
 typedef unsigned long long u64;
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kQT = 64;   // VALU sweep: queries per workgroup
 constexpr int kCT = 128;  // candidates per tile (both sweeps)
@@ -286,14 +287,16 @@ __global__ __launch_bounds__(256) void knn_mfma_sweep_kernel(const float4 *__res
     u64 *list = lists + (size_t)blockIdx.x * kMQ * cap;
 
     // One candidate tile: global -> registers (in flight during the matrix instructions) -> LDS.
-    float4 stage[kLoadsPerThread];
+    // The staging array is a native vector type with compile-time indices: as an array of
+    // HIP float4 structs it was placed in scratch memory, where every load waited for the last.
+    v4f stage[kLoadsPerThread];
     auto fetch = [&](int tile) {
-        const float4 *src = Xp + (size_t)tile * kTileFloat4 + tid;
+        const v4f *src = reinterpret_cast<const v4f *>(Xp) + (size_t)tile * kTileFloat4 + tid;
 #pragma unroll
         for (int r = 0; r < kLoadsPerThread; ++r) stage[r] = src[r * 256];
     };
     auto stash = [&](int buf) {
-        float4 *dst = a_lds + buf * kTileFloat4 + tid;
+        v4f *dst = reinterpret_cast<v4f *>(a_lds) + buf * kTileFloat4 + tid;
 #pragma unroll
         for (int r = 0; r < kLoadsPerThread; ++r) dst[r * 256] = stage[r];
     };
