@@ -13,9 +13,9 @@ constexpr int kTerms = 4;         // charges per point (src/fit_tsne.cu:254)
 constexpr int kFft = 1024;        // padded transform length, >= 2 * 3 * n_boxes - 1
 constexpr int kNodePad = 512;     // leading dimension of the transposed spectra (>= nodes per dim)
 constexpr int kMaxBoxes = 170;    // 3 * 170 = 510 nodes <= kNodePad
-constexpr int kTileBoxes = 10;    // boxes per side of a spreading tile (30 x 30 nodes, 14.4 KB in LDS)
+constexpr int kTileBoxes = 10;    // boxes per side of a spreading tile (30 x 30 nodes x 4 terms, 28.8 KB of LDS)
 constexpr int kMaxTiles = 17 * 17;  // ceil(kMaxBoxes / kTileBoxes)^2
-constexpr int kChunkPoints = 2048;  // points one workgroup spreads into its private LDS tile
+constexpr int kChunkPoints = 1024;  // points one workgroup spreads into its private LDS tile
 
 // Lagrange node positions inside a box and the basis denominators, formed in
 // fp32 exactly as the reference does on the host (src/fit_tsne.cu:303-321).

@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void bounds_kernel(const float *__restrict__ v
 // Step prologue: clears Z and the bounds slot the coming update will fill.
 // ---------------------------------------------------------------------------
 __global__ void step_prologue_kernel(LoopScalars *sc, int next_slot, int *tile_count) {
-    if (threadIdx.x < kMaxTiles) tile_count[threadIdx.x] = 0;
+    for (int t = threadIdx.x; t < kMaxTiles; t += blockDim.x) tile_count[t] = 0;
     if (threadIdx.x == 0) {
         sc->z_sum = 0.0f;
         if (next_slot >= 0) {
@@ -200,7 +200,7 @@ __global__ void step_prologue_kernel(LoopScalars *sc, int next_slot, int *tile_c
 // The reference issues 36 global atomics per point.  Nodes belong to exactly
 // one box, so here the points are first grouped by 10 x 10-box tile with a
 // counting sort (count, scan, scatter: positions only, the P matrix keeps its
-// order); then a workgroup takes up to 2048 points of one tile, accumulates
+// order); then a workgroup takes up to 1024 points of one tile, accumulates
 // them into a private 30 x 30-node tile in LDS with (integer) LDS atomics, and
 // adds the non-zero nodes of its tile to the grid with one global atomic each.
 // ---------------------------------------------------------------------------
@@ -215,35 +215,42 @@ __device__ __forceinline__ int tile_of(float x, float y, const Bounds &bd, int n
     return (box_of(y, bd, n_boxes) / kTileBoxes) * tiles_per_dim + box_of(x, bd, n_boxes) / kTileBoxes;
 }
 
-__global__ __launch_bounds__(256) void tile_count_kernel(const float *__restrict__ emb, int N, const LoopScalars *sc,
+__global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restrict__ emb, int N, const LoopScalars *sc,
                                                          int slot, int n_boxes, int *__restrict__ tile_count) {
     __shared__ int hist[kMaxTiles];
     const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
     const int n_tiles = tiles_per_dim * tiles_per_dim;
-    for (int b = threadIdx.x; b < n_tiles; b += 256) hist[b] = 0;
+    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;
     __syncthreads();
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < N; i += gridDim.x * 256)
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x)
         atomicAdd(&hist[tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim)], 1);
     __syncthreads();
-    for (int b = threadIdx.x; b < n_tiles; b += 256)
+    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x)
         if (hist[b]) atomicAdd(&tile_count[b], hist[b]);
 }
 
 // One workgroup: exclusive scan of the tile counts and of the chunk counts,
 // write cursors, cut every tile into chunks of at most kChunkPoints points.
-__global__ __launch_bounds__(512) void tile_scan_kernel(const int *__restrict__ tile_count, int n_tiles,
-                                                        int *__restrict__ tile_cursor, int4 *__restrict__ chunks,
-                                                        int *__restrict__ num_chunks) {
-    __shared__ int pts[512], chk[512];
+// Two tiles per thread (kMaxTiles <= 2 * 1024).
+__global__ __launch_bounds__(1024) void tile_scan_kernel(const int *__restrict__ tile_count, int n_tiles,
+                                                         int *__restrict__ tile_cursor, int4 *__restrict__ chunks,
+                                                         int *__restrict__ num_chunks) {
+    static_assert(kMaxTiles <= 2048, "the scan handles two tiles per thread");
+    __shared__ int pts[1024], chk[1024];
     const int t = threadIdx.x;
-    const int cnt = t < n_tiles ? tile_count[t] : 0;
-    const int nchunk = (cnt + kChunkPoints - 1) / kChunkPoints;
-    pts[t] = cnt;
-    chk[t] = nchunk;
+    int cnt[2], nchunk[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int tile = 2 * t + k;
+        cnt[k] = tile < n_tiles ? tile_count[tile] : 0;
+        nchunk[k] = (cnt[k] + kChunkPoints - 1) / kChunkPoints;
+    }
+    pts[t] = cnt[0] + cnt[1];
+    chk[t] = nchunk[0] + nchunk[1];
     __syncthreads();
-    // Hillis-Steele inclusive scans over 512 slots.
-    for (int off = 1; off < 512; off <<= 1) {
+    // Hillis-Steele inclusive scans over 1024 slots.
+    for (int off = 1; off < 1024; off <<= 1) {
         const int a = t >= off ? pts[t - off] : 0;
         const int b = t >= off ? chk[t - off] : 0;
         __syncthreads();
@@ -251,20 +258,26 @@ __global__ __launch_bounds__(512) void tile_scan_kernel(const int *__restrict__ 
         chk[t] += b;
         __syncthreads();
     }
-    const int first_point = pts[t] - cnt, first_chunk = chk[t] - nchunk;
-    if (t < n_tiles) {
-        tile_cursor[t] = first_point;
-        for (int c = 0; c < nchunk; ++c)
-            chunks[first_chunk + c] =
-                make_int4(t, first_point + c * kChunkPoints, min(kChunkPoints, cnt - c * kChunkPoints), 0);
+    int first_point = pts[t] - cnt[0] - cnt[1], first_chunk = chk[t] - nchunk[0] - nchunk[1];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int tile = 2 * t + k;
+        if (tile < n_tiles) {
+            tile_cursor[tile] = first_point;
+            for (int c = 0; c < nchunk[k]; ++c)
+                chunks[first_chunk + c] =
+                    make_int4(tile, first_point + c * kChunkPoints, min(kChunkPoints, cnt[k] - c * kChunkPoints), 0);
+        }
+        first_point += cnt[k];
+        first_chunk += nchunk[k];
     }
-    if (t == 511) *num_chunks = chk[t];
+    if (t == 1023) *num_chunks = chk[t];
 }
 
 // Same point-to-workgroup assignment as tile_count_kernel: the workgroup
 // reserves a run per tile with one global atomic, then ranks its points inside
 // the run with LDS atomics.
-__global__ __launch_bounds__(256) void tile_scatter_kernel(const float *__restrict__ emb, int N,
+__global__ __launch_bounds__(1024) void tile_scatter_kernel(const float *__restrict__ emb, int N,
                                                            const LoopScalars *sc, int slot, int n_boxes,
                                                            int *__restrict__ tile_cursor,
                                                            float2 *__restrict__ tile_xy) {
@@ -272,18 +285,18 @@ __global__ __launch_bounds__(256) void tile_scatter_kernel(const float *__restri
     __shared__ int base[kMaxTiles];
     const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
     const int n_tiles = tiles_per_dim * tiles_per_dim;
-    for (int b = threadIdx.x; b < n_tiles; b += 256) hist[b] = 0;
+    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;
     __syncthreads();
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < N; i += gridDim.x * 256)
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x)
         atomicAdd(&hist[tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim)], 1);
     __syncthreads();
-    for (int b = threadIdx.x; b < n_tiles; b += 256) {
+    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) {
         base[b] = hist[b] ? atomicAdd(&tile_cursor[b], hist[b]) : 0;
         hist[b] = 0;
     }
     __syncthreads();
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < N; i += gridDim.x * 256) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
         const float x = emb[i], y = emb[N + i];
         const int t = tile_of(x, y, bd, n_boxes, tiles_per_dim);
         const int r = atomicAdd(&hist[t], 1);
@@ -295,6 +308,8 @@ __global__ __launch_bounds__(256) void tile_scatter_kernel(const float *__restri
 // coordinate and |Lx * Ly| <= 1.875^2 < 4, a contribution to plane t is bounded by
 // B = (4, 4m, 4m, 8m^2); the scale 2^50 / B keeps a contribution below 2^50 and
 // the sum of a chunk's 2048 contributions below 2^61.
+constexpr int kSpreadThreads = 512;  // per chunk of kChunkPoints points: the chunk's critical path sets the kernel time
+
 struct SpreadScales {
     double to_fixed[kTerms];
     double from_fixed[kTerms];
@@ -323,7 +338,7 @@ __device__ __forceinline__ void add_fixed(unsigned long long *dst, float v, doub
 // 64-bit integer LDS atomics are about 25x faster, so the private tile is kept
 // in 64-bit fixed point (which also makes a chunk's sums independent of the
 // order of the additions) and converted to fp32 when it is flushed.
-__global__ __launch_bounds__(256) void spread_kernel(const float2 *__restrict__ tile_xy,
+__global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__restrict__ tile_xy,
                                                      const int4 *__restrict__ chunks,
                                                      const int *__restrict__ num_chunks, const LoopScalars *sc,
                                                      int slot, int n_boxes, LagrangeConsts lc,
@@ -335,11 +350,11 @@ __global__ __launch_bounds__(256) void spread_kernel(const float2 *__restrict__ 
     const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
     const int bx0 = (ch.x % tiles_per_dim) * kTileBoxes;
     const int by0 = (ch.x / tiles_per_dim) * kTileBoxes;
-    for (int e = threadIdx.x; e < kTileNodes * kTileNodes * kTerms; e += 256) acc[e] = 0ull;
+    for (int e = threadIdx.x; e < kTileNodes * kTileNodes * kTerms; e += kSpreadThreads) acc[e] = 0ull;
     __syncthreads();
     const Bounds bd = load_bounds(sc, slot, n_boxes);
     const SpreadScales fx = spread_scales(sc, slot);
-    for (int p = threadIdx.x; p < ch.z; p += 256) {
+    for (int p = threadIdx.x; p < ch.z; p += kSpreadThreads) {
         const float2 pt = tile_xy[ch.y + p];
         const float x = pt.x, y = pt.y;
         int bx, by;
@@ -363,7 +378,7 @@ __global__ __launch_bounds__(256) void spread_kernel(const float2 *__restrict__ 
     }
     __syncthreads();
     const int G = n_boxes * kInterp;
-    for (int e = threadIdx.x; e < kTileNodes * kTileNodes * kTerms; e += 256) {
+    for (int e = threadIdx.x; e < kTileNodes * kTileNodes * kTerms; e += kSpreadThreads) {
         const long long v = (long long)acc[e];
         if (v != 0) {
             const int node = e / kTerms, t = e % kTerms;
@@ -565,16 +580,17 @@ __global__ __launch_bounds__(256) void gather_forces_kernel(const float *__restr
                                                             float *__restrict__ rep, float *__restrict__ phi_out,
                                                             LoopScalars *sc) {
     __shared__ float partial[256 / kWave];
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const Bounds bd = load_bounds(sc_in, slot, n_boxes);
+    const int G = n_boxes * kInterp;
     float z = 0.0f;
-    if (i < N) {
-        const Bounds bd = load_bounds(sc_in, slot, n_boxes);
+    // Grid-stride: the workgroup count stays small because every workgroup ends with an atomic on
+    // the one Z accumulator, and same-address atomics serialise.
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
         const float x = emb[i], y = emb[N + i];
         int bx, by;
         float Lx[kInterp], Ly[kInterp];
         bin_and_weights(x, bd, n_boxes, lc, bx, Lx);
         bin_and_weights(y, bd, n_boxes, lc, by, Ly);
-        const int G = n_boxes * kInterp;
         float4 phi = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
         for (int a = 0; a < kInterp; ++a) {
@@ -588,7 +604,7 @@ __global__ __launch_bounds__(256) void gather_forces_kernel(const float *__restr
                 phi.w += lw * yt.w;
             }
         }
-        z = (1 + x * x + y * y) * phi.x - 2 * (x * phi.y + y * phi.z) + phi.w;
+        z += (1 + x * x + y * y) * phi.x - 2 * (x * phi.y + y * phi.z) + phi.w;
         rep[i] = x * phi.x - phi.y;
         rep[N + i] = y * phi.x - phi.z;
         if (phi_out) reinterpret_cast<float4 *>(phi_out)[i] = phi;
@@ -638,27 +654,29 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
                      float *charges_out, hipStream_t s) {
     const int N = p->num_points, G = p->n_nodes, nb = p->n_boxes;
     if (profile_mark(p, kKernelPrologue, s)) return 1;
-    step_prologue_kernel<<<1, 320, 0, s>>>(p->scalars, slot ^ 1, p->tile_count);
+    step_prologue_kernel<<<1, 256, 0, s>>>(p->scalars, slot ^ 1, p->tile_count);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelKernelRows, s)) return 1;
     kernel_rows_kernel<<<div_up(G, 4), 256, 0, s>>>(p->scalars, slot, nb, p->twiddles, p->kernel_rows);
     TSNE_LAUNCHED(s);
     const int tiles_per_dim = (nb + kTileBoxes - 1) / kTileBoxes;
-    const int sort_blocks = std::min(div_up(N, 256 * 4), 1024);
+    // Few, large workgroups: every workgroup ends with one global atomic per tile counter, and
+    // same-address atomics serialise (about a thousand per counter cost ~20 us).
+    const int sort_blocks = std::min(div_up(N, 1024 * 4), 256);
     if (profile_mark(p, kKernelTileCount, s)) return 1;
-    tile_count_kernel<<<sort_blocks, 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_count);
+    tile_count_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_count);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelTileScan, s)) return 1;
-    tile_scan_kernel<<<1, 512, 0, s>>>(p->tile_count, tiles_per_dim * tiles_per_dim, p->tile_cursor, p->chunks,
+    tile_scan_kernel<<<1, 1024, 0, s>>>(p->tile_count, tiles_per_dim * tiles_per_dim, p->tile_cursor, p->chunks,
                                       p->num_chunks);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelTileScatter, s)) return 1;
-    tile_scatter_kernel<<<sort_blocks, 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_cursor, p->tile_xy);
+    tile_scatter_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_cursor, p->tile_xy);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelSpread, s)) return 1;
     // Upper bound on the number of chunks; surplus workgroups exit at once.
     const int spread_blocks = N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1;
-    spread_kernel<<<spread_blocks, 256, 0, s>>>(p->tile_xy, p->chunks, p->num_chunks, p->scalars, slot, nb,
+    spread_kernel<<<spread_blocks, kSpreadThreads, 0, s>>>(p->tile_xy, p->chunks, p->num_chunks, p->scalars, slot, nb,
                                                 p->lagrange, reinterpret_cast<float *>(p->node_charges));
     TSNE_LAUNCHED(s);
     if (charges_out)
@@ -676,7 +694,7 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
                                                           p->node_potentials);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelGather, s)) return 1;
-    gather_forces_kernel<<<div_up(N, 256), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
+    gather_forces_kernel<<<std::min(div_up(N, 256), 1024), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
                                                         p->node_potentials, rep, point_potentials, p->scalars);
     TSNE_LAUNCHED(s);
     return 0;

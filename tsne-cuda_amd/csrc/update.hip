@@ -9,6 +9,7 @@
 #include "plan.h"
 
 #include <algorithm>
+#include <cstdint>
 
 namespace tsnehip {
 
@@ -80,6 +81,77 @@ __global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, fl
     }
 }
 
+// Four consecutive points per thread, 16-byte accesses.  Requires N % 4 == 0 and 16-byte aligned
+// arrays (then the y halves at offset N are aligned too).
+template <bool FUSED>
+__global__ __launch_bounds__(256) void update_vec4_kernel(float *__restrict__ emb, float *__restrict__ attr,
+                                                          float *__restrict__ rep, float *__restrict__ gains,
+                                                          float *__restrict__ old, int N, float eta,
+                                                          const float *__restrict__ z_ptr, float z_offset,
+                                                          float momentum, float exaggeration,
+                                                          float2 *__restrict__ yxy, LoopScalars *sc, int next_slot) {
+    const float normalization = *z_ptr - z_offset;
+    float lo = INFINITY, hi = -INFINITY;
+    const int n4 = N / 4;
+    float4 *emb4 = reinterpret_cast<float4 *>(emb), *attr4 = reinterpret_cast<float4 *>(attr);
+    float4 *rep4 = reinterpret_cast<float4 *>(rep), *gains4 = reinterpret_cast<float4 *>(gains);
+    float4 *old4 = reinterpret_cast<float4 *>(old);
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += gridDim.x * blockDim.x) {
+        const float4 ex = emb4[i], ey = emb4[n4 + i];
+        const float4 ax = attr4[i], ay = attr4[n4 + i];
+        const float4 rx = rep4[i], ry = rep4[n4 + i];
+        float4 gx = gains4[i], gy = gains4[n4 + i];
+        float4 ux = old4[i], uy = old4[n4 + i];
+        step_coordinate(gx.x, ux.x, ax.x, rx.x, exaggeration, normalization, momentum, eta);
+        step_coordinate(gx.y, ux.y, ax.y, rx.y, exaggeration, normalization, momentum, eta);
+        step_coordinate(gx.z, ux.z, ax.z, rx.z, exaggeration, normalization, momentum, eta);
+        step_coordinate(gx.w, ux.w, ax.w, rx.w, exaggeration, normalization, momentum, eta);
+        step_coordinate(gy.x, uy.x, ay.x, ry.x, exaggeration, normalization, momentum, eta);
+        step_coordinate(gy.y, uy.y, ay.y, ry.y, exaggeration, normalization, momentum, eta);
+        step_coordinate(gy.z, uy.z, ay.z, ry.z, exaggeration, normalization, momentum, eta);
+        step_coordinate(gy.w, uy.w, ay.w, ry.w, exaggeration, normalization, momentum, eta);
+        const float4 nx = make_float4(ex.x + ux.x, ex.y + ux.y, ex.z + ux.z, ex.w + ux.w);
+        const float4 ny = make_float4(ey.x + uy.x, ey.y + uy.y, ey.z + uy.z, ey.w + uy.w);
+        emb4[i] = nx;
+        emb4[n4 + i] = ny;
+        attr4[i] = zero;
+        attr4[n4 + i] = zero;
+        rep4[i] = zero;
+        rep4[n4 + i] = zero;
+        old4[i] = ux;
+        old4[n4 + i] = uy;
+        gains4[i] = gx;
+        gains4[n4 + i] = gy;
+        if (FUSED) {
+            float4 *y4 = reinterpret_cast<float4 *>(yxy) + 2 * (size_t)i;
+            y4[0] = make_float4(nx.x, ny.x, nx.y, ny.y);
+            y4[1] = make_float4(nx.z, ny.z, nx.w, ny.w);
+            lo = fminf(lo, fminf(fminf(fminf(nx.x, nx.y), fminf(nx.z, nx.w)), fminf(fminf(ny.x, ny.y), fminf(ny.z, ny.w))));
+            hi = fmaxf(hi, fmaxf(fmaxf(fmaxf(nx.x, nx.y), fmaxf(nx.z, nx.w)), fmaxf(fmaxf(ny.x, ny.y), fmaxf(ny.z, ny.w))));
+        }
+    }
+    if (FUSED) {
+        __shared__ float wlo[256 / kWave], whi[256 / kWave];
+        lo = group_min<kWave>(lo);
+        hi = group_max<kWave>(hi);
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            wlo[threadIdx.x / kWave] = lo;
+            whi[threadIdx.x / kWave] = hi;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int k = 1; k < 256 / kWave; ++k) {
+                lo = fminf(lo, wlo[k]);
+                hi = fmaxf(hi, whi[k]);
+            }
+            atomicMin(&sc->min_enc[next_slot], float_to_ordered(lo));
+            atomicMax(&sc->max_enc[next_slot], float_to_ordered(hi));
+        }
+    }
+}
+
 __global__ void clear_scalar_kernel(float *p) {
     if (threadIdx.x == 0 && blockIdx.x == 0) *p = 0.0f;
 }
@@ -111,8 +183,23 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
     const int N = p->num_points;
     const float *z_ptr = normalization ? normalization : &p->scalars->z_sum;
     const float z_offset = normalization ? 0.0f : (float)N;
-    const int blocks = std::min(div_up(N, 256), 2048);
     if (profile_mark(p, kKernelUpdate, s)) return 1;
+    auto aligned16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (N % 4 == 0 && aligned16(embedding) && aligned16(attr) && aligned16(rep) && aligned16(gains) &&
+        aligned16(old_forces)) {
+        const int blocks = std::min(div_up(N / 4, 256), 512);  // few workgroups: one pair of same-address atomics each
+        if (next_slot >= 0) {
+            update_vec4_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr,
+                                                            z_offset, momentum, exaggeration, p->yxy, p->scalars,
+                                                            next_slot);
+        } else {
+            update_vec4_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr,
+                                                             z_offset, momentum, exaggeration, nullptr, nullptr, 0);
+        }
+        TSNE_LAUNCHED(s);
+        return 0;
+    }
+    const int blocks = std::min(div_up(N, 256), 2048);
     if (next_slot >= 0) {
         update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_offset,
                                                    momentum, exaggeration, p->yxy, p->scalars, next_slot);
