@@ -152,6 +152,45 @@ __device__ __forceinline__ void compact_query(u64 *list, int cap, int want, int 
     __syncthreads();
 }
 
+// Wave-private versions for the matrix sweep, where a query's list, counter and threshold are only
+// ever touched by the wave that owns the query: one wave sorts in its own LDS buffer without any
+// workgroup barrier (LDS operations of a wave execute in order; the wavefront fence only stops the
+// compiler from reordering them), while the other waves keep issuing matrix instructions.
+__device__ __forceinline__ void wave_bitonic_sort(u64 *buf, int cap, int lane) {
+    for (int k = 2; k <= cap; k <<= 1) {
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int t = lane; t < cap / 2; t += kWave) {
+                const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+                const int hi = lo | j;
+                const bool up = (lo & k) == 0;
+                const u64 a = buf[lo], b = buf[hi];
+                if ((a > b) == up) {
+                    buf[lo] = b;
+                    buf[hi] = a;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        }
+    }
+}
+
+// list: this query's cap entries in global memory; leaves the sorted keys in buf.
+__device__ __forceinline__ int wave_compact(u64 *list, int cap, int want, int *cnt, u64 *thr, u64 *buf, int lane) {
+    __threadfence_block();  // this wave's appends to the list are complete
+    const int n = *cnt;
+    for (int e = lane; e < cap; e += kWave) buf[e] = e < n ? list[e] : ~0ull;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    wave_bitonic_sort(buf, cap, lane);
+    const int keep = min(n, want);
+    for (int e = lane; e < keep; e += kWave) list[e] = buf[e];
+    if (lane == 0) {
+        *cnt = keep;
+        if (n >= want) *thr = buf[want - 1];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    return n;
+}
+
 // ---------------------------------------------------------------------------
 // VALU sweep.  qlist == nullptr: queries are 0..N-1; otherwise the nq listed ones.
 // ---------------------------------------------------------------------------
@@ -262,7 +301,7 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
 // MFMA sweep.  KSTEPS = Daug / 2 k-steps of v_mfma_f32_32x32x2f32.
 // Dynamic LDS: two candidate tiles, copied verbatim from the packed points
 //   a[buf][cand block (4)][step group (S4)][lane (64)] float4   (4 steps per float4)
-// followed by the sort buffer (cap keys).
+// followed by one sort buffer (cap keys) per wave.
 // Output per query: the `want` best candidates by approximate distance
 // (cand, -1 padded) and tau = the approximate distance of the last one kept
 // (+inf when fewer than `want` candidates exist), both without the |q|^2 term.
@@ -277,7 +316,7 @@ __global__ __launch_bounds__(256) void knn_mfma_sweep_kernel(const float4 *__res
     constexpr int kLoadsPerThread = kTileFloat4 / 256;    // == S4
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     float4 *a_lds = reinterpret_cast<float4 *>(lds_raw);
-    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + 2 * kTileFloat4);
+    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + 2 * kTileFloat4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
     __shared__ u64 thr[kMQ];
     __shared__ int cnt[kMQ];
 
@@ -366,44 +405,55 @@ __global__ __launch_bounds__(256) void knn_mfma_sweep_kernel(const float4 *__res
                 float best = fminf(acc0[0], acc1[0]);
 #pragma unroll
                 for (int v = 1; v < 16; ++v) best = fminf(best, fminf(acc0[v], acc1[v]));
+                // A query meets about K' ln(N / K') passing candidates during the sweep and the 64 lanes
+                // serve different queries, so most block pairs have some lane that passes: the per-element
+                // test below is a single compare, and only elements with a passing lane run the key / append
+                // code (key < limit implies dist <= limit_d, so nothing is lost).
                 if (best <= limit_d) {
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
                             const float dist = half ? acc1[v] : acc0[v];
-                            const int j = c0 + (cb + half) * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
-                            const u64 key = pack_key(dist, j);
-                            if (key < limit && j < N && j != q && q < N) {
-                                const int slot = atomicAdd(&cnt[wave * 32 + qn], 1);
-                                list[(size_t)(wave * 32 + qn) * cap + slot] = key;
+                            if (dist <= limit_d) {
+                                const int j = c0 + (cb + half) * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
+                                const u64 key = pack_key(dist, j);
+                                if (key < limit && j < N && j != q && q < N) {
+                                    const int slot = atomicAdd(&cnt[wave * 32 + qn], 1);
+                                    list[(size_t)(wave * 32 + qn) * cap + slot] = key;
+                                }
                             }
                         }
                     }
                 }
             }
-            __syncthreads();  // all waves are done with tile `buf`; counters are final for this tile
-            const int crowded = (tid < kMQ) && (cnt[tid] > cap - kCT);
-            if (__syncthreads_or(crowded)) {
-                for (int ql = 0; ql < kMQ; ++ql)
-                    if (cnt[ql] > cap - kCT) compact_query(list, cap, want, cnt, thr, ql, sortbuf, tid);
+            // Lists that a further tile could overflow are compacted by their own wave, right away.
+            {
+                u64 crowded = __ballot(cnt[wave * 32 + qn] > cap - kCT) & 0xffffffffull;  // lanes l, l+32 share a query
+                while (crowded) {
+                    const int ql = wave * 32 + (__ffsll((long long)crowded) - 1);
+                    crowded &= crowded - 1;
+                    wave_compact(list + (size_t)ql * cap, cap, want, &cnt[ql], &thr[ql], sortbuf, lane);
+                }
             }
+            __syncthreads();  // all waves are done with tile `buf`
             if (more) {
                 stash(buf ^ 1);
                 __syncthreads();
                 buf ^= 1;
             }
         }
-        for (int ql = 0; ql < kMQ; ++ql) {
+        // Final ordering and output, every wave for its own 32 queries.
+        for (int b = 0; b < 32; ++b) {
+            const int ql = wave * 32 + b;
             const int qq = q0 + ql;
             if (qq >= N) break;
-            const int n = cnt[ql];
-            __syncthreads();
-            compact_query(list, cap, want, cnt, thr, ql, sortbuf, tid);
-            for (int e = tid; e < want; e += 256) cand[(size_t)qq * want + e] = e < n ? key_index(sortbuf[e]) : -1;
-            if (tid == 0) tau[qq] = n >= want ? key_distance(sortbuf[want - 1]) : INFINITY;
-            __syncthreads();
+            const int n = wave_compact(list + (size_t)ql * cap, cap, want, &cnt[ql], &thr[ql], sortbuf, lane);
+            for (int e = lane; e < want; e += kWave) cand[(size_t)qq * want + e] = e < n ? key_index(sortbuf[e]) : -1;
+            if (lane == 0) tau[qq] = n >= want ? key_distance(sortbuf[want - 1]) : INFINITY;
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         }
+        __syncthreads();  // before the next query tile re-initialises thr / cnt and the LDS tiles
     }
 }
 
@@ -514,7 +564,7 @@ template <int KSTEPS>
 int launch_mfma_sweep(const float4 *Xp, int N, int D, int Dnorm, int want, int cap, u64 *lists, int num_qtiles,
                       int grid, int *cand, float *tau, hipStream_t s) {
     constexpr int S4 = (KSTEPS + 3) / 4;
-    const size_t lds = sizeof(float4) * 2 * 4 * S4 * 64 + sizeof(u64) * cap;
+    const size_t lds = sizeof(float4) * 2 * 4 * S4 * 64 + sizeof(u64) * 4 * cap;  // two tiles + a sort buffer per wave
     TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_sweep_kernel<KSTEPS>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     knn_mfma_sweep_kernel<KSTEPS><<<grid, 256, lds, s>>>(Xp, N, D, Dnorm, want, cap, lists, num_qtiles, cand, tau);
@@ -603,7 +653,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
     const int want = std::min(N - 1, (K - 1) + std::max(32, (K - 1) / 2));  // K' candidates kept per query
     const int mcap = next_pow2(want + kCT) < 256 ? 256 : next_pow2(want + kCT);
-    const size_t mfma_lds = sizeof(float4) * 2 * 4 * ((ksteps + 3) / 4) * 64 + sizeof(u64) * mcap;
+    const size_t mfma_lds = sizeof(float4) * 2 * 4 * ((ksteps + 3) / 4) * 64 + sizeof(u64) * 4 * mcap;
     const bool mfma_fits = ksteps <= kMfmaMaxSteps && mcap <= 4096 && mfma_lds <= 150 * 1024;
     bool use_mfma = mode == 2 || (mode == 0 && mfma_fits && N >= 8192);
     if (mode == 2 && !mfma_fits) {
