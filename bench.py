@@ -127,6 +127,10 @@ def main():
                "sample": "%d gradient steps of the same %d x %d workload (P and neighbours from the GPU stages), "
                          "C++/OpenMP restatement" % (args.cpu_steps, n, k)}
 
+    # HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes whose
+    # summary sits in profiles/bench_c3_1M_hbm_counters.txt (386803 x 2 KiB fetched + 7826 x 1 KiB written);
+    # the counters belong to that exact workload, so other sizes report null.
+    traffic = 800.2e6 if (args.workload == "c3" and n == 1000000 and k == 90) else None
     out = {
         "metric": "gradient_iters_per_sec",
         "value": iters_per_s,
@@ -147,7 +151,7 @@ def main():
                      "reblock_pattern": reblock_s,
                      "gradient_loop_%d_steps" % args.steps: loop_s, "data_generation_host": gen_s},
         "roofline": {"bound": "hbm", "kernel": "attractive_blocked_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "bytes_per_launch": attr_bytes, "ms_per_launch": attr_ms},
         "kernels_us": kernels_us,
         "cpu_baseline": cpu,
