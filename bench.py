@@ -66,9 +66,16 @@ def main():
         return out, time.perf_counter() - a
 
     # ---- one-shot stages, inputs resident in HBM -------------------------
+    # As RunTsne does on entry, the points are renumbered in locality order first
+    # (the numbering is arbitrary; kNN and the attractive kernel run faster on it).
     dX = torch.from_numpy(X).cuda()
-    (idx, d2), knn_s = timed(lambda: stages.knn(dX, k))
+    order, order_s = timed(lambda: stages.locality_order(dX))
+    dXs, gather_s = timed(lambda: stages.gather_rows(dX, order))
     del dX
+    (idx, d2), knn_s = timed(lambda: stages.knn(dXs, k))
+    del dXs
+    order_h = order.cpu().numpy().astype(np.int64)
+    y0 = np.concatenate([y0[:n][order_h], y0[n:][order_h]])
     _, norm_s = timed(lambda: stages.max_normalize_(d2))
     cond, perp_s = timed(lambda: stages.perplexity(d2, fit["perplexity"], 1e-4))
     P, sym_s = timed(lambda: stages.symmetrize(cond, idx))
@@ -147,7 +154,7 @@ def main():
         "config": {"workload": "%s: %d x %d fp32, perplexity %g, K=%d, lr %g; step = one gradient iteration"
                                % (args.workload, n, d, fit["perplexity"], k, eta)},
         "fit_seconds": fit_s,
-        "phases_s": {"knn": knn_s, "max_normalize": norm_s, "perplexity": perp_s, "symmetrize": sym_s,
+        "phases_s": {"locality_order": order_s + gather_s, "knn": knn_s, "max_normalize": norm_s, "perplexity": perp_s, "symmetrize": sym_s,
                      "reblock_pattern": reblock_s,
                      "gradient_loop_%d_steps" % args.steps: loop_s, "data_generation_host": gen_s},
         "roofline": {"bound": "hbm", "kernel": "attractive_blocked_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,

@@ -54,6 +54,21 @@ int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neig
 int tsne_hip_knn_select(const float *points, int num_points, int num_dims, int num_neighbors, int *indices,
                         float *sq_dist, void *stream, int sweep, int *stats);
 
+/* Locality ordering of the points: order[new] = old (int32, device, num_points
+ * entries) such that points that are close in the input space get close numbers
+ * (nearest of up to 256 pivots taken from the data, pivots chained greedily;
+ * deterministic; the identity for fewer than 16384 points).  Nothing in t-SNE
+ * depends on the numbering of the points; RunTsne renumbers them this way on
+ * entry and restores the caller's numbering on exit because the attractive-force
+ * kernel and the neighbour search are faster on locally ordered points.  No
+ * counterpart in the reference, whose neighbour search gets its locality from the
+ * FAISS IVF lists (src/util/distance_utils.cu:101-127).  Synchronises the stream. */
+int tsne_hip_locality_order(const float *points, int num_points, int num_dims, int *order, void *stream);
+
+/* rows_out[r] = rows_in[order[r]] for num_rows rows of num_cols floats. */
+int tsne_hip_gather_rows(const float *rows_in, const int *order, int num_rows, int num_cols, float *rows_out,
+                         void *stream);
+
 /* In-place division of n values by their largest absolute value.
  * Replaces tsnecuda::util::MaxNormalizeDeviceVector (src/util/math_utils.cu:66-74). */
 int tsne_hip_max_normalize(float *values, int64_t n, void *stream);

@@ -90,3 +90,23 @@ def test_min_grad_norm_stops_early(c0_problem, capfd):
     out = capfd.readouterr().out
     assert "Reached minimum gradient norm" in out
     assert "_time_knn:" in out and "total_time:" in out
+
+
+def test_renumbering_is_invisible_to_the_caller(monkeypatch):
+    """RunTsne renumbers 16384 or more points in locality order on entry and
+    restores the caller's numbering on exit: a short fit gives the same
+    embedding, row for row, with the renumbering switched off."""
+    from tsnecuda import TSNE, synthetic
+    n = 20000
+    X = synthetic.gaussian_clusters(n, d=16, clusters=5, seed=11)
+    Y0 = synthetic.initial_embedding(n, seed=4)
+    kw = dict(perplexity=20.0, num_neighbors=60, n_iter=15, perplexity_epsilon=1e-4)
+    monkeypatch.setenv("TSNE_LOCALITY_ORDER", "1")
+    a = TSNE(**kw).fit_transform(X, y=Y0)
+    snaps = TSNE(return_style="snapshots", num_snapshots=3, **kw).fit_transform(X, y=Y0)
+    monkeypatch.setenv("TSNE_LOCALITY_ORDER", "0")
+    b = TSNE(**kw).fit_transform(X, y=Y0)
+    assert np.linalg.norm(a - b) <= 1e-3 * np.linalg.norm(b)
+    assert np.linalg.norm(snaps[-1] - b) <= 1e-3 * np.linalg.norm(b)
+    # the first snapshot is the embedding after one step: still close to the start, row for row
+    assert np.abs(snaps[0] - Y0).max() < 1e-2

@@ -308,6 +308,46 @@ def test_attractive_blocked_pattern(stages, n, k):
     plan.close()
 
 
+def test_attractive_blocked_clustered_pattern(stages):
+    """A pattern whose rows reference only a few column partitions (what the
+    locality ordering produces): runs longer than one work item share a staged
+    partition, other partitions are skipped."""
+    n, k = 40000, 60
+    rng = np.random.default_rng(5)
+    block = np.arange(n) // 10000  # four blocks of 10000 points
+    idx = (block[:, None] * 10000 + rng.integers(0, 10000, (n, k))).astype(np.int32)
+    idx[:, 0] = np.arange(n)
+    P = (rng.random((n, k)) * 1e-5).astype(np.float32)
+    P[:, 0] = 0.0
+    y = (rng.standard_normal(2 * n) * 8.0).astype(np.float32)
+    want = oracle.attractive(P, idx, y)
+    plan = stages.Plan(n, k)
+    plan.prepare_attractive(dev(P), dev(idx))
+    got = plan.attractive(None, None, dev(y)).cpu().numpy()
+    assert rel_l2(got, want) <= 1e-4
+    plan.close()
+
+
+def test_locality_order(stages):
+    """The renumbering is a permutation, deterministic, and groups clustered
+    points: along the new order the cluster label changes only a few times."""
+    from tsnecuda import synthetic
+    n = 40000
+    X = synthetic.gaussian_clusters(n, d=20, clusters=4, seed=3)
+    a = stages.locality_order(dev(X)).cpu().numpy()
+    b = stages.locality_order(dev(X)).cpu().numpy()
+    assert np.array_equal(a, b)
+    assert np.array_equal(np.sort(a), np.arange(n))
+    labels = (a % 4)  # gaussian_clusters: label = index mod clusters
+    changes = int((labels[1:] != labels[:-1]).sum())
+    assert changes <= 8, changes  # (pivot count) - 1 at the very most
+    Xs = stages.gather_rows(dev(X), dev(a.astype(np.int32))).cpu().numpy()
+    assert np.array_equal(Xs, X[a])
+    # small inputs keep their numbering
+    small = stages.locality_order(dev(X[:1000])).cpu().numpy()
+    assert np.array_equal(small, np.arange(1000))
+
+
 def test_iterate_with_prepared_pattern(stages, c0_problem):
     c = c0_problem
     n = c["X"].shape[0]

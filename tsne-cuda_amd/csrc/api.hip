@@ -111,6 +111,24 @@ int tsne_hip_knn_select(const float *points, int num_points, int num_dims, int n
                         stats);
 }
 
+int tsne_hip_locality_order(const float *points, int num_points, int num_dims, int *order, void *stream) {
+    TSNE_REQUIRE(points && order, "locality_order: null pointer argument");
+    TSNE_REQUIRE(num_points > 0 && num_dims > 0, "locality_order: num_points and num_dims must be positive");
+    hipStream_t s = (hipStream_t)stream;
+    std::vector<int> host;
+    if (locality_order(points, num_points, num_dims, host, s)) return 1;
+    TSNE_TRY(hipMemcpyAsync(order, host.data(), sizeof(int) * (size_t)num_points, hipMemcpyHostToDevice, s));
+    TSNE_TRY(hipStreamSynchronize(s));  // `host` goes out of scope
+    return 0;
+}
+
+int tsne_hip_gather_rows(const float *rows_in, const int *order, int num_rows, int num_cols, float *rows_out,
+                         void *stream) {
+    TSNE_REQUIRE(rows_in && order && rows_out, "gather_rows: null pointer argument");
+    TSNE_REQUIRE(num_rows > 0 && num_cols > 0, "gather_rows: num_rows and num_cols must be positive");
+    return launch_gather_rows(rows_in, order, num_rows, num_cols, rows_out, (hipStream_t)stream);
+}
+
 int tsne_hip_max_normalize(float *values, int64_t n, void *stream) {
     TSNE_REQUIRE(values && n > 0, "max_normalize: need a non-empty array");
     hipStream_t s = (hipStream_t)stream;

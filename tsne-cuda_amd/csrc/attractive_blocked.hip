@@ -41,7 +41,8 @@ constexpr double kRoundMagic = 6755399441055744.0;  // 1.5 * 2^52: adding it rou
 constexpr int kBlock = 1024;
 constexpr int kMaxParts = 1024;
 static_assert(kBlock == kMaxParts, "the partition scan uses one thread per slot");
-constexpr int kPrefetch = 4;        // entries per thread loaded ahead of the partition
+constexpr int kPrefetch = 4;        // entries per thread in one work item
+constexpr unsigned int kItemEntries = kPrefetch * kBlock;
 
 // ---------------------------------------------------------------------------
 // Re-blocking: one workgroup per strip.  Histogram of the strip's entries over
@@ -49,8 +50,9 @@ constexpr int kPrefetch = 4;        // entries per thread loaded ahead of the pa
 // partition with LDS atomics.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
-                                                         int N, int K, int strip_rows, int n_parts,
-                                                         float *__restrict__ ent_p, unsigned int *__restrict__ ent_c,
+                                                         int N, int K, int strip_rows, int max_items,
+                                                         int seg_stride, float *__restrict__ ent_p,
+                                                         unsigned int *__restrict__ ent_c,
                                                          unsigned int *__restrict__ seg, float *__restrict__ p_max) {
     __shared__ unsigned int cursor[kMaxParts];
     __shared__ unsigned int scan[kMaxParts];
@@ -75,16 +77,42 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
         __syncthreads();
     }
     const unsigned int first = scan[tid] - mine;
-    if (tid < n_parts) seg[(size_t)strip * (n_parts + 1) + tid] = first;
-    if (tid == n_parts - 1) seg[(size_t)strip * (n_parts + 1) + n_parts] = first + mine;
     cursor[tid] = first;
     __syncthreads();
+    // Work list of the strip: every referenced partition contributes ceil(entries / kItemEntries) items
+    // (runs of at most kItemEntries entries that share the partition); a second scan, over the item counts.
+    const unsigned int items = (mine + kItemEntries - 1u) / kItemEntries;
+    scan[tid] = items;
+    __syncthreads();
+    for (int off = 1; off < kMaxParts; off <<= 1) {
+        const unsigned int add = tid >= off ? scan[tid - off] : 0u;
+        __syncthreads();
+        scan[tid] += add;
+        __syncthreads();
+    }
+    unsigned int *hdr = seg + (size_t)strip * seg_stride;
+    unsigned int *item_begin = hdr + 1;
+    unsigned int *item_part = hdr + 2 + max_items;
+    for (unsigned int it = 0; it < items; ++it) {
+        const unsigned int slot = scan[tid] - items + it;
+        item_begin[slot] = first + it * kItemEntries;
+        item_part[slot] = (unsigned int)tid;
+    }
+    if (tid == kMaxParts - 1) {
+        hdr[0] = scan[tid];
+        item_begin[scan[tid]] = count;
+    }
+    // Entries are visited neighbour slot by neighbour slot, so that neighbouring positions of a
+    // partition's run belong to different rows: a wave of the force kernel then spreads its LDS
+    // atomics over many accumulators even when most neighbours of a row share one partition.
     float biggest = 0.0f;
-    for (unsigned int e = tid; e < count; e += kBlock) {
+    for (unsigned int v = tid; v < count; v += kBlock) {
+        const unsigned int slot = v / (unsigned int)nrows;
+        const unsigned int row_local = v - slot * (unsigned int)nrows;
+        const unsigned int e = row_local * (unsigned int)K + slot;
         const int col = idx[base + e];
         const int part = col / kPartPoints;
         const unsigned int pos = atomicAdd(&cursor[part], 1u);
-        const unsigned int row_local = e / (unsigned int)K;
         const float pv = pij[base + e];
         biggest = fmaxf(biggest, fabsf(pv));
         ent_p[base + pos] = pv;
@@ -121,7 +149,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
                                                                     const float2 *__restrict__ yxy,
                                                                     const float *__restrict__ p_max,
                                                                     float *__restrict__ attr, int N, int K,
-                                                                    int strip_rows, int n_parts) {
+                                                                    int strip_rows, int max_items, int seg_stride) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     float2 *part = reinterpret_cast<float2 *>(lds_raw);
     float2 *yi = part + kPartPoints;
@@ -132,7 +160,14 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
     const int row0 = strip * strip_rows;
     const int nrows = min(strip_rows, N - row0);
     const size_t base = (size_t)row0 * K;
-    const unsigned int *my_seg = seg + (size_t)strip * (n_parts + 1);
+    // The work list is read through the constant address space: it is never written while this
+    // kernel runs, and constant-space loads at uniform addresses are scalar loads, which do not
+    // queue behind the vector loads in flight.
+    typedef const __attribute__((address_space(4))) unsigned int *ConstWords;
+    ConstWords hdr = (ConstWords)(seg + (size_t)strip * seg_stride);
+    const int n_items = (int)hdr[0];
+    ConstWords my_seg = hdr + 1;               // n_items + 1 entry offsets
+    ConstWords my_part = hdr + 2 + max_items;  // partition of each item
     const float pm = *p_max;
     const double scale = pm > 0.0f ? 2251799813685248.0 / (double)pm : 1.0;  // 2^51 / p_max
 
@@ -156,21 +191,27 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         unsigned int pc[kPrefetch];
         float4 stage[kPartLoads];
         unsigned int b, e;
+        bool fresh;  // the item starts a new partition (uniform over the workgroup)
     };
     // All loads are unconditional (addresses clamped into range) so that none waits for another.
-    auto issue = [&](PhaseRegs &R, int p) {
-        R.b = my_seg[p];
-        R.e = my_seg[p + 1];
-        const unsigned int last = R.e > R.b ? R.e - 1u : R.b;  // an empty bucket re-reads its neighbour's entry, unused
+    const size_t last_entry = (size_t)nrows * K - 1;
+    auto issue = [&](PhaseRegs &R, int item) {
+        R.b = my_seg[item];
+        R.e = my_seg[item + 1];
+        const int p = (int)my_part[item];
+        R.fresh = item == 0 || p != (int)my_part[item - 1];
 #pragma unroll
         for (int k = 0; k < kPrefetch; ++k) {
-            const unsigned int t = min(R.b + tid + k * kBlock, last);
-            R.pv[k] = ent_p[base + min((size_t)t, (size_t)nrows * K - 1)];
-            R.pc[k] = ent_c[base + min((size_t)t, (size_t)nrows * K - 1)];
+            const size_t t = min((size_t)R.b + tid + k * kBlock, last_entry);
+            R.pv[k] = ent_p[base + t];
+            R.pc[k] = ent_c[base + t];
         }
+        // Every item issues the same number of loads, so the compiler's outstanding-load counts stay
+        // exact and no wait ever covers a younger prefetch.  An item that re-uses the staged partition
+        // points all lanes at one address instead: a single cache line per load, nothing to ingest.
 #pragma unroll
         for (int k = 0; k < kPartLoads; ++k)
-            R.stage[k] = yxy4[min(p * (kPartPoints / 2) + tid + k * kBlock, last_pair_all)];
+            R.stage[k] = yxy4[R.fresh ? min(p * (kPartPoints / 2) + tid + k * kBlock, last_pair_all) : 0];
     };
     auto consume = [&](PhaseRegs &R) {
 #pragma unroll
@@ -185,41 +226,31 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
                 add_force(acc, rl, w * dx, w * dy, scale);
             }
         }
-        // Buckets larger than kPrefetch * kBlock entries (skewed data): the rest.
-        for (unsigned int t = R.b + tid + kPrefetch * kBlock; t < R.e; t += kBlock) {
-            const float v = ent_p[base + t];
-            const unsigned int c = ent_c[base + t];
-            const unsigned int rl = c >> kColBits;
-            const float2 yj = part[c & ((1u << kColBits) - 1u)];
-            const float2 y0 = yi[rl];
-            const float dx = y0.x - yj.x, dy = y0.y - yj.y;
-            const float w = v * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
-            add_force(acc, rl, w * dx, w * dy, scale);
-        }
     };
     auto stage_to_lds = [&](PhaseRegs &R) {
-        __syncthreads();  // everyone is done reading the previous partition (first time: yi / acc are set)
+        if (!R.fresh) return;  // same partition as the previous item: it is already staged
+        __syncthreads();       // everyone is done reading the previous partition (first time: yi / acc are set)
 #pragma unroll
         for (int k = 0; k < kPartLoads; ++k) part4[tid + k * kBlock] = R.stage[k];
         __syncthreads();
     };
 
-    // Prefetch distance two: while phase p is consumed, the loads of phases
-    // p+1 and p+2 are in flight (a memory round trip is several phases long).
+    // Prefetch distance two: while item p is consumed, the loads of items
+    // p+1 and p+2 are in flight (a memory round trip is several items long).
     PhaseRegs R0, R1, R2;
-    issue(R0, 0);
-    if (1 < n_parts) issue(R1, 1);
-    for (int p = 0; p < n_parts; p += 3) {
+    if (0 < n_items) issue(R0, 0);
+    if (1 < n_items) issue(R1, 1);
+    for (int p = 0; p < n_items; p += 3) {
         stage_to_lds(R0);
-        if (p + 2 < n_parts) issue(R2, p + 2);
+        if (p + 2 < n_items) issue(R2, p + 2);
         consume(R0);
-        if (p + 1 >= n_parts) break;
+        if (p + 1 >= n_items) break;
         stage_to_lds(R1);
-        if (p + 3 < n_parts) issue(R0, p + 3);
+        if (p + 3 < n_items) issue(R0, p + 3);
         consume(R1);
-        if (p + 2 >= n_parts) break;
+        if (p + 2 >= n_items) break;
         stage_to_lds(R2);
-        if (p + 4 < n_parts) issue(R1, p + 4);
+        if (p + 4 < n_items) issue(R1, p + 4);
         consume(R2);
     }
     __syncthreads();
@@ -269,10 +300,13 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     p->strip_rows = strip_rows;
     p->n_strips = div_up(N, strip_rows);
     p->n_parts = n_parts;
+    // A strip's work list: one item per referenced partition plus one per further kItemEntries entries.
+    p->max_items = n_parts + (int)(((int64_t)strip_rows * K) / kItemEntries) + 1;
+    p->seg_stride = 2 * p->max_items + 4;
     const size_t nnz = (size_t)N * K;
     bool ok = hipMalloc(&p->ent_p, sizeof(float) * nnz) == hipSuccess &&
               hipMalloc(&p->ent_c, sizeof(unsigned int) * nnz) == hipSuccess &&
-              hipMalloc(&p->seg, sizeof(unsigned int) * (size_t)p->n_strips * (n_parts + 1)) == hipSuccess;
+              hipMalloc(&p->seg, sizeof(unsigned int) * (size_t)p->n_strips * p->seg_stride) == hipSuccess;
     if (!ok) {
         release_blocked(p);
         set_error("attractive_prepare: out of device memory for the re-blocked pattern (%zu bytes)", nnz * 8);
@@ -280,15 +314,12 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     }
     clear_pmax_kernel<<<1, 64, 0, s>>>(&p->scalars->vmax);
     TSNE_LAUNCHED(s);
-    reblock_kernel<<<p->n_strips, kBlock, 0, s>>>(pij, indices, N, K, strip_rows, n_parts, p->ent_p, p->ent_c, p->seg,
+    reblock_kernel<<<p->n_strips, kBlock, 0, s>>>(pij, indices, N, K, strip_rows, p->max_items, p->seg_stride, p->ent_p,
+                                                  p->ent_c, p->seg,
                                                   &p->scalars->vmax);
     TSNE_LAUNCHED(s);
-    static bool attr_set = false;
-    if (!attr_set) {
-        TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attractive_blocked_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBlockedLds));
-        attr_set = true;
-    }
+    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attractive_blocked_kernel),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBlockedLds));
     p->blocked_ready = true;
     return 0;
 }
@@ -302,7 +333,8 @@ int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s) {
     if (profile_mark(p, kKernelAttractive, s)) return 1;
     attractive_blocked_kernel<<<p->n_strips, kBlock, kBlockedLds, s>>>(p->ent_p, p->ent_c, p->seg, p->yxy,
                                                                        &p->scalars->vmax, attr, p->num_points,
-                                                                       p->num_neighbors, p->strip_rows, p->n_parts);
+                                                                       p->num_neighbors, p->strip_rows, p->max_items,
+                                                                       p->seg_stride);
     TSNE_LAUNCHED(s);
     return 0;
 }

@@ -53,6 +53,7 @@ struct DeviceBuffer {
         if (ptr) (void)hipFree(ptr);
         ptr = nullptr;
     }
+    void swap(DeviceBuffer &other) { std::swap(ptr, other.ptr); }
     template <typename T>
     T *as() const {
         return static_cast<T *>(ptr);
@@ -125,6 +126,45 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     DeviceBuffer d_points(sizeof(float) * (size_t)N * D);
     hip_or_die(hipMemcpy(d_points.ptr, opt.points, sizeof(float) * (size_t)N * D, hipMemcpyHostToDevice),
                "copy of the input points");
+    // Renumber the points so that neighbours in the input space get close
+    // numbers (the kNN sweep and the attractive kernel are faster that way);
+    // the caller's numbering is restored wherever an embedding leaves this
+    // function.  order[new] = old.  TSNE_LOCALITY_ORDER=0 keeps the numbering.
+    std::vector<int> order;
+    bool renumbered = false;
+    if (env_int("TSNE_LOCALITY_ORDER", 1) != 0 && tsnehip::locality_pivot_count(N) > 0) {
+        TSNE_OR_DIE(tsnehip::locality_order(d_points.as<float>(), N, D, order, stream), "locality ordering");
+        DeviceBuffer d_order(sizeof(int) * (size_t)N), d_sorted(sizeof(float) * (size_t)N * D);
+        hip_or_die(hipMemcpy(d_order.ptr, order.data(), sizeof(int) * (size_t)N, hipMemcpyHostToDevice),
+                   "copy of the point order");
+        TSNE_OR_DIE(tsnehip::launch_gather_rows(d_points.as<float>(), d_order.as<int>(), N, D, d_sorted.as<float>(),
+                                                stream),
+                    "point renumbering");
+        hip_or_die(hipStreamSynchronize(stream), "point renumbering");
+        d_points.swap(d_sorted);
+        renumbered = true;
+    }
+    // Embeddings cross this boundary as 2N floats, xs then ys, in the caller's numbering.
+    std::vector<float> h_swap;
+    auto to_internal = [&](std::vector<float> &emb) {
+        if (!renumbered) return;
+        h_swap.resize(emb.size());
+        for (int i = 0; i < N; ++i) {
+            h_swap[i] = emb[order[i]];
+            h_swap[(size_t)N + i] = emb[(size_t)N + order[i]];
+        }
+        emb.swap(h_swap);
+    };
+    auto to_caller = [&](const float *internal, float *out) {
+        if (!renumbered) {
+            if (out != internal) std::memcpy(out, internal, sizeof(float) * 2 * (size_t)N);
+            return;
+        }
+        for (int i = 0; i < N; ++i) {
+            out[order[i]] = internal[i];
+            out[(size_t)N + order[i]] = internal[(size_t)N + i];
+        }
+    };
     t_init = clock.stop();
 
     // ---- neighbours ------------------------------------------------------
@@ -185,6 +225,7 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     }
     DeviceBuffer d_emb(sizeof(float) * 2 * (size_t)N), d_gains(sizeof(float) * 2 * (size_t)N),
         d_old(sizeof(float) * 2 * (size_t)N), d_norm(sizeof(float));
+    to_internal(h_emb);
     hip_or_die(hipMemcpy(d_emb.ptr, h_emb.data(), sizeof(float) * h_emb.size(), hipMemcpyHostToDevice),
                "copy of the initial embedding");
     {
@@ -234,6 +275,7 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     if (verbose)
         for (auto &e : ev) hip_or_die(hipEventCreate(&e), "event creation");
 
+    std::vector<float> h_out;
     float normalization = -1.0f;
     int slot = 0;
     clock.start();
@@ -295,14 +337,15 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         if (want_dump && step % dump_interval == 0) {
             hip_or_die(hipMemcpy(h_emb.data(), d_emb.ptr, sizeof(float) * h_emb.size(), hipMemcpyDeviceToHost),
                        "dump");
-            for (int i = 0; i < N; ++i) dump_file << h_emb[i] << " " << h_emb[i + N] << std::endl;
+            h_out.resize(h_emb.size());
+            to_caller(h_emb.data(), h_out.data());
+            for (int i = 0; i < N; ++i) dump_file << h_out[i] << " " << h_out[i + N] << std::endl;
         }
         // At most num_snapshots - 1 in-loop snapshots, so that the final
         // embedding always fits as the last of num_snapshots blocks.
         if (want_snap && step % snap_interval == 0 && snap_num < opt.num_snapshots - 1) {
-            hip_or_die(hipMemcpy(opt.return_data + (size_t)snap_num * 2 * N, d_emb.ptr, sizeof(float) * 2 * N,
-                                 hipMemcpyDeviceToHost),
-                       "snapshot");
+            hip_or_die(hipMemcpy(h_emb.data(), d_emb.ptr, sizeof(float) * 2 * N, hipMemcpyDeviceToHost), "snapshot");
+            to_caller(h_emb.data(), opt.return_data + (size_t)snap_num * 2 * N);
             snap_num += 1;
         }
     }
@@ -336,7 +379,8 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     if (opt.return_data != nullptr) {
         float *dst = opt.return_data;
         if (opt.return_style == RETURN_STYLE::SNAPSHOT) dst += (size_t)snap_num * 2 * N;
-        hip_or_die(hipMemcpy(dst, d_emb.ptr, sizeof(float) * 2 * N, hipMemcpyDeviceToHost), "result copy");
+        hip_or_die(hipMemcpy(h_emb.data(), d_emb.ptr, sizeof(float) * 2 * N, hipMemcpyDeviceToHost), "result copy");
+        to_caller(h_emb.data(), dst);
     }
     tsne_hip_plan_destroy(plan);
     opt.trained = true;

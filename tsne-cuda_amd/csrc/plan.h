@@ -71,8 +71,8 @@ struct tsne_hip_plan {
     // Re-blocked copy of the sparse pattern for the LDS-staged attractive kernel.
     float *ent_p = nullptr;         // nnz probabilities, grouped by (row strip, column partition)
     unsigned int *ent_c = nullptr;  // nnz packed (column within partition | row within strip << 14)
-    unsigned int *seg = nullptr;    // n_strips x (n_parts + 1) bucket offsets inside a strip
-    int strip_rows = 0, n_strips = 0, n_parts = 0;
+    unsigned int *seg = nullptr;    // per strip seg_stride words: item count, item offsets, item partitions
+    int strip_rows = 0, n_strips = 0, n_parts = 0, max_items = 0, seg_stride = 0;
     bool blocked_ready = false;
 
     // Optional per-kernel timing: an event is recorded before every kernel of

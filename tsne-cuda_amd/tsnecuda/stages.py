@@ -26,6 +26,8 @@ def lib():
         L.tsne_hip_knn.argtypes = [_vp, c_int, c_int, c_int, _vp, _vp, _vp]
         L.tsne_hip_knn_select.argtypes = [_vp, c_int, c_int, c_int, _vp, _vp, _vp, c_int, ctypes.POINTER(c_int)]
         L.tsne_hip_knn_select.restype = c_int
+        L.tsne_hip_locality_order.argtypes = [_vp, c_int, c_int, _vp, _vp]
+        L.tsne_hip_gather_rows.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
         L.tsne_hip_max_normalize.argtypes = [_vp, c_i64, _vp]
         L.tsne_hip_perplexity.argtypes = [_vp, c_int, c_int, c_float, c_float, _vp, _vp, _vp]
         L.tsne_hip_symmetrize.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
@@ -46,7 +48,7 @@ def lib():
         L.tsne_hip_profile_end.argtypes = [_vp, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_int)]
         for name in ("profile_begin", "profile_end", "profile_kernel_count"):
             getattr(L, "tsne_hip_" + name).restype = c_int
-        for name in ("knn", "max_normalize", "perplexity", "symmetrize", "plan_create", "attractive",
+        for name in ("locality_order", "gather_rows", "knn", "max_normalize", "perplexity", "symmetrize", "plan_create", "attractive",
                      "repulsive", "update", "iterate", "sum_squares"):
             getattr(L, "tsne_hip_" + name).restype = c_int
         _lib = L
@@ -91,6 +93,24 @@ def knn_select(points, num_neighbors, sweep):
     _check(lib().tsne_hip_knn_select(_ptr(points), n, d, num_neighbors, _ptr(idx), _ptr(dist), _stream(), sweep,
                                      stats))
     return idx, dist, (int(stats[0]), int(stats[1]))
+
+
+def locality_order(points):
+    """order[new] = old (int32): the renumbering RunTsne applies on entry."""
+    points = _f32(points)
+    n, d = points.shape
+    order = torch.empty(n, dtype=torch.int32, device=points.device)
+    _check(lib().tsne_hip_locality_order(_ptr(points), n, d, _ptr(order), _stream()))
+    return order
+
+
+def gather_rows(rows, order):
+    rows = _f32(rows)
+    n, d = rows.shape
+    assert order.is_cuda and order.dtype == torch.int32 and order.numel() == n
+    out = torch.empty_like(rows)
+    _check(lib().tsne_hip_gather_rows(_ptr(rows), _ptr(order), n, d, _ptr(out), _stream()))
+    return out
 
 
 def max_normalize_(values):
