@@ -297,28 +297,92 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
     }
 }
 
+// Bounding ball of every tile of kCT consecutive points: the centre is the tile's mean, the
+// radius the largest distance of a member to it, inflated by 1e-3 (far more than the fp32
+// rounding of a sum over at most 128 dimensions) so that it is an upper bound.
+// centers_t is D x T (dimension-major).  One workgroup of 128 threads per tile; D <= 128.
+__global__ __launch_bounds__(128) void tile_balls_kernel(const float *__restrict__ X, int N, int D, int T,
+                                                         float *__restrict__ centers_t, float *__restrict__ radius) {
+    __shared__ float c[128];
+    __shared__ float wmax[2];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int first = t * kCT;
+    const int count = min(kCT, N - first);
+    for (int d = tid; d < D; d += 128) {
+        float sum = 0.0f;
+        for (int i = 0; i < count; ++i) sum += X[(size_t)(first + i) * D + d];
+        sum /= (float)count;
+        c[d] = sum;
+        centers_t[(size_t)d * T + t] = sum;
+    }
+    __syncthreads();
+    float d2 = 0.0f;
+    if (tid < count) {
+        const float *x = X + (size_t)(first + tid) * D;
+        for (int d = 0; d < D; ++d) {
+            const float diff = x[d] - c[d];
+            d2 = fmaf(diff, diff, d2);
+        }
+    }
+    d2 = group_max<kWave>(d2);
+    if ((tid & (kWave - 1)) == 0) wmax[tid / kWave] = d2;
+    __syncthreads();
+    if (tid == 0) radius[t] = sqrtf(fmaxf(wmax[0], wmax[1])) * (1.0f + 1e-3f) + 1e-30f;
+}
+
+constexpr int kHomeTiles = 8;  // candidate tiles on either side of the query tile that are always swept
+
+struct SweepArgs {
+    const float4 *Xp;
+    int N, D, Dnorm, want, cap;
+    u64 *lists;
+    int num_qtiles;
+    int *cand;
+    float *tau;
+    const float *norms;      // |x|^2 per point
+    const float *centers_t;  // D x T tile centres
+    const float *radius;     // T tile radii (upper bounds)
+    int bitmap_words;        // ceil(T / 32)
+};
+
 // ---------------------------------------------------------------------------
 // MFMA sweep.  KSTEPS = Daug / 2 k-steps of v_mfma_f32_32x32x2f32.
 // Dynamic LDS: two candidate tiles, copied verbatim from the packed points
 //   a[buf][cand block (4)][step group (S4)][lane (64)] float4   (4 steps per float4)
-// followed by one sort buffer (cap keys) per wave.
+// followed by one sort buffer (cap keys) per wave and the visit bitmap (one bit per tile).
+//
+// Tiles are visited in two phases.  First the query tile's own neighbourhood in the point
+// numbering (kHomeTiles tiles on either side), which gives every query a finite threshold.
+// Then only the tiles whose bounding ball can still hold a point below the largest of those
+// thresholds: with c, r the centre and radius of a tile's ball, every point x of tile t has
+// |q - x| >= |c_a - c_t| - r_a - r_t for every query q of tile a (triangle inequality), so the
+// tile is skipped when that bound, squared, exceeds max_q (threshold_q + |q|^2).  A threshold
+// only ever decreases and the final verification of a query compares with its final threshold,
+// so a skipped tile cannot hold one of its neighbours.  On numberings without locality the
+// balls are large and nothing is skipped.
 // Output per query: the `want` best candidates by approximate distance
 // (cand, -1 padded) and tau = the approximate distance of the last one kept
 // (+inf when fewer than `want` candidates exist), both without the |q|^2 term.
 // ---------------------------------------------------------------------------
 template <int KSTEPS>
-__global__ __launch_bounds__(256) void knn_mfma_sweep_kernel(const float4 *__restrict__ Xp, int N, int D, int Dnorm,
-                                                             int want, int cap, u64 *__restrict__ lists,
-                                                             int num_qtiles, int *__restrict__ cand,
-                                                             float *__restrict__ tau) {
+__global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_kernel(const SweepArgs args) {
+    const float4 *__restrict__ Xp = args.Xp;
+    const int N = args.N, D = args.D, Dnorm = args.Dnorm, want = args.want, cap = args.cap;
+    const int num_qtiles = args.num_qtiles;
+    u64 *__restrict__ lists = args.lists;
+    int *__restrict__ cand = args.cand;
+    float *__restrict__ tau = args.tau;
     constexpr int S4 = (KSTEPS + 3) / 4;
     constexpr int kTileFloat4 = 4 * S4 * 64;              // float4 per candidate tile
     constexpr int kLoadsPerThread = kTileFloat4 / 256;    // == S4
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     float4 *a_lds = reinterpret_cast<float4 *>(lds_raw);
     u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + 2 * kTileFloat4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
+    unsigned int *bitmap = reinterpret_cast<unsigned int *>(reinterpret_cast<u64 *>(a_lds + 2 * kTileFloat4) + 4 * (size_t)cap);
     __shared__ u64 thr[kMQ];
     __shared__ int cnt[kMQ];
+    __shared__ float qcenter[128];
+    __shared__ float tmax_part[2];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -364,15 +428,11 @@ __global__ __launch_bounds__(256) void knn_mfma_sweep_kernel(const float4 *__res
                 }
             }
         }
-        fetch(0);
-        __syncthreads();
-        stash(0);
-        __syncthreads();
         int buf = 0;
-        for (int ct = 0; ct < num_ctiles; ++ct) {
+        // One tile: compute it from LDS buffer `buf` while the next one travels through registers.
+        auto process = [&](int ct, int next_ct) {
             const int c0 = ct * kCT;
-            const bool more = ct + 1 < num_ctiles;
-            if (more) fetch(ct + 1);
+            if (next_ct >= 0) fetch(next_ct);
             const u64 limit = thr[wave * 32 + qn];
             // ~0 is "no threshold yet": its distance field does not decode to a number.
             const float limit_d = limit == ~0ull ? INFINITY : key_distance(limit);
@@ -437,11 +497,83 @@ __global__ __launch_bounds__(256) void knn_mfma_sweep_kernel(const float4 *__res
                 }
             }
             __syncthreads();  // all waves are done with tile `buf`
-            if (more) {
+            if (next_ct >= 0) {
                 stash(buf ^ 1);
                 __syncthreads();
                 buf ^= 1;
             }
+        };
+
+        // Phase 1: the query tile's neighbourhood; phase 2: the tiles the bitmap keeps.
+        const int T = num_ctiles;
+        const int h0 = max(qt - kHomeTiles, 0), h1 = min(qt + kHomeTiles, T - 1);
+        int word_idx = -1;
+        unsigned int cur_word = 0u;
+        // Next set bit of the bitmap, ascending; every wave walks the same words.
+        auto next_tile = [&]() -> int {
+            while (cur_word == 0u) {
+                ++word_idx;
+                if (word_idx >= args.bitmap_words) return -1;
+                cur_word = bitmap[word_idx];
+            }
+            const int b = __ffs((int)cur_word) - 1;
+            cur_word &= cur_word - 1u;
+            return word_idx * 32 + b;
+        };
+        fetch(h0);
+        __syncthreads();
+        stash(0);
+        __syncthreads();
+        bool home = true;
+        int cur = h0;
+        while (cur >= 0) {
+            int nxt = home ? (cur < h1 ? cur + 1 : -1) : next_tile();
+            process(cur, nxt);
+            if (nxt < 0 && home && (h0 > 0 || h1 < T - 1)) {
+                home = false;
+                // Thresholds from what the neighbourhood held.
+                for (int b = 0; b < 32; ++b) {
+                    const int ql = wave * 32 + b;
+                    if (q0 + ql < N)
+                        wave_compact(list + (size_t)ql * cap, cap, want, &cnt[ql], &thr[ql], sortbuf, lane);
+                }
+                for (int w = tid; w < args.bitmap_words; w += 256) bitmap[w] = 0u;
+                if (tid < D) qcenter[tid] = args.centers_t[(size_t)tid * T + qt];
+                __syncthreads();
+                if (tid < kMQ) {
+                    // Largest squared distance any query of the tile would still accept (rounded up).
+                    float v = -INFINITY;
+                    if (q0 + tid < N) {
+                        const u64 t = thr[tid];
+                        v = t == ~0ull ? INFINITY : key_distance(t) + args.norms[q0 + tid];
+                        v += 1e-5f * fabsf(v) + 1e-30f;
+                    }
+                    v = group_max<kWave>(v);
+                    if (lane == 0) tmax_part[wave] = v;
+                }
+                __syncthreads();
+                const float tmax = fmaxf(tmax_part[0], tmax_part[1]);
+                const float ra = args.radius[qt];
+                for (int t = tid; t < T; t += 256) {
+                    if (t >= h0 && t <= h1) continue;
+                    float d2 = 0.0f;
+                    for (int d = 0; d < D; ++d) {
+                        const float diff = qcenter[d] - args.centers_t[(size_t)d * T + t];
+                        d2 = fmaf(diff, diff, d2);
+                    }
+                    const float lb = sqrtf(d2) * (1.0f - 1e-3f) - (ra + args.radius[t]);
+                    const bool skip = lb > 0.0f && lb * lb > tmax;  // false for NaN: visit
+                    if (!skip) atomicOr(&bitmap[t >> 5], 1u << (t & 31));
+                }
+                __syncthreads();
+                nxt = next_tile();
+                if (nxt >= 0) {
+                    fetch(nxt);
+                    stash(buf);  // the barrier that ended the last tile freed both buffers
+                    __syncthreads();
+                }
+            }
+            cur = nxt;
         }
         // Final ordering and output, every wave for its own 32 queries.
         for (int b = 0; b < 32; ++b) {
@@ -561,23 +693,22 @@ int next_pow2(int v) {
 }
 
 template <int KSTEPS>
-int launch_mfma_sweep(const float4 *Xp, int N, int D, int Dnorm, int want, int cap, u64 *lists, int num_qtiles,
-                      int grid, int *cand, float *tau, hipStream_t s) {
+int launch_mfma_sweep(const SweepArgs &args, int grid, hipStream_t s) {
     constexpr int S4 = (KSTEPS + 3) / 4;
-    const size_t lds = sizeof(float4) * 2 * 4 * S4 * 64 + sizeof(u64) * 4 * cap;  // two tiles + a sort buffer per wave
+    // two tiles + a sort buffer per wave + the visit bitmap
+    const size_t lds = sizeof(float4) * 2 * 4 * S4 * 64 + sizeof(u64) * 4 * args.cap + sizeof(unsigned int) * args.bitmap_words;
     TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_sweep_kernel<KSTEPS>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    knn_mfma_sweep_kernel<KSTEPS><<<grid, 256, lds, s>>>(Xp, N, D, Dnorm, want, cap, lists, num_qtiles, cand, tau);
+    knn_mfma_sweep_kernel<KSTEPS><<<grid, 256, lds, s>>>(args);
     TSNE_TRY(hipGetLastError());
     return 0;
 }
 
 // Instantiated step counts: every count up to 32 (62 dimensions), then multiples of 4.
-int dispatch_mfma_sweep(int ksteps, const float4 *Xp, int N, int D, int Dnorm, int want, int cap, u64 *lists,
-                        int num_qtiles, int grid, int *cand, float *tau, hipStream_t s) {
+int dispatch_mfma_sweep(int ksteps, const SweepArgs &args, int grid, hipStream_t s) {
 #define TSNE_MFMA_CASE(KS) \
     case KS:               \
-        return launch_mfma_sweep<KS>(Xp, N, D, Dnorm, want, cap, lists, num_qtiles, grid, cand, tau, s);
+        return launch_mfma_sweep<KS>(args, grid, s);
     switch (ksteps) {
         TSNE_MFMA_CASE(2) TSNE_MFMA_CASE(3) TSNE_MFMA_CASE(4) TSNE_MFMA_CASE(5) TSNE_MFMA_CASE(6)
         TSNE_MFMA_CASE(7) TSNE_MFMA_CASE(8) TSNE_MFMA_CASE(9) TSNE_MFMA_CASE(10) TSNE_MFMA_CASE(11)
@@ -653,7 +784,10 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
     const int want = std::min(N - 1, (K - 1) + std::max(32, (K - 1) / 2));  // K' candidates kept per query
     const int mcap = next_pow2(want + kCT) < 256 ? 256 : next_pow2(want + kCT);
-    const size_t mfma_lds = sizeof(float4) * 2 * 4 * ((ksteps + 3) / 4) * 64 + sizeof(u64) * 4 * mcap;
+    const int num_tiles = div_up(N, kCT);
+    const int bitmap_words = div_up(num_tiles, 32);
+    const size_t mfma_lds = sizeof(float4) * 2 * 4 * ((ksteps + 3) / 4) * 64 + sizeof(u64) * 4 * mcap +
+                            sizeof(unsigned int) * bitmap_words;
     const bool mfma_fits = ksteps <= kMfmaMaxSteps && mcap <= 4096 && mfma_lds <= 150 * 1024;
     bool use_mfma = mode == 2 || (mode == 0 && mfma_fits && N >= 8192);
     if (mode == 2 && !mfma_fits) {
@@ -680,12 +814,13 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     }
 
     const int S4 = (ksteps + 3) / 4;
-    DeviceMem Xp, norms, lists, cand, tau, scal, fail_list;
+    DeviceMem Xp, norms, lists, cand, tau, scal, fail_list, centers, radius;
     const int num_qtiles = div_up(N, kMQ);
     const int grid = std::min(num_qtiles, cus * 2);
     if (!Xp.alloc(sizeof(float4) * (size_t)Npad * S4 * 2) || !norms.alloc(sizeof(float) * Npad) ||
         !lists.alloc(sizeof(u64) * (size_t)grid * kMQ * mcap) || !cand.alloc(sizeof(int) * (size_t)N * want) ||
-        !tau.alloc(sizeof(float) * N) || !scal.alloc(2 * sizeof(int)) || !fail_list.alloc(sizeof(int) * N)) {
+        !tau.alloc(sizeof(float) * N) || !scal.alloc(2 * sizeof(int)) || !fail_list.alloc(sizeof(int) * N) ||
+        !centers.alloc(sizeof(float) * (size_t)D * num_tiles) || !radius.alloc(sizeof(float) * num_tiles)) {
         set_error("knn: out of device memory for the candidate buffers");
         return 1;
     }
@@ -695,9 +830,24 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm, S4,
                                                                           Npad, Xp.as<float4>());
     TSNE_TRY(hipGetLastError());
-    if (dispatch_mfma_sweep(ksteps, Xp.as<float4>(), N, D, Dnorm, want, mcap, lists.as<u64>(), num_qtiles, grid,
-                            cand.as<int>(), tau.as<float>(), s))
-        return 1;
+    tile_balls_kernel<<<num_tiles, 128, 0, s>>>(points, N, D, num_tiles, centers.as<float>(), radius.as<float>());
+    TSNE_TRY(hipGetLastError());
+    SweepArgs args;
+    args.Xp = Xp.as<float4>();
+    args.N = N;
+    args.D = D;
+    args.Dnorm = Dnorm;
+    args.want = want;
+    args.cap = mcap;
+    args.lists = lists.as<u64>();
+    args.num_qtiles = num_qtiles;
+    args.cand = cand.as<int>();
+    args.tau = tau.as<float>();
+    args.norms = norms.as<float>();
+    args.centers_t = centers.as<float>();
+    args.radius = radius.as<float>();
+    args.bitmap_words = bitmap_words;
+    if (dispatch_mfma_sweep(ksteps, args, grid, s)) return 1;
     const int sort_n = next_pow2(want) < 64 ? 64 : next_pow2(want);
     knn_rerank_kernel<<<div_up(N, 4), 256, sizeof(u64) * 4 * sort_n, s>>>(
         points, norms.as<float>(), N, D, K, want, sort_n, cand.as<int>(), tau.as<float>(), scal.as<float>(), indices,
