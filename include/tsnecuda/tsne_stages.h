@@ -48,9 +48,12 @@ int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neig
  * shape (what tsne_hip_knn does), 1 = vector-ALU sweep, 2 = matrix-instruction
  * (MFMA) candidate sweep followed by an exact re-rank and verification (at most
  * 126 dimensions).  Results are identical whichever sweep runs.  stats (host
- * pointer to two ints, may be NULL): [0] = 1 if the matrix sweep ran,
- * [1] = queries the verification sent back to the vector sweep.  Same
- * reference counterpart as tsne_hip_knn. */
+ * pointer to three ints, may be NULL): [0] = 1 if the matrix sweep ran,
+ * [1] = queries the verification sent back to the vector sweep, [2] = per
+ * mille of the (query tile, candidate tile) pairs the matrix sweep computed (it
+ * skips candidate tiles whose bounding ball lies beyond every threshold of the
+ * query tile, which pays on locality-ordered points).  Same reference
+ * counterpart as tsne_hip_knn. */
 int tsne_hip_knn_select(const float *points, int num_points, int num_dims, int num_neighbors, int *indices,
                         float *sq_dist, void *stream, int sweep, int *stats);
 

@@ -386,6 +386,28 @@ def test_knn_matrix_sweep_is_exact(stages, n, d, k):
     assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
 
 
+@pytest.mark.parametrize("scale,d", [(30.0, 12), (2.5, 6), (0.7, 4)])
+def test_knn_matrix_sweep_tile_skipping_is_exact(stages, scale, d):
+    """On locality-ordered points the matrix sweep skips candidate tiles by their
+    bounding balls.  Well separated clusters (most tiles skipped), touching
+    clusters (the bound decides tile by tile) and one blob (nothing to skip) all
+    give the vector sweep's result bit for bit; rows are also checked against
+    the oracle."""
+    from tsnecuda import synthetic
+    n, k = 60000, 40
+    X = synthetic.gaussian_clusters(n, d=d, clusters=7, center_scale=scale, seed=int(scale * 10) + d)
+    dX = dev(X)
+    Xs = stages.gather_rows(dX, stages.locality_order(dX))
+    idx, d2, stats = stages.knn_select(Xs, k, 2)
+    assert stats[0] == 1
+    idx_v, d2_v, _ = stages.knn_select(Xs, k, 1)
+    assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
+    rows = (n // 3, n // 3 + 96)
+    idx_o, d2_o = oracle.knn(Xs.cpu().numpy(), k, rows=rows)
+    assert np.array_equal(idx[rows[0]:rows[1]].cpu().numpy(), idx_o)
+    assert np.array_equal(d2[rows[0]:rows[1]].cpu().numpy(), d2_o)
+
+
 def test_knn_matrix_sweep_verification_falls_back(stages):
     """Points far from the origin with tiny mutual distances: the approximate
     |c|^2 - 2 q.c distances cannot separate them, the verification must notice

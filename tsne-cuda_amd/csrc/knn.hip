@@ -33,6 +33,7 @@
 #include <algorithm>
 #include <climits>
 #include <cmath>
+#include <cstring>
 #include <vector>
 
 namespace tsnehip {
@@ -49,6 +50,13 @@ constexpr int kDC = 32;   // VALU sweep: dimensions staged per chunk
 constexpr int kMQ = 128;  // MFMA sweep: queries per workgroup (4 waves x 32)
 constexpr int kMfmaMaxSteps = 64;  // k-steps of 2 dimensions: up to 126 dimensions + 2 augmented
 static_assert(kMQ == kCT, "query tiles and candidate tiles share the packed layout");
+
+// v_min3_f32 without the quieting moves the library fminf adds for signalling NaNs.
+__device__ __forceinline__ float min3(float a, float b, float c) {
+    float r;
+    asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 
 __device__ __forceinline__ u64 pack_key(float d, int j) {
     return ((u64)float_to_ordered(d) << 32) | (unsigned int)j;
@@ -343,6 +351,7 @@ struct SweepArgs {
     const float *centers_t;  // D x T tile centres
     const float *radius;     // T tile radii (upper bounds)
     int bitmap_words;        // ceil(T / 32)
+    unsigned long long *tiles_swept;  // statistics: (query tile, candidate tile) pairs computed
 };
 
 // ---------------------------------------------------------------------------
@@ -462,27 +471,46 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
                     }
                 }
                 // Register v of lane l holds candidate row 8*(v/4) + 4*(l/32) + v%4 of the block, query column l%32.
-                float best = fminf(acc0[0], acc1[0]);
+                // Smallest of the lane's 32 values, three operands per instruction (the accumulators are
+                // never signalling NaNs, so the library fminf's quieting moves are left out).
+                float best = min3(acc0[0], acc0[1], acc0[2]);
 #pragma unroll
-                for (int v = 1; v < 16; ++v) best = fminf(best, fminf(acc0[v], acc1[v]));
+                for (int v = 3; v + 1 < 16; v += 2) best = min3(best, acc0[v], acc0[v + 1]);
+                best = min3(best, acc0[15], acc1[0]);
+#pragma unroll
+                for (int v = 1; v + 1 < 16; v += 2) best = min3(best, acc1[v], acc1[v + 1]);
+                best = fminf(best, acc1[15]);
                 // A query meets about K' ln(N / K') passing candidates during the sweep and the 64 lanes
-                // serve different queries, so most block pairs have some lane that passes: the per-element
-                // test below is a single compare, and only elements with a passing lane run the key / append
-                // code (key < limit implies dist <= limit_d, so nothing is lost).
+                // serve different queries, so most block pairs have some lane that passes.  A lane first
+                // counts its passing elements (compare + add-with-carry each), reserves that many list
+                // slots with one LDS atomic and then stores the keys: no atomic round trip per element.
+                // The test is on the distance alone; an element that ties with the threshold's distance
+                // but not its index is appended too and sorted out by the next compaction.
                 if (best <= limit_d) {
+                    const int jbase = c0 + cb * 32 + 4 * kh;  // element (half, v) is candidate jbase + 32 half + 8 (v / 4) + v % 4
+                    // Only the last tile has candidates beyond N and only the query's own tile holds the
+                    // query: those two tiles knock the excluded elements out by raising them to +inf.
+                    if (c0 + kCT > N || (unsigned int)(q0 - c0) < (unsigned int)kCT) {
 #pragma unroll
-                    for (int half = 0; half < 2; ++half) {
+                        for (int e = 0; e < 16; ++e) {
+                            const int j = jbase + 8 * (e >> 2) + (e & 3);
+                            if (j >= N || j == q) acc0[e] = INFINITY;
+                            if (j + 32 >= N || j + 32 == q) acc1[e] = INFINITY;
+                        }
+                    }
+                    const float lim = q < N ? limit_d : -INFINITY;
+                    int n = 0;
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const float dist = half ? acc1[v] : acc0[v];
-                            if (dist <= limit_d) {
-                                const int j = c0 + (cb + half) * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
-                                const u64 key = pack_key(dist, j);
-                                if (key < limit && j < N && j != q && q < N) {
-                                    const int slot = atomicAdd(&cnt[wave * 32 + qn], 1);
-                                    list[(size_t)(wave * 32 + qn) * cap + slot] = key;
-                                }
-                            }
+                    for (int e = 0; e < 32; ++e) n += ((e < 16 ? acc0[e & 15] : acc1[e & 15]) <= lim) ? 1 : 0;
+                    if (n != 0) {
+                        const int slot = atomicAdd(&cnt[wave * 32 + qn], n);
+                        u64 *dst = list + (size_t)(wave * 32 + qn) * cap + slot;
+                        float lim2 = lim;
+                        asm volatile("" : "+v"(lim2));  // compare again rather than keep 32 lane masks alive
+#pragma unroll
+                        for (int e = 0; e < 32; ++e) {
+                            const float dist = e < 16 ? acc0[e & 15] : acc1[e & 15];
+                            if (dist <= lim2) *dst++ = pack_key(dist, jbase + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
                         }
                     }
                 }
@@ -526,7 +554,9 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
         __syncthreads();
         bool home = true;
         int cur = h0;
+        unsigned int swept = 0;
         while (cur >= 0) {
+            ++swept;
             int nxt = home ? (cur < h1 ? cur + 1 : -1) : next_tile();
             process(cur, nxt);
             if (nxt < 0 && home && (h0 > 0 || h1 < T - 1)) {
@@ -575,6 +605,7 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
             }
             cur = nxt;
         }
+        if (tid == 0) atomicAdd(args.tiles_swept, (unsigned long long)swept);
         // Final ordering and output, every wave for its own 32 queries.
         for (int b = 0; b < 32; ++b) {
             const int ql = wave * 32 + b;
@@ -752,10 +783,11 @@ int run_valu_sweep(const float *Xt, int N, int Npad, int D, int K, const int *ql
 }  // namespace
 
 // mode: 0 = choose, 1 = VALU sweep only, 2 = matrix-instruction sweep (error if the shape does not fit).
-// stats (optional, 2 ints): [0] = 1 if the matrix-instruction sweep ran, [1] = queries redone by the VALU sweep.
+// stats (optional, 3 ints): [0] = 1 if the matrix-instruction sweep ran, [1] = queries redone by the VALU sweep,
+// [2] = per mille of the (query tile, candidate tile) pairs the matrix sweep computed.
 int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s, int mode,
                  int *stats) {
-    if (stats) stats[0] = stats[1] = 0;
+    if (stats) stats[0] = stats[1] = stats[2] = 0;
     if (N <= 0 || D <= 0 || K <= 0) {
         set_error("knn: num_points, num_dims and num_neighbors must be positive (got %d, %d, %d)", N, D, K);
         return 1;
@@ -819,12 +851,12 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     const int grid = std::min(num_qtiles, cus * 2);
     if (!Xp.alloc(sizeof(float4) * (size_t)Npad * S4 * 2) || !norms.alloc(sizeof(float) * Npad) ||
         !lists.alloc(sizeof(u64) * (size_t)grid * kMQ * mcap) || !cand.alloc(sizeof(int) * (size_t)N * want) ||
-        !tau.alloc(sizeof(float) * N) || !scal.alloc(2 * sizeof(int)) || !fail_list.alloc(sizeof(int) * N) ||
+        !tau.alloc(sizeof(float) * N) || !scal.alloc(4 * sizeof(int)) || !fail_list.alloc(sizeof(int) * N) ||
         !centers.alloc(sizeof(float) * (size_t)D * num_tiles) || !radius.alloc(sizeof(float) * num_tiles)) {
         set_error("knn: out of device memory for the candidate buffers");
         return 1;
     }
-    TSNE_TRY(hipMemsetAsync(scal.p, 0, 2 * sizeof(int), s));  // [0] max |x|^2 (float bits), [1] fail count
+    TSNE_TRY(hipMemsetAsync(scal.p, 0, 4 * sizeof(int), s));  // [0] max |x|^2 (float bits), [1] fail count, [2..3] tiles swept (64-bit)
     norms_kernel<<<div_up(Npad, 256), 256, 0, s>>>(points, N, D, Npad, norms.as<float>(), scal.as<float>());
     TSNE_TRY(hipGetLastError());
     pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm, S4,
@@ -847,19 +879,23 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     args.centers_t = centers.as<float>();
     args.radius = radius.as<float>();
     args.bitmap_words = bitmap_words;
+    args.tiles_swept = reinterpret_cast<unsigned long long *>(scal.as<int>() + 2);
     if (dispatch_mfma_sweep(ksteps, args, grid, s)) return 1;
     const int sort_n = next_pow2(want) < 64 ? 64 : next_pow2(want);
     knn_rerank_kernel<<<div_up(N, 4), 256, sizeof(u64) * 4 * sort_n, s>>>(
         points, norms.as<float>(), N, D, K, want, sort_n, cand.as<int>(), tau.as<float>(), scal.as<float>(), indices,
         sq_dist, scal.as<int>() + 1, fail_list.as<int>());
     TSNE_TRY(hipGetLastError());
-    int host_scal[2] = {0, 0};
+    int host_scal[4] = {0, 0, 0, 0};
     TSNE_TRY(hipMemcpyAsync(host_scal, scal.p, sizeof(host_scal), hipMemcpyDeviceToHost, s));
     TSNE_TRY(hipStreamSynchronize(s));
     const int failed = host_scal[1];
     if (stats) {
         stats[0] = 1;
         stats[1] = failed;
+        unsigned long long swept = 0;
+        std::memcpy(&swept, host_scal + 2, sizeof(swept));
+        stats[2] = (int)((1000.0 * (double)swept) / ((double)num_tiles * (double)num_tiles) + 0.5);
     }
     if (failed > 0) {
         if (build_transposed()) return 1;

@@ -84,15 +84,16 @@ def knn(points, num_neighbors):
 
 def knn_select(points, num_neighbors, sweep):
     """knn() with an explicit sweep (1 = vector ALU, 2 = matrix instructions).
-    Returns (indices, sq_dist, stats) with stats = (matrix sweep ran, queries redone)."""
+    Returns (indices, sq_dist, stats) with stats = (matrix sweep ran, queries redone,
+    per mille of tile pairs computed)."""
     points = _f32(points)
     n, d = points.shape
     idx = torch.empty((n, num_neighbors), dtype=torch.int32, device=points.device)
     dist = torch.empty((n, num_neighbors), dtype=torch.float32, device=points.device)
-    stats = (ctypes.c_int * 2)()
+    stats = (ctypes.c_int * 3)()
     _check(lib().tsne_hip_knn_select(_ptr(points), n, d, num_neighbors, _ptr(idx), _ptr(dist), _stream(), sweep,
                                      stats))
-    return idx, dist, (int(stats[0]), int(stats[1]))
+    return idx, dist, (int(stats[0]), int(stats[1]), int(stats[2]))
 
 
 def locality_order(points):
