@@ -160,43 +160,92 @@ __device__ __forceinline__ void compact_query(u64 *list, int cap, int want, int 
     __syncthreads();
 }
 
-// Wave-private versions for the matrix sweep, where a query's list, counter and threshold are only
-// ever touched by the wave that owns the query: one wave sorts in its own LDS buffer without any
-// workgroup barrier (LDS operations of a wave execute in order; the wavefront fence only stops the
-// compiler from reordering them), while the other waves keep issuing matrix instructions.
-__device__ __forceinline__ void wave_bitonic_sort(u64 *buf, int cap, int lane) {
-    for (int k = 2; k <= cap; k <<= 1) {
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int t = lane; t < cap / 2; t += kWave) {
-                const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1));
-                const int hi = lo | j;
-                const bool up = (lo & k) == 0;
-                const u64 a = buf[lo], b = buf[hi];
-                if ((a > b) == up) {
-                    buf[lo] = b;
-                    buf[hi] = a;
-                }
-            }
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        }
+// Wave-private selection for the matrix sweep, where a query's list, counter and threshold are
+// only ever touched by the wave that owns the query.  The sweep never needs its candidates in
+// order, only the `want` smallest of them and the distance of the last one kept, so a compaction
+// is a radix select on the distance bits, six bits per pass: lane l owns histogram bin l, a wave
+// scan finds the bin that holds the want-th smallest.  The bits are taken relative to the smallest
+// distance present, which skips the leading bits all keys share.  No workgroup barrier is involved
+// (LDS operations of a wave execute in order; the wavefront fences only stop the compiler from
+// reordering them), so the other waves keep issuing matrix instructions meanwhile.
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const int o = __shfl_up(v, off, kWave);
+        if (lane >= off) v += o;
     }
+    return v;
 }
 
-// list: this query's cap entries in global memory; leaves the sorted keys in buf.
-__device__ __forceinline__ int wave_compact(u64 *list, int cap, int want, int *cnt, u64 *thr, u64 *buf, int lane) {
+// list: this query's entries in global memory (n = *cnt of them); buf: cap keys of LDS; hist: 64 words
+// of LDS.  Afterwards list[0, min(n, want)) holds the entries kept (in no particular order), *cnt their
+// number, and *thr is lowered to (distance of the want-th smallest, all index bits set) when n >= want.
+// Returns the number of entries kept.
+__device__ __forceinline__ int wave_select(u64 *list, int want, int *cnt, u64 *thr, u64 *buf, unsigned int *hist,
+                                           int lane) {
     __threadfence_block();  // this wave's appends to the list are complete
     const int n = *cnt;
-    for (int e = lane; e < cap; e += kWave) buf[e] = e < n ? list[e] : ~0ull;
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    wave_bitonic_sort(buf, cap, lane);
-    const int keep = min(n, want);
-    for (int e = lane; e < keep; e += kWave) list[e] = buf[e];
-    if (lane == 0) {
-        *cnt = keep;
-        if (n >= want) *thr = buf[want - 1];
+    if (n < want) return n;
+    unsigned int lo = ~0u, hi = 0u;
+    for (int e = lane; e < n; e += kWave) {
+        const u64 key = list[e];
+        buf[e] = key;
+        const unsigned int bits = (unsigned int)(key >> 32);
+        lo = min(lo, bits);
+        hi = max(hi, bits);
+    }
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) {
+        lo = min(lo, (unsigned int)__shfl_xor((int)lo, m, kWave));
+        hi = max(hi, (unsigned int)__shfl_xor((int)hi, m, kWave));
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    return n;
+    // Radix select of the want-th smallest value of (bits - lo).
+    unsigned int prefix = 0u;
+    int rank = want;  // 1-based rank among the keys that match the prefix
+    int shift = 32 - __clz((int)(hi - lo));  // significant bits of the range (0 when all distances are equal)
+    if (hi == lo) shift = 0;
+    while (shift > 0) {
+        const int w = shift < 6 ? shift : 6;
+        shift -= w;
+        hist[lane] = 0u;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        for (int e = lane; e < n; e += kWave) {
+            const unsigned int v = (unsigned int)(buf[e] >> 32) - lo;
+            if ((unsigned int)((u64)v >> (shift + w)) == prefix) atomicAdd(&hist[(v >> shift) & ((1u << w) - 1u)], 1u);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        const int c = (int)hist[lane];
+        const int incl = wave_inclusive_scan(c, lane);
+        const int b = __ffsll((long long)__ballot(incl >= rank)) - 1;  // some lane qualifies: the last one holds all matches
+        rank -= __shfl(incl - c, b, kWave);
+        prefix = (prefix << w) | (unsigned int)b;
+    }
+    const unsigned int dstar = lo + prefix;
+    // Keep everything below dstar and the first `rank` entries equal to it.
+    const int need_eq = rank, c_lt = want - rank;
+    int base_lt = 0, base_eq = 0;
+    const u64 below = (1ull << lane) - 1ull;
+    for (int e0 = 0; e0 < n; e0 += kWave) {
+        const int e = e0 + lane;
+        const u64 key = e < n ? buf[e] : 0ull;
+        const unsigned int bits = (unsigned int)(key >> 32);
+        const bool lt = e < n && bits < dstar, eq = e < n && bits == dstar;
+        const u64 m_lt = __ballot(lt), m_eq = __ballot(eq);
+        if (lt) list[base_lt + __popcll(m_lt & below)] = key;
+        if (eq) {
+            const int k = base_eq + __popcll(m_eq & below);
+            if (k < need_eq) list[c_lt + k] = key;
+        }
+        base_lt += __popcll(m_lt);
+        base_eq += __popcll(m_eq);
+    }
+    if (lane == 0) {
+        *cnt = want;
+        *thr = ((u64)dstar << 32) | 0xffffffffull;
+    }
+    __threadfence_block();
+    return want;
 }
 
 // ---------------------------------------------------------------------------
@@ -351,6 +400,7 @@ struct SweepArgs {
     const float *centers_t;  // D x T tile centres
     const float *radius;     // T tile radii (upper bounds)
     int bitmap_words;        // ceil(T / 32)
+    int trigger;             // a list longer than this is compacted after the tile (<= cap - kCT)
     unsigned long long *tiles_swept;  // statistics: (query tile, candidate tile) pairs computed
 };
 
@@ -391,6 +441,7 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
     __shared__ u64 thr[kMQ];
     __shared__ int cnt[kMQ];
     __shared__ float qcenter[128];
+    __shared__ unsigned int hist_all[4][kWave];
     __shared__ float tmax_part[2];
 
     const int tid = threadIdx.x;
@@ -517,11 +568,11 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
             }
             // Lists that a further tile could overflow are compacted by their own wave, right away.
             {
-                u64 crowded = __ballot(cnt[wave * 32 + qn] > cap - kCT) & 0xffffffffull;  // lanes l, l+32 share a query
+                u64 crowded = __ballot(cnt[wave * 32 + qn] > args.trigger) & 0xffffffffull;  // lanes l, l+32 share a query
                 while (crowded) {
                     const int ql = wave * 32 + (__ffsll((long long)crowded) - 1);
                     crowded &= crowded - 1;
-                    wave_compact(list + (size_t)ql * cap, cap, want, &cnt[ql], &thr[ql], sortbuf, lane);
+                    wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
                 }
             }
             __syncthreads();  // all waves are done with tile `buf`
@@ -565,7 +616,7 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
                 for (int b = 0; b < 32; ++b) {
                     const int ql = wave * 32 + b;
                     if (q0 + ql < N)
-                        wave_compact(list + (size_t)ql * cap, cap, want, &cnt[ql], &thr[ql], sortbuf, lane);
+                        wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
                 }
                 for (int w = tid; w < args.bitmap_words; w += 256) bitmap[w] = 0u;
                 if (tid < D) qcenter[tid] = args.centers_t[(size_t)tid * T + qt];
@@ -611,9 +662,12 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
             const int ql = wave * 32 + b;
             const int qq = q0 + ql;
             if (qq >= N) break;
-            const int n = wave_compact(list + (size_t)ql * cap, cap, want, &cnt[ql], &thr[ql], sortbuf, lane);
-            for (int e = lane; e < want; e += kWave) cand[(size_t)qq * want + e] = e < n ? key_index(sortbuf[e]) : -1;
-            if (lane == 0) tau[qq] = n >= want ? key_distance(sortbuf[want - 1]) : INFINITY;
+            const int n = wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
+            for (int e = lane; e < want; e += kWave)
+                cand[(size_t)qq * want + e] = e < n ? key_index(list[(size_t)ql * cap + e]) : -1;
+            // Every candidate that was dropped, by a compaction or by the filter, had a distance >= the
+            // threshold of the moment, and thresholds only decrease.
+            if (lane == 0) tau[qq] = thr[ql] == ~0ull ? INFINITY : key_distance(thr[ql]);
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         }
         __syncthreads();  // before the next query tile re-initialises thr / cnt and the LDS tiles
@@ -879,6 +933,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     args.centers_t = centers.as<float>();
     args.radius = radius.as<float>();
     args.bitmap_words = bitmap_words;
+    args.trigger = mcap - kCT;  // as late as possible: a later selection costs the same and sees more candidates
     args.tiles_swept = reinterpret_cast<unsigned long long *>(scal.as<int>() + 2);
     if (dispatch_mfma_sweep(ksteps, args, grid, s)) return 1;
     const int sort_n = next_pow2(want) < 64 ? 64 : next_pow2(want);
