@@ -135,9 +135,9 @@ def main():
                          "C++/OpenMP restatement" % (args.cpu_steps, n, k)}
 
     # HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes whose
-    # summary sits in profiles/bench_c3_1M_hbm_counters.txt (386803 x 2 KiB fetched + 7826 x 1 KiB written);
+    # summary sits in profiles/bench_c3_1M_hbm_counters.txt (424126 x 2 KiB fetched + 7826 x 1 KiB written);
     # the counters belong to that exact workload, so other sizes report null.
-    traffic = 800.2e6 if (args.workload == "c3" and n == 1000000 and k == 90) else None
+    traffic = 876.6e6 if (args.workload == "c3" and n == 1000000 and k == 90) else None
     out = {
         "metric": "gradient_iters_per_sec",
         "value": iters_per_s,
