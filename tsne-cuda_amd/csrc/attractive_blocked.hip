@@ -9,15 +9,16 @@
 //   * rows are cut into strips (one workgroup each, <= 4096 rows),
 //   * columns into partitions of kPartPoints points,
 //   * inside a strip the entries are grouped by partition; an entry is 8 bytes:
-//     the probability and a packed (column within partition | row within strip).
+//     the probability and a packed (column within partition | row within strip),
+//   * a strip's work list names, in order, runs ("items") of at most
+//     kItemEntries entries that share a partition; partitions the strip never
+//     references do not appear in it.
 //
 // A workgroup keeps its strip's positions and force accumulators in LDS and
-// walks the partitions in order; for each one it stages that partition's
-// positions in LDS, so every neighbour gather is an LDS read and every
-// accumulation an LDS atomic.  HBM sees the 8 bytes per entry once, coalesced,
-// plus the positions once per workgroup (served by the L2, since all
-// workgroups walk the partitions in step).  The next partition and its entries
-// are prefetched into registers while the current one is being consumed.
+// walks its work list; the partition an item refers to is staged in LDS, so
+// every neighbour gather is an LDS read and every accumulation an LDS atomic.
+// HBM sees the 8 bytes per entry once, coalesced, plus the positions of the
+// referenced partitions once per workgroup (mostly served by the L2).
 //
 // Accumulators are 64-bit fixed point: on gfx950 an LDS float atomic add costs
 // ~190 clocks per wave instruction while 64-bit integer LDS atomics run about
@@ -27,7 +28,7 @@
 // below 2^50 and a row sum of K < 4096 terms below 2^62.
 //
 // Semantics are those of src/kernels/attr_forces.cu:129-184 of the reference;
-// only the order of the fp32 additions inside a row differs.
+// only the order of the additions inside a row differs.
 #include "plan.h"
 
 namespace tsnehip {
@@ -42,7 +43,10 @@ constexpr int kBlock = 1024;
 constexpr int kMaxParts = 1024;
 static_assert(kBlock == kMaxParts, "the partition scan uses one thread per slot");
 constexpr int kPrefetch = 4;        // entries per thread in one work item
-constexpr unsigned int kItemEntries = kPrefetch * kBlock;
+constexpr int kStreamThreads = 768; // force kernel: waves 0-11 stream entries ...
+constexpr int kLoadThreads = kBlock - kStreamThreads;  // ... waves 12-15 stage the partitions
+constexpr unsigned int kItemEntries = kPrefetch * kStreamThreads;
+constexpr int kPadItems = 4;        // empty records after a strip's last item: the pipelined loop needs no guards
 
 // ---------------------------------------------------------------------------
 // Re-blocking: one workgroup per strip.  Histogram of the strip's entries over
@@ -52,7 +56,6 @@ constexpr unsigned int kItemEntries = kPrefetch * kBlock;
 __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
                                                          int N, int K, int strip_rows, int max_items,
                                                          int seg_stride, float *__restrict__ ent_p,
-                                                         unsigned int *__restrict__ ent_c,
                                                          unsigned int *__restrict__ seg, float *__restrict__ p_max) {
     __shared__ unsigned int cursor[kMaxParts];
     __shared__ unsigned int scan[kMaxParts];
@@ -90,18 +93,33 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
         scan[tid] += add;
         __syncthreads();
     }
+    // Layout of a strip's list: {item count, fresh count, -, -}, then one record per item
+    // {first entry, end entry, partition, 1 if the item opens the partition}, kPadItems empty records,
+    // then the partitions in the order they are opened.
     unsigned int *hdr = seg + (size_t)strip * seg_stride;
-    unsigned int *item_begin = hdr + 1;
-    unsigned int *item_part = hdr + 2 + max_items;
+    uint4 *records = reinterpret_cast<uint4 *>(hdr + 4);
+    unsigned int *fresh_parts = hdr + 4 + 4 * (max_items + kPadItems);
     for (unsigned int it = 0; it < items; ++it) {
         const unsigned int slot = scan[tid] - items + it;
-        item_begin[slot] = first + it * kItemEntries;
-        item_part[slot] = (unsigned int)tid;
+        const unsigned int b = first + it * kItemEntries;
+        records[slot] = make_uint4(b, min(first + mine, b + kItemEntries), (unsigned int)tid, it == 0 ? 1u : 0u);
     }
-    if (tid == kMaxParts - 1) {
-        hdr[0] = scan[tid];
-        item_begin[scan[tid]] = count;
+    const unsigned int n_items_total = scan[kMaxParts - 1];
+    if (tid < kPadItems) records[n_items_total + tid] = make_uint4(count, count, 0u, 0u);
+    if (tid == 0) hdr[0] = n_items_total;
+    __syncthreads();
+    // Third scan, over the "referenced at all" flags: the order in which partitions are opened.
+    const unsigned int flag = mine > 0u ? 1u : 0u;
+    scan[tid] = flag;
+    __syncthreads();
+    for (int off = 1; off < kMaxParts; off <<= 1) {
+        const unsigned int add = tid >= off ? scan[tid - off] : 0u;
+        __syncthreads();
+        scan[tid] += add;
+        __syncthreads();
     }
+    if (flag) fresh_parts[scan[tid] - 1u] = (unsigned int)tid;
+    if (tid == kMaxParts - 1) hdr[1] = scan[tid];
     // Entries are visited neighbour slot by neighbour slot, so that neighbouring positions of a
     // partition's run belong to different rows: a wave of the force kernel then spreads its LDS
     // atomics over many accumulators even when most neighbours of a row share one partition.
@@ -115,8 +133,8 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
         const unsigned int pos = atomicAdd(&cursor[part], 1u);
         const float pv = pij[base + e];
         biggest = fmaxf(biggest, fabsf(pv));
-        ent_p[base + pos] = pv;
-        ent_c[base + pos] = (unsigned int)(col - part * kPartPoints) | (row_local << kColBits);
+        reinterpret_cast<uint2 *>(ent_p)[base + pos] =
+            make_uint2(__float_as_uint(pv), (unsigned int)(col - part * kPartPoints) | (row_local << kColBits));
     }
     biggest = group_max<kWave>(biggest);
     // Non-negative floats order like their bit patterns.
@@ -130,6 +148,17 @@ __global__ void clear_pmax_kernel(float *p_max) {
 // ---------------------------------------------------------------------------
 // One workgroup per strip; dynamic LDS: part[kPartPoints] float2, then
 // yi[kStripMax] float2, then acc_x[kStripMax] and acc_y[kStripMax], 64-bit fixed point.
+//
+// The waves have two roles.  Waves 0-11 stream the strip's entries item by item
+// (three rotating register sets, two items in flight, all loads unconditional so
+// that the outstanding-load counts the compiler works with are exact) and do the
+// LDS gathers and accumulations.  Waves 12-15 only stage partitions: they hold
+// the next partition in registers, and when the streaming waves reach an item
+// that opens it, everybody meets at a barrier, the staging waves write it to LDS,
+// a second barrier releases the streaming waves, and the staging waves go and
+// fetch the partition after that.  A barrier does not wait for memory, so the
+// entry stream never drains at a partition switch.  Both roles execute two
+// barriers per opened partition and one at the end.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int rl, float vx, float vy,
                                           double scale) {
@@ -144,7 +173,6 @@ __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int 
 }
 
 __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float *__restrict__ ent_p,
-                                                                    const unsigned int *__restrict__ ent_c,
                                                                     const unsigned int *__restrict__ seg,
                                                                     const float2 *__restrict__ yxy,
                                                                     const float *__restrict__ p_max,
@@ -164,10 +192,11 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
     // kernel runs, and constant-space loads at uniform addresses are scalar loads, which do not
     // queue behind the vector loads in flight.
     typedef const __attribute__((address_space(4))) unsigned int *ConstWords;
+    typedef unsigned int Record __attribute__((ext_vector_type(4)));
     ConstWords hdr = (ConstWords)(seg + (size_t)strip * seg_stride);
     const int n_items = (int)hdr[0];
-    ConstWords my_seg = hdr + 1;               // n_items + 1 entry offsets
-    ConstWords my_part = hdr + 2 + max_items;  // partition of each item
+    const int n_fresh = (int)hdr[1];
+    ConstWords fresh_parts = hdr + 4 + 4 * (max_items + kPadItems);
     const float pm = *p_max;
     const double scale = pm > 0.0f ? 2251799813685248.0 / (double)pm : 1.0;  // 2^51 / p_max
 
@@ -176,82 +205,94 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         acc[r] = 0ull;
         acc[kStripMax + r] = 0ull;
     }
+    // (the first partition switch's barriers also publish yi / acc)
 
-    constexpr int kPartLoads = kPartPoints / (2 * kBlock);  // float4 (two points) loads per thread
-    static_assert(kPartPoints % (2 * kBlock) == 0, "partition staging assumes whole float4 rounds");
-    const float4 *yxy4 = reinterpret_cast<const float4 *>(yxy);
-    float4 *part4 = reinterpret_cast<float4 *>(part);
-    const int last_pair_all = (N - 1) / 2;  // yxy is padded, so a pair may run one point past N
-
-    // Register sets rotate between "being consumed" and "in flight", so the
-    // prefetch of later phases overlaps the LDS work of phase p without any
-    // register copies (a copy would have to wait for the load it copies).
-    struct PhaseRegs {
-        float pv[kPrefetch];
-        unsigned int pc[kPrefetch];
-        float4 stage[kPartLoads];
-        unsigned int b, e;
-        bool fresh;  // the item starts a new partition (uniform over the workgroup)
-    };
-    // All loads are unconditional (addresses clamped into range) so that none waits for another.
-    const size_t last_entry = (size_t)nrows * K - 1;
-    auto issue = [&](PhaseRegs &R, int item) {
-        R.b = my_seg[item];
-        R.e = my_seg[item + 1];
-        const int p = (int)my_part[item];
-        R.fresh = item == 0 || p != (int)my_part[item - 1];
+    if (tid >= kStreamThreads) {
+        // ---- staging waves ----
+        const int lt = tid - kStreamThreads;
+        constexpr int kPartLoads = kPartPoints / (2 * kLoadThreads);  // float4 (two points) loads per thread
+        static_assert(kPartPoints % (2 * kLoadThreads) == 0, "partition staging assumes whole float4 rounds");
+        // A native vector type with compile-time indices: an array of HIP float4 structs ends up
+        // in scratch memory, where every load waits for the one before.
+        typedef float Quad __attribute__((ext_vector_type(4)));
+        const Quad *yxy4 = reinterpret_cast<const Quad *>(yxy);
+        Quad *part4 = reinterpret_cast<Quad *>(part);
+        const int last_pair_all = (N - 1) / 2;  // yxy is padded, so a pair may run one point past N
+        Quad stage[kPartLoads];
+        auto fetch = [&](int k) {
+            const int p = (int)fresh_parts[k];
 #pragma unroll
-        for (int k = 0; k < kPrefetch; ++k) {
-            const size_t t = min((size_t)R.b + tid + k * kBlock, last_entry);
-            R.pv[k] = ent_p[base + t];
-            R.pc[k] = ent_c[base + t];
+            for (int u = 0; u < kPartLoads; ++u)
+                stage[u] = yxy4[min(p * (kPartPoints / 2) + lt + u * kLoadThreads, last_pair_all)];
+        };
+        if (n_fresh > 0) fetch(0);
+        for (int k = 0; k < n_fresh; ++k) {
+            __syncthreads();  // the streaming waves are done with the partition in LDS
+#pragma unroll
+            for (int u = 0; u < kPartLoads; ++u) part4[lt + u * kLoadThreads] = stage[u];
+            __syncthreads();  // partition k is staged
+            if (k + 1 < n_fresh) fetch(k + 1);
         }
-        // Every item issues the same number of loads, so the compiler's outstanding-load counts stay
-        // exact and no wait ever covers a younger prefetch.  An item that re-uses the staged partition
-        // points all lanes at one address instead: a single cache line per load, nothing to ingest.
+    } else {
+        // ---- streaming waves ----
+        typedef unsigned int Entry __attribute__((ext_vector_type(2)));  // {probability bits, packed row / column}
+        const Entry *ent = reinterpret_cast<const Entry *>(ent_p);
+        struct PhaseRegs {
+            Entry en[kPrefetch];
+            Record rec;  // {first entry, end entry, partition, opens a partition}
+        };
+        const size_t last_entry = (size_t)nrows * K - 1;
+        auto issue = [&](PhaseRegs &R) {
 #pragma unroll
-        for (int k = 0; k < kPartLoads; ++k)
-            R.stage[k] = yxy4[R.fresh ? min(p * (kPartPoints / 2) + tid + k * kBlock, last_pair_all) : 0];
-    };
-    auto consume = [&](PhaseRegs &R) {
-#pragma unroll
-        for (int k = 0; k < kPrefetch; ++k) {
-            const unsigned int t = R.b + tid + k * kBlock;
-            if (t < R.e) {
-                const unsigned int rl = R.pc[k] >> kColBits;
-                const float2 yj = part[R.pc[k] & ((1u << kColBits) - 1u)];
-                const float2 y0 = yi[rl];
-                const float dx = y0.x - yj.x, dy = y0.y - yj.y;
-                const float w = R.pv[k] * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
-                add_force(acc, rl, w * dx, w * dy, scale);
+            for (int k = 0; k < kPrefetch; ++k) {
+                const size_t t = min((size_t)R.rec.x + tid + k * kStreamThreads, last_entry);
+                R.en[k] = ent[base + t];
             }
-        }
-    };
-    auto stage_to_lds = [&](PhaseRegs &R) {
-        if (!R.fresh) return;  // same partition as the previous item: it is already staged
-        __syncthreads();       // everyone is done reading the previous partition (first time: yi / acc are set)
+        };
+        auto consume = [&](PhaseRegs &R) {
+            if (R.rec.w) {
+                __syncthreads();  // everyone is done with the previous partition
+                __syncthreads();  // the staging waves have written the new one
+            }
 #pragma unroll
-        for (int k = 0; k < kPartLoads; ++k) part4[tid + k * kBlock] = R.stage[k];
-        __syncthreads();
-    };
-
-    // Prefetch distance two: while item p is consumed, the loads of items
-    // p+1 and p+2 are in flight (a memory round trip is several items long).
-    PhaseRegs R0, R1, R2;
-    if (0 < n_items) issue(R0, 0);
-    if (1 < n_items) issue(R1, 1);
-    for (int p = 0; p < n_items; p += 3) {
-        stage_to_lds(R0);
-        if (p + 2 < n_items) issue(R2, p + 2);
-        consume(R0);
-        if (p + 1 >= n_items) break;
-        stage_to_lds(R1);
-        if (p + 3 < n_items) issue(R0, p + 3);
-        consume(R1);
-        if (p + 2 >= n_items) break;
-        stage_to_lds(R2);
-        if (p + 4 < n_items) issue(R1, p + 4);
-        consume(R2);
+            for (int k = 0; k < kPrefetch; ++k) {
+                const unsigned int t = R.rec.x + tid + k * kStreamThreads;
+                if (t < R.rec.y) {
+                    const unsigned int rl = R.en[k].y >> kColBits;
+                    const float2 yj = part[R.en[k].y & ((1u << kColBits) - 1u)];
+                    const float2 y0 = yi[rl];
+                    const float dx = y0.x - yj.x, dy = y0.y - yj.y;
+                    const float w = __uint_as_float(R.en[k].x) * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
+                    add_force(acc, rl, w * dx, w * dy, scale);
+                }
+            }
+        };
+        // Prefetch distance two: while item p is consumed, the loads of items p+1 and p+2 are in
+        // flight; the record of item p+3 is fetched (a scalar load) a whole item before it is needed.
+        // The list ends in kPadItems empty records, so nothing here is guarded.
+        typedef const __attribute__((address_space(4))) Record *ConstRecords;
+        ConstRecords records = (ConstRecords)(seg + (size_t)strip * seg_stride + 4);
+        PhaseRegs R0, R1, R2;
+        Record next0, next1, next2;
+        R0.rec = records[0];
+        R1.rec = records[1];
+        R2.rec = records[2];
+        issue(R0);
+        issue(R1);
+        for (int p = 0; p < n_items; p += 3) {
+            next0 = records[p + 3];
+            issue(R2);
+            consume(R0);
+            R0.rec = next0;
+            next1 = records[p + 4];
+            issue(R0);
+            consume(R1);
+            R1.rec = next1;
+            next2 = records[p + 5];
+            issue(R1);
+            consume(R2);
+            R2.rec = next2;
+        }
     }
     __syncthreads();
     const double inv_scale = 1.0 / scale;
@@ -269,10 +310,8 @@ static_assert(kBlockedLds <= 160 * 1024, "one workgroup must fit the 160 KB of L
 
 void release_blocked(tsne_hip_plan *p) {
     (void)hipFree(p->ent_p);
-    (void)hipFree(p->ent_c);
     (void)hipFree(p->seg);
     p->ent_p = nullptr;
-    p->ent_c = nullptr;
     p->seg = nullptr;
     p->blocked_ready = false;
 }
@@ -302,10 +341,9 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     p->n_parts = n_parts;
     // A strip's work list: one item per referenced partition plus one per further kItemEntries entries.
     p->max_items = n_parts + (int)(((int64_t)strip_rows * K) / kItemEntries) + 1;
-    p->seg_stride = 2 * p->max_items + 4;
+    p->seg_stride = 4 + 4 * (p->max_items + kPadItems) + ((n_parts + 3) & ~3);
     const size_t nnz = (size_t)N * K;
-    bool ok = hipMalloc(&p->ent_p, sizeof(float) * nnz) == hipSuccess &&
-              hipMalloc(&p->ent_c, sizeof(unsigned int) * nnz) == hipSuccess &&
+    bool ok = hipMalloc(&p->ent_p, 2 * sizeof(float) * nnz) == hipSuccess &&
               hipMalloc(&p->seg, sizeof(unsigned int) * (size_t)p->n_strips * p->seg_stride) == hipSuccess;
     if (!ok) {
         release_blocked(p);
@@ -315,7 +353,7 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     clear_pmax_kernel<<<1, 64, 0, s>>>(&p->scalars->vmax);
     TSNE_LAUNCHED(s);
     reblock_kernel<<<p->n_strips, kBlock, 0, s>>>(pij, indices, N, K, strip_rows, p->max_items, p->seg_stride, p->ent_p,
-                                                  p->ent_c, p->seg,
+                                                  p->seg,
                                                   &p->scalars->vmax);
     TSNE_LAUNCHED(s);
     TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attractive_blocked_kernel),
@@ -331,7 +369,7 @@ int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s) {
         return 1;
     }
     if (profile_mark(p, kKernelAttractive, s)) return 1;
-    attractive_blocked_kernel<<<p->n_strips, kBlock, kBlockedLds, s>>>(p->ent_p, p->ent_c, p->seg, p->yxy,
+    attractive_blocked_kernel<<<p->n_strips, kBlock, kBlockedLds, s>>>(p->ent_p, p->seg, p->yxy,
                                                                        &p->scalars->vmax, attr, p->num_points,
                                                                        p->num_neighbors, p->strip_rows, p->max_items,
                                                                        p->seg_stride);

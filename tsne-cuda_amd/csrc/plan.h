@@ -69,9 +69,9 @@ struct tsne_hip_plan {
     float *rep = nullptr;   // 2N
 
     // Re-blocked copy of the sparse pattern for the LDS-staged attractive kernel.
-    float *ent_p = nullptr;         // nnz probabilities, grouped by (row strip, column partition)
-    unsigned int *ent_c = nullptr;  // nnz packed (column within partition | row within strip << 14)
-    unsigned int *seg = nullptr;    // per strip seg_stride words: item count, item offsets, item partitions
+    float *ent_p = nullptr;         // nnz entries {probability, packed (column in partition | row in strip << 13)},
+                                    // 8 bytes each, grouped by (row strip, column partition)
+    unsigned int *seg = nullptr;    // per strip seg_stride words: counts, item records, partitions in opening order
     int strip_rows = 0, n_strips = 0, n_parts = 0, max_items = 0, seg_stride = 0;
     bool blocked_ready = false;
 
