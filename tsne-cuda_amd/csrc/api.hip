@@ -1,6 +1,7 @@
 // Stage-level C ABI: argument checks, plan lifetime, and the fused gradient loop.
 #include <cmath>
 #include <cstdarg>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -91,6 +92,36 @@ int check_plan(const tsne_hip_plan *p, const char *who) {
 }  // namespace
 }  // namespace tsnehip
 
+namespace tsnehip {
+
+static bool overlap_enabled() {
+    static const bool on = [] {
+        const char *v = std::getenv("TSNE_OVERLAP");
+        return !(v && v[0] == '0');
+    }();
+    return on;
+}
+
+int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
+                float *old_forces, float eta, float momentum, float exaggeration, int slot, float *normalization,
+                hipStream_t s) {
+    const bool overlap = overlap_enabled() && !p->profiling && p->side_stream != nullptr;
+    hipStream_t rs = overlap ? p->side_stream : s;
+    if (overlap) {
+        TSNE_TRY(hipEventRecord(p->fork_event, s));
+        TSNE_TRY(hipStreamWaitEvent(rs, p->fork_event, 0));
+    }
+    if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, rs)) return 1;
+    if (overlap) TSNE_TRY(hipEventRecord(p->join_event, rs));
+    if (pij ? launch_attractive(p, pij, indices, p->attr, s) : launch_attractive_blocked(p, p->attr, s)) return 1;
+    if (overlap) TSNE_TRY(hipStreamWaitEvent(s, p->join_event, 0));
+    if (normalization && launch_finish_z(p, normalization, s)) return 1;
+    return launch_update(p, embedding, p->attr, p->rep, gains, old_forces, eta, nullptr, momentum, exaggeration,
+                         slot ^ 1, s);
+}
+
+}  // namespace tsnehip
+
 using namespace tsnehip;
 
 extern "C" {
@@ -165,6 +196,9 @@ int tsne_hip_symmetrize(const float *pij_non_symmetric, const int *indices, int 
 void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     if (!p) return;
     for (hipEvent_t e : p->events) (void)hipEventDestroy(e);
+    if (p->fork_event) (void)hipEventDestroy(p->fork_event);
+    if (p->join_event) (void)hipEventDestroy(p->join_event);
+    if (p->side_stream) (void)hipStreamDestroy(p->side_stream);
     release_blocked(p);
     (void)hipFree(p->yxy);
     (void)hipFree(p->tile_xy);
@@ -239,6 +273,9 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
              hipMemset(p->attr, 0, sizeof(float) * 2 * N) == hipSuccess &&
              hipMemset(p->rep, 0, sizeof(float) * 2 * N) == hipSuccess;
     }
+    ok = ok && hipStreamCreateWithFlags(&p->side_stream, hipStreamNonBlocking) == hipSuccess &&
+         hipEventCreateWithFlags(&p->fork_event, hipEventDisableTiming) == hipSuccess &&
+         hipEventCreateWithFlags(&p->join_event, hipEventDisableTiming) == hipSuccess;
     if (!ok) {
         set_error("plan_create: device allocation or initialisation failed: %s",
                   hipGetErrorString(hipGetLastError()));
@@ -312,12 +349,8 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
         const bool late = step >= force_magnify_iters;
         const float momentum = late ? post_exaggeration_momentum : pre_exaggeration_momentum;
         const float exaggeration = late ? 1.0f : early_exaggeration;
-        if (launch_repulsive(plan, embedding, slot, plan->rep, nullptr, nullptr, s)) return 1;
-        if (pij ? launch_attractive(plan, pij, indices, plan->attr, s) : launch_attractive_blocked(plan, plan->attr, s))
-            return 1;
-        if (normalization && step == step_end - 1 && launch_finish_z(plan, normalization, s)) return 1;
-        if (launch_update(plan, embedding, plan->attr, plan->rep, gains, old_forces, eta, nullptr, momentum,
-                          exaggeration, slot ^ 1, s))
+        if (launch_step(plan, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot,
+                        (normalization && step == step_end - 1) ? normalization : nullptr, s))
             return 1;
         slot ^= 1;
     }

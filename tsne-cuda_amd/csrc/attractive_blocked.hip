@@ -35,9 +35,11 @@ namespace tsnehip {
 
 namespace {
 
-constexpr int kColBits = 13;
-constexpr int kPartPoints = 8192;   // == 1 << kColBits; 64 KB of (x, y) pairs
-constexpr int kStripMax = 4096;     // rows per strip: 32 KB of positions + 64 KB of accumulators
+constexpr int kColBits = 12;
+constexpr int kPartPoints = 4096;   // == 1 << kColBits; 32 KB of (x, y) pairs
+constexpr int kStripMax = 3968;     // rows per strip: 31 KB of positions + 62 KB of accumulators; with the
+                                    // partition 125 KB, which leaves 35 KB of a CU's LDS to the kernels of the
+                                    // repulsive chain that run beside this one
 constexpr double kRoundMagic = 6755399441055744.0;  // 1.5 * 2^52: adding it rounds a double to an integer
 constexpr int kBlock = 1024;
 constexpr int kMaxParts = 1024;

@@ -290,20 +290,31 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         const bool printing = verbose && step % print_interval == 0;
         const bool timing = printing;  // phase timers sample the steps that already synchronise
 
-        if (timing) hip_or_die(hipEventRecord(ev[0], stream), "event");
-        TSNE_OR_DIE(tsnehip::launch_repulsive(plan, d_emb.as<float>(), slot, plan->rep, nullptr, nullptr, stream),
-                    "repulsive forces");
-        if (timing) hip_or_die(hipEventRecord(ev[1], stream), "event");
-        TSNE_OR_DIE(blocked ? tsnehip::launch_attractive_blocked(plan, plan->attr, stream)
-                            : tsnehip::launch_attractive(plan, d_pij.as<float>(), d_idx.as<int>(), plan->attr, stream),
-                    "attractive forces");
-        if (timing) hip_or_die(hipEventRecord(ev[2], stream), "event");
-        if (step + 1 == iterations || want_stop)
-            TSNE_OR_DIE(tsnehip::launch_finish_z(plan, d_norm.as<float>(), stream), "normalisation");
-        TSNE_OR_DIE(tsnehip::launch_update(plan, d_emb.as<float>(), plan->attr, plan->rep, d_gains.as<float>(),
-                                           d_old.as<float>(), opt.learning_rate, nullptr, momentum, exaggeration,
-                                           slot ^ 1, stream),
-                    "update");
+        const bool want_norm = step + 1 == iterations || want_stop;
+        if (!timing) {
+            // Repulsive chain and attractive kernel side by side (plan's side stream), joined before the update.
+            TSNE_OR_DIE(tsnehip::launch_step(plan, blocked ? nullptr : d_pij.as<float>(),
+                                             blocked ? nullptr : d_idx.as<int>(), d_emb.as<float>(),
+                                             d_gains.as<float>(), d_old.as<float>(), opt.learning_rate, momentum,
+                                             exaggeration, slot, want_norm ? d_norm.as<float>() : nullptr, stream),
+                        "gradient step");
+        } else {
+            // Sampled steps run the phases one after the other so that the phase timers mean something.
+            hip_or_die(hipEventRecord(ev[0], stream), "event");
+            TSNE_OR_DIE(tsnehip::launch_repulsive(plan, d_emb.as<float>(), slot, plan->rep, nullptr, nullptr, stream),
+                        "repulsive forces");
+            hip_or_die(hipEventRecord(ev[1], stream), "event");
+            TSNE_OR_DIE(blocked ? tsnehip::launch_attractive_blocked(plan, plan->attr, stream)
+                                : tsnehip::launch_attractive(plan, d_pij.as<float>(), d_idx.as<int>(), plan->attr,
+                                                             stream),
+                        "attractive forces");
+            hip_or_die(hipEventRecord(ev[2], stream), "event");
+            if (want_norm) TSNE_OR_DIE(tsnehip::launch_finish_z(plan, d_norm.as<float>(), stream), "normalisation");
+            TSNE_OR_DIE(tsnehip::launch_update(plan, d_emb.as<float>(), plan->attr, plan->rep, d_gains.as<float>(),
+                                               d_old.as<float>(), opt.learning_rate, nullptr, momentum, exaggeration,
+                                               slot ^ 1, stream),
+                        "update");
+        }
         slot ^= 1;
         if (timing) hip_or_die(hipEventRecord(ev[3], stream), "event");
 

@@ -13,8 +13,9 @@ constexpr int kTerms = 4;         // charges per point (src/fit_tsne.cu:254)
 constexpr int kFft = 1024;        // padded transform length, >= 2 * 3 * n_boxes - 1
 constexpr int kNodePad = 512;     // leading dimension of the transposed spectra (>= nodes per dim)
 constexpr int kMaxBoxes = 170;    // 3 * 170 = 510 nodes <= kNodePad
-constexpr int kTileBoxes = 10;    // boxes per side of a spreading tile (30 x 30 nodes x 4 terms, 28.8 KB of LDS)
-constexpr int kMaxTiles = 17 * 17;  // ceil(kMaxBoxes / kTileBoxes)^2
+constexpr int kTileBoxes = 7;     // boxes per side of a spreading tile (21 x 21 nodes x 4 terms x 8 B = 14.1 KB of LDS:
+                                  // two spreading workgroups fit beside the attractive kernel workgroup of a CU)
+constexpr int kMaxTiles = 25 * 25;  // ceil(kMaxBoxes / kTileBoxes)^2
 constexpr int kChunkPoints = 1024;  // points one workgroup spreads into its private LDS tile
 
 // Lagrange node positions inside a box and the basis denominators, formed in
@@ -75,6 +76,11 @@ struct tsne_hip_plan {
     int strip_rows = 0, n_strips = 0, n_parts = 0, max_items = 0, seg_stride = 0;
     bool blocked_ready = false;
 
+    // The repulsive chain and the attractive kernel of a step are independent: the fused loop runs
+    // the chain on this side stream (default priority) and joins before the update.
+    hipStream_t side_stream = nullptr;
+    hipEvent_t fork_event = nullptr, join_event = nullptr;
+
     // Optional per-kernel timing: an event is recorded before every kernel of
     // the loop and one after the last; a kernel's time is the gap to the next
     // event on the same in-order stream.
@@ -98,6 +104,12 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
 // Writes Z = z_sum - N to the device scalar *normalization.
 int launch_finish_z(tsne_hip_plan *p, float *normalization, hipStream_t s);
 int launch_pack_xy(tsne_hip_plan *p, const float *embedding, hipStream_t s);
+// One gradient step: repulsive chain, attractive forces (prepared pattern when pij is null), optional
+// normalisation output, update.  The chain overlaps the attractive kernel unless profiling is on or
+// TSNE_OVERLAP=0 is set.
+int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
+                float *old_forces, float eta, float momentum, float exaggeration, int slot, float *normalization,
+                hipStream_t s);
 int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, float *attr, hipStream_t s);
 int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s);
 void release_blocked(tsne_hip_plan *p);

@@ -450,12 +450,13 @@ __global__ __launch_bounds__(256) void conv_rows_forward_kernel(float4 *__restri
                                                                 const LoopScalars *sc, int slot,
                                                                 const float2 *__restrict__ twiddles,
                                                                 float2 *__restrict__ row_spectra) {
-    __shared__ float2 tw[kFft];
+    // 32 KB of LDS, twiddles straight from memory (an 8 KB table every CU keeps in its L1): small
+    // enough to run next to the attractive kernel's workgroup on the same CU.
     __shared__ float2 s[4][kFft];  // [row * 2 + pair]
+    const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int m0 = blockIdx.x * 2;
     const float s3 = r2_plane_scale(sc, slot);
-    for (int e = tid; e < kFft; e += 256) tw[e] = twiddles[e];
     for (int e = tid; e < 2 * kFft; e += 256) {
         const int r = e >> kLog2Fft, n = e & (kFft - 1);
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -487,18 +488,12 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
                                                            const float *__restrict__ kernel_rows,
                                                            const float2 *__restrict__ twiddles,
                                                            float2 *__restrict__ col_results) {
-    __shared__ float2 tw[kFft];
-    __shared__ float2 s[5][kFft];  // [col * 2 + pair], then the kernel columns
+    // 24 KB of LDS: the two plane pairs go through one after the other (the kernel columns are
+    // transformed with the first), twiddles come straight from memory.
+    __shared__ float2 s[3][kFft];  // [col], then the kernel columns
+    const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int c0 = blockIdx.x * 2;
-    for (int e = tid; e < kFft; e += 512) tw[e] = twiddles[e];
-    for (int e = tid; e < 4 * kFft; e += 512) {
-        const int f = e >> kLog2Fft, m = e & (kFft - 1);
-        const int col = f >> 1, pair = f & 1;
-        float2 v = make_float2(0.f, 0.f);
-        if (m < G) v = row_spectra[((size_t)pair * kFft + c0 + col) * kNodePad + m];
-        s[f][m] = v;
-    }
     {
         int v0 = rev4(c0), v1 = rev4(c0 + 1);
         v0 = min(v0, kFft - v0);
@@ -510,26 +505,34 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
                 v.x = kernel_rows[(size_t)v0 * kNodePad + a];
                 v.y = kernel_rows[(size_t)v1 * kNodePad + a];
             }
-            s[4][m] = v;
+            s[2][m] = v;
         }
     }
-    __syncthreads();
-    fft_forward(&s[0][0], 5, tw, tid, 512);
-    for (int e = tid; e < 4 * kFft; e += 512) {
-        const int f = e >> kLog2Fft, m = e & (kFft - 1);
-        const float2 kk = s[4][m];
-        const float kv = (f >> 1) ? kk.y : kk.x;
-        float2 v = s[f][m];
-        v.x *= kv;
-        v.y *= kv;
-        s[f][m] = v;
-    }
-    __syncthreads();
-    fft_inverse(&s[0][0], 4, tw, tid, 512);
-    for (int e = tid; e < 4 * kFft; e += 512) {
-        const int f = e >> kLog2Fft, m = e & (kFft - 1);
-        const int col = f >> 1, pair = f & 1;
-        if (m < G) col_results[((size_t)pair * kFft + c0 + col) * kNodePad + m] = s[f][m];
+    for (int pair = 0; pair < 2; ++pair) {
+        for (int e = tid; e < 2 * kFft; e += 512) {
+            const int col = e >> kLog2Fft, m = e & (kFft - 1);
+            float2 v = make_float2(0.f, 0.f);
+            if (m < G) v = row_spectra[((size_t)pair * kFft + c0 + col) * kNodePad + m];
+            s[col][m] = v;
+        }
+        __syncthreads();
+        fft_forward(&s[0][0], pair == 0 ? 3 : 2, tw, tid, 512);
+        for (int e = tid; e < 2 * kFft; e += 512) {
+            const int col = e >> kLog2Fft, m = e & (kFft - 1);
+            const float2 kk = s[2][m];
+            const float kv = col ? kk.y : kk.x;
+            float2 v = s[col][m];
+            v.x *= kv;
+            v.y *= kv;
+            s[col][m] = v;
+        }
+        __syncthreads();
+        fft_inverse(&s[0][0], 2, tw, tid, 512);
+        for (int e = tid; e < 2 * kFft; e += 512) {
+            const int col = e >> kLog2Fft, m = e & (kFft - 1);
+            if (m < G) col_results[((size_t)pair * kFft + c0 + col) * kNodePad + m] = s[col][m];
+        }
+        __syncthreads();
     }
 }
 
@@ -541,11 +544,10 @@ __global__ __launch_bounds__(256) void conv_rows_inverse_kernel(const float2 *__
                                                                 const LoopScalars *sc, int slot,
                                                                 const float2 *__restrict__ twiddles,
                                                                 float4 *__restrict__ node_potentials) {
-    __shared__ float2 tw[kFft];
-    __shared__ float2 s[4][kFft];  // [row * 2 + pair]
+    __shared__ float2 s[4][kFft];  // [row * 2 + pair]; twiddles from memory, as in the forward pass
+    const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int m0 = blockIdx.x * 2;
-    for (int e = tid; e < kFft; e += 256) tw[e] = twiddles[e];
     for (int e = tid; e < 2 * kFft; e += 256) {
         const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
         const float4 v =
