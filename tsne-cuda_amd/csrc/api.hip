@@ -49,9 +49,8 @@ int profile_mark(tsne_hip_plan *p, int id, hipStream_t s) {
 namespace {
 
 const char *const kLoopKernelNames[kKernelCount] = {
-    "step_prologue_kernel",     "kernel_rows_kernel",  "tile_count_kernel",        "tile_scan_kernel",
-    "tile_scatter_kernel",      "spread_kernel",       "conv_rows_forward_kernel", "conv_columns_kernel",
-    "conv_rows_inverse_kernel", "gather_forces_kernel", "attractive_kernel",       "update_kernel"};
+    "tile_count_kernel",        "tile_scatter_kernel",  "spread_kernel",     "conv_rows_forward_kernel", "conv_columns_kernel",
+    "conv_rows_inverse_kernel", "gather_forces_kernel", "attractive_kernel", "update_kernel"};
 
 LagrangeConsts make_lagrange() {
     // fp32 arithmetic in the order of src/fit_tsne.cu:303-321.
@@ -245,7 +244,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
               hipMalloc(&p->tile_count, sizeof(int) * kMaxTiles) == hipSuccess &&
               hipMalloc(&p->tile_cursor, sizeof(int) * kMaxTiles) == hipSuccess &&
               hipMalloc(&p->chunks, sizeof(int4) * p->max_chunks) == hipSuccess &&
-              hipMalloc(&p->num_chunks, sizeof(int)) == hipSuccess &&
+              hipMalloc(&p->num_chunks, 2 * sizeof(int)) == hipSuccess &&
               hipMalloc(&p->node_charges, sizeof(float4) * G2) == hipSuccess &&
               hipMalloc(&p->node_potentials, sizeof(float4) * G2) == hipSuccess &&
               hipMalloc(&p->row_spectra, sizeof(float2) * spec) == hipSuccess &&
@@ -265,7 +264,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
              hipMemset(p->yxy, 0, sizeof(float2) * (N + 2)) == hipSuccess &&
              hipMemset(p->node_charges, 0, sizeof(float4) * G2) == hipSuccess &&
              hipMemset(p->tile_count, 0, sizeof(int) * kMaxTiles) == hipSuccess &&
-             hipMemset(p->num_chunks, 0, sizeof(int)) == hipSuccess &&
+             hipMemset(p->num_chunks, 0, 2 * sizeof(int)) == hipSuccess &&
              hipMemset(p->row_spectra, 0, sizeof(float2) * spec) == hipSuccess &&
              hipMemset(p->col_results, 0, sizeof(float2) * spec) == hipSuccess &&
              hipMemset(p->kernel_rows, 0, sizeof(float) * (size_t)(kFft / 2 + 1) * kNodePad) == hipSuccess &&

@@ -27,10 +27,7 @@ struct LagrangeConsts {
 
 // Kernels of one gradient step, in launch order (profiling slots).
 enum LoopKernel {
-    kKernelPrologue = 0,
-    kKernelKernelRows,
-    kKernelTileCount,
-    kKernelTileScan,
+    kKernelTileCount = 0,
     kKernelTileScatter,
     kKernelSpread,
     kKernelConvRowsForward,
@@ -57,7 +54,7 @@ struct tsne_hip_plan {
     int *tile_count = nullptr;     // points per tile
     int *tile_cursor = nullptr;    // running write position per tile during the scatter
     int4 *chunks = nullptr;        // (tile, first point, count, -) per spreading workgroup
-    int *num_chunks = nullptr;
+    int *num_chunks = nullptr;  // [0] chunks of the current step, [1] ticket counter of the tile count kernel
     int max_chunks = 0;
     float4 *node_charges = nullptr;     // n_nodes^2, one float4 (4 terms) per node
     float4 *node_potentials = nullptr;  // n_nodes^2

@@ -180,20 +180,6 @@ __global__ __launch_bounds__(256) void bounds_kernel(const float *__restrict__ v
 }
 
 // ---------------------------------------------------------------------------
-// Step prologue: clears Z and the bounds slot the coming update will fill.
-// ---------------------------------------------------------------------------
-__global__ void step_prologue_kernel(LoopScalars *sc, int next_slot, int *tile_count) {
-    for (int t = threadIdx.x; t < kMaxTiles; t += blockDim.x) tile_count[t] = 0;
-    if (threadIdx.x == 0) {
-        sc->z_sum = 0.0f;
-        if (next_slot >= 0) {
-            sc->min_enc[next_slot] = 0xffffffffu;
-            sc->max_enc[next_slot] = 0u;
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
 // Spread: w[node][t] += Lx_a * Ly_b * q[t] (src/kernels/nbodyfft.cu:107-139).
 // The row index of the node grid is the x node.
 //
@@ -215,35 +201,21 @@ __device__ __forceinline__ int tile_of(float x, float y, const Bounds &bd, int n
     return (box_of(y, bd, n_boxes) / kTileBoxes) * tiles_per_dim + box_of(x, bd, n_boxes) / kTileBoxes;
 }
 
-__global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restrict__ emb, int N, const LoopScalars *sc,
-                                                         int slot, int n_boxes, int *__restrict__ tile_count) {
-    __shared__ int hist[kMaxTiles];
-    const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
-    const int n_tiles = tiles_per_dim * tiles_per_dim;
-    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;
-    __syncthreads();
-    const Bounds bd = load_bounds(sc, slot, n_boxes);
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x)
-        atomicAdd(&hist[tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim)], 1);
-    __syncthreads();
-    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x)
-        if (hist[b]) atomicAdd(&tile_count[b], hist[b]);
-}
-
-// One workgroup: exclusive scan of the tile counts and of the chunk counts,
-// write cursors, cut every tile into chunks of at most kChunkPoints points.
-// Two tiles per thread (kMaxTiles <= 2 * 1024).
-__global__ __launch_bounds__(1024) void tile_scan_kernel(const int *__restrict__ tile_count, int n_tiles,
-                                                         int *__restrict__ tile_cursor, int4 *__restrict__ chunks,
-                                                         int *__restrict__ num_chunks) {
+// Exclusive scan of the tile counts and of the chunk counts by one workgroup of 1024
+// threads: write cursors, every tile cut into chunks of at most kChunkPoints points.
+// Two tiles per thread (kMaxTiles <= 2 * 1024).  Leaves the counters at zero for the
+// next step.
+__device__ __forceinline__ void scan_tiles(int *__restrict__ tile_count, int n_tiles, int *__restrict__ tile_cursor,
+                                           int4 *__restrict__ chunks, int *__restrict__ num_chunks, int *pts,
+                                           int *chk) {
     static_assert(kMaxTiles <= 2048, "the scan handles two tiles per thread");
-    __shared__ int pts[1024], chk[1024];
     const int t = threadIdx.x;
     int cnt[2], nchunk[2];
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
         const int tile = 2 * t + k;
-        cnt[k] = tile < n_tiles ? tile_count[tile] : 0;
+        // The counts were produced by other workgroups' atomics: read them where atomics live.
+        cnt[k] = tile < n_tiles ? atomicExch(&tile_count[tile], 0) : 0;
         nchunk[k] = (cnt[k] + kChunkPoints - 1) / kChunkPoints;
     }
     pts[t] = cnt[0] + cnt[1];
@@ -272,6 +244,50 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(const int *__restrict__
         first_chunk += nchunk[k];
     }
     if (t == 1023) *num_chunks = chk[t];
+}
+
+// First kernel of a step's repulsive chain.  Counts the points per tile; the workgroup that
+// finishes last (a ticket counter tells) scans the counts.  Its first thread also clears Z and
+// the bounds slot the coming update will fill.  tile_count is all zero on entry and on exit.
+__global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restrict__ emb, int N, LoopScalars *sc,
+                                                         int slot, int next_slot, int n_boxes,
+                                                         int *__restrict__ tile_count,
+                                                         int *__restrict__ tile_cursor, int4 *__restrict__ chunks,
+                                                         int *__restrict__ num_chunks, int *__restrict__ ticket) {
+    __shared__ int hist[kMaxTiles];
+    __shared__ int pts[1024], chk[1024];
+    __shared__ int last;
+    const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
+    const int n_tiles = tiles_per_dim * tiles_per_dim;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        sc->z_sum = 0.0f;
+        if (next_slot >= 0) {
+            sc->min_enc[next_slot] = 0xffffffffu;
+            sc->max_enc[next_slot] = 0u;
+        }
+    }
+    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;
+    __syncthreads();
+    const Bounds bd = load_bounds(sc, slot, n_boxes);
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x)
+        atomicAdd(&hist[tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim)], 1);
+    __syncthreads();
+    // The counters live where device-scope atomics are performed, so no cache maintenance is needed
+    // to publish them (a device-wide fence would write back and invalidate the L2 of every XCD, once
+    // per wave): an atomic that has returned its old value has been performed, and the ticket is
+    // taken after all of this workgroup's atomics have returned.
+    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) {
+        if (hist[b]) {
+            const int before = atomicAdd(&tile_count[b], hist[b]);
+            asm volatile("" ::"v"(before));
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) last = atomicAdd(ticket, 1) == (int)gridDim.x - 1;
+    __syncthreads();
+    if (!last) return;
+    scan_tiles(tile_count, n_tiles, tile_cursor, chunks, num_chunks, pts, chk);
+    if (threadIdx.x == 0) *ticket = 0;
 }
 
 // Same point-to-workgroup assignment as tile_count_kernel: the workgroup
@@ -406,16 +422,13 @@ __device__ __forceinline__ float kernel_value(float lo, float h, int a, int b) {
     return (float)(1.0 / (s * s));
 }
 
-__global__ __launch_bounds__(256) void kernel_rows_kernel(const LoopScalars *sc, int slot, int n_boxes,
-                                                          const float2 *__restrict__ twiddles,
-                                                          float *__restrict__ kernel_rows) {
-    __shared__ float2 tw[kFft];
-    __shared__ float2 s[2][kFft];
+__device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *sc, int slot, int n_boxes,
+                                                  const float2 *__restrict__ tw, float *__restrict__ kernel_rows,
+                                                  float2 (*s)[kFft]) {
     const int tid = threadIdx.x;
     const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    const int a0 = blockIdx.x * 4;
-    for (int e = tid; e < kFft; e += 256) tw[e] = twiddles[e];
+    const int a0 = block * 4;
     for (int e = tid; e < 2 * kFft; e += 256) {
         const int f = e >> kLog2Fft, m = e & (kFft - 1);
         const int b = m < kFft / 2 ? m : kFft - m;
@@ -446,15 +459,23 @@ __global__ __launch_bounds__(256) void kernel_rows_kernel(const LoopScalars *sc,
 // starts from zero without a memset.  Output is transposed:
 // row_spectra[pair][pos][m], pos = digit-reversed frequency position.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void conv_rows_forward_kernel(float4 *__restrict__ w, int G,
+__global__ __launch_bounds__(256) void conv_rows_forward_kernel(float4 *__restrict__ w, int G, int n_boxes,
                                                                 const LoopScalars *sc, int slot,
                                                                 const float2 *__restrict__ twiddles,
-                                                                float2 *__restrict__ row_spectra) {
+                                                                float2 *__restrict__ row_spectra,
+                                                                float *__restrict__ kernel_rows) {
     // 32 KB of LDS, twiddles straight from memory (an 8 KB table every CU keeps in its L1): small
     // enough to run next to the attractive kernel's workgroup on the same CU.
     __shared__ float2 s[4][kFft];  // [row * 2 + pair]
     const float2 *tw = twiddles;
     const int tid = threadIdx.x;
+    // The workgroups past the row pairs produce the kernel's row spectra (needed by the column
+    // pass only): the two jobs are independent and share the launch.
+    const int row_blocks = (G + 1) / 2;
+    if ((int)blockIdx.x >= row_blocks) {
+        kernel_rows_block(blockIdx.x - row_blocks, sc, slot, n_boxes, tw, kernel_rows, s);
+        return;
+    }
     const int m0 = blockIdx.x * 2;
     const float s3 = r2_plane_scale(sc, slot);
     for (int e = tid; e < 2 * kFft; e += 256) {
@@ -655,22 +676,13 @@ int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_
 int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *rep, float *point_potentials,
                      float *charges_out, hipStream_t s) {
     const int N = p->num_points, G = p->n_nodes, nb = p->n_boxes;
-    if (profile_mark(p, kKernelPrologue, s)) return 1;
-    step_prologue_kernel<<<1, 256, 0, s>>>(p->scalars, slot ^ 1, p->tile_count);
-    TSNE_LAUNCHED(s);
-    if (profile_mark(p, kKernelKernelRows, s)) return 1;
-    kernel_rows_kernel<<<div_up(G, 4), 256, 0, s>>>(p->scalars, slot, nb, p->twiddles, p->kernel_rows);
-    TSNE_LAUNCHED(s);
     const int tiles_per_dim = (nb + kTileBoxes - 1) / kTileBoxes;
     // Few, large workgroups: every workgroup ends with one global atomic per tile counter, and
     // same-address atomics serialise (about a thousand per counter cost ~20 us).
     const int sort_blocks = std::min(div_up(N, 1024 * 4), 256);
     if (profile_mark(p, kKernelTileCount, s)) return 1;
-    tile_count_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_count);
-    TSNE_LAUNCHED(s);
-    if (profile_mark(p, kKernelTileScan, s)) return 1;
-    tile_scan_kernel<<<1, 1024, 0, s>>>(p->tile_count, tiles_per_dim * tiles_per_dim, p->tile_cursor, p->chunks,
-                                      p->num_chunks);
+    tile_count_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, slot ^ 1, nb, p->tile_count,
+                                                   p->tile_cursor, p->chunks, p->num_chunks, p->num_chunks + 1);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelTileScatter, s)) return 1;
     tile_scatter_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_cursor, p->tile_xy);
@@ -685,8 +697,8 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
         TSNE_TRY(hipMemcpyAsync(charges_out, p->node_charges, sizeof(float4) * (size_t)G * G,
                                 hipMemcpyDeviceToDevice, s));
     if (profile_mark(p, kKernelConvRowsForward, s)) return 1;
-    conv_rows_forward_kernel<<<div_up(G, 2), 256, 0, s>>>(p->node_charges, G, p->scalars, slot, p->twiddles,
-                                                          p->row_spectra);
+    conv_rows_forward_kernel<<<div_up(G, 2) + div_up(G, 4), 256, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
+                                                                         p->twiddles, p->row_spectra, p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
     conv_columns_kernel<<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
