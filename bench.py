@@ -34,6 +34,7 @@ def main():
     ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end fit through pymodule_tsne")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-steps", type=int, default=20, help="gradient steps of the CPU baseline sample")
+    ap.add_argument("--cpu-knn-rows", type=int, default=512, help="query rows of the CPU baseline's kNN sample")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 10 plain 256 MiB device copies (known traffic, to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -130,9 +131,17 @@ def main():
         a = time.perf_counter()
         oracle.iterate(P_h, idx_h, y0, args.cpu_steps, eta=eta)
         cpu_s = time.perf_counter() - a
+        # ... and its exact kNN on a slice of the query rows against all points.
+        knn_rows = min(n, args.cpu_knn_rows)
+        a = time.perf_counter()
+        oracle.knn(X, k, rows=(0, knn_rows))
+        knn_cpu_s = time.perf_counter() - a
         cpu = {"value": args.cpu_steps / cpu_s, "unit": "iter/s", "cores": oracle.num_threads(), "kind": "port",
-               "sample": "%d gradient steps of the same %d x %d workload (P and neighbours from the GPU stages), "
-                         "C++/OpenMP restatement" % (args.cpu_steps, n, k)}
+               "sample": "%d gradient steps of the same %d x %d workload (P and neighbours from the GPU stages) and "
+                         "the exact kNN of %d query rows against all %d points, C++/OpenMP restatement"
+                         % (args.cpu_steps, n, k, knn_rows, n),
+               "knn_query_rows_per_s": knn_rows / knn_cpu_s,
+               "fit_seconds_extrapolated": n / (knn_rows / knn_cpu_s) + 1000.0 / (args.cpu_steps / cpu_s)}
 
     # HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes whose
     # summary sits in profiles/bench_c3_1M_hbm_counters.txt (424126 x 2 KiB fetched + 7826 x 1 KiB written);
