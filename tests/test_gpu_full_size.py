@@ -1,0 +1,106 @@
+"""Parity at the benchmark's own size: config c3, 1,000,000 x 50, K = 90.
+
+The oracle is fast enough for everything but the full neighbour search, so the
+stages after kNN are compared directly (same tolerances as at 5000 points) and
+kNN through a sample of query rows, each against all million candidates.  The
+points are renumbered in locality order first, as RunTsne does.
+"""
+import numpy as np
+import pytest
+
+import oracle
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+N, K, PERPLEXITY, EPS = 1000000, 90, 30.0, 1e-4
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, np.float64).ravel()
+    b = np.asarray(b, np.float64).ravel()
+    return float(np.linalg.norm(a - b) / np.linalg.norm(b))
+
+
+@pytest.fixture(scope="module")
+def c3():
+    from tsnecuda import stages, synthetic
+    X, fit = synthetic.make_config("c3")
+    assert X.shape == (N, 50) and fit["num_neighbors"] == K
+    dX = torch.from_numpy(X).cuda()
+    order = stages.locality_order(dX)
+    dXs = stages.gather_rows(dX, order)
+    del dX
+    idx, d2, stats = stages.knn_select(dXs, K, 0)
+    Xs = dXs.cpu().numpy()
+    del dXs
+    dn = stages.max_normalize_(d2.clone())
+    cond = stages.perplexity(dn, PERPLEXITY, EPS)
+    P = stages.symmetrize(cond, idx)
+    Y0 = synthetic.initial_embedding(N)
+    y0 = np.concatenate([Y0[:, 0], Y0[:, 1]]).astype(np.float32)
+    return dict(stages=stages, order=order.cpu().numpy(), Xs=Xs, idx=idx, d2=d2, dn=dn, cond=cond, P=P, y0=y0,
+                knn_stats=stats)
+
+
+def test_order_is_a_permutation_and_the_sweep_skips_tiles(c3):
+    assert np.array_equal(np.sort(c3["order"]), np.arange(N))
+    ran_matrix_sweep, redone, per_mille = c3["knn_stats"]
+    assert ran_matrix_sweep == 1 and redone == 0
+    assert per_mille <= 300  # four equal clusters: a quarter of the tile pairs, plus the cluster borders
+
+
+def test_knn_rows_bit_exact(c3):
+    """192 query rows spread over the numbering, each against all 1M points."""
+    idx, d2 = c3["idx"], c3["d2"]
+    for first in (0, 333312, N - 64):
+        io, do = oracle.knn(c3["Xs"], K, rows=(first, first + 64))
+        assert np.array_equal(io, idx[first:first + 64].cpu().numpy())
+        assert np.array_equal(do, d2[first:first + 64].cpu().numpy())
+    # structure of every row: self first at distance 0, ascending distances, indices in range and distinct per row
+    assert torch.equal(idx[:, 0].long(), torch.arange(N, device="cuda"))
+    assert bool((d2[:, 0] == 0).all()) and bool((d2[:, 1:] >= d2[:, :-1]).all())
+    assert int(idx.min()) >= 0 and int(idx.max()) < N
+    srt = torch.sort(idx, dim=1).values
+    assert bool((srt[:, 1:] != srt[:, :-1]).all())
+
+
+def test_normalise_perplexity_symmetrise(c3):
+    d2_h, idx_h = c3["d2"].cpu().numpy(), c3["idx"].cpu().numpy()
+    dn_o, _ = oracle.max_normalize(d2_h)
+    assert np.array_equal(c3["dn"].cpu().numpy(), dn_o)
+    p_o = oracle.perplexity(dn_o, PERPLEXITY, EPS)
+    p_g = c3["cond"].cpu().numpy()
+    assert np.allclose(p_g.sum(1), 1.0, atol=2e-5)
+    # rows whose search follows the oracle's path agree to 1e-5; the rest stop one bisection step apart
+    # (the row entropy carries ~1e-6 of fp32 summation noise against eps = 1e-4)
+    close = np.abs(p_g - p_o).max(1) <= 1e-5 * np.maximum(p_o.max(1), 1e-30)
+    assert close.mean() >= 0.95
+    ent = -(p_g * np.log(np.maximum(p_g, 1e-30))).sum(1)
+    assert np.abs(ent - np.log(PERPLEXITY)).max() < 3e-4
+    P_o = oracle.symmetrize(p_g, idx_h)  # same conditional probabilities in: isolates the symmetrisation
+    assert np.allclose(c3["P"].cpu().numpy(), P_o, rtol=1e-6, atol=1e-12)
+    c3["P_h"], c3["idx_h"] = P_o, idx_h
+
+
+def test_forces_and_fused_steps(c3):
+    st = c3["stages"]
+    P_h, idx_h = c3["P"].cpu().numpy(), c3["idx"].cpu().numpy()
+    plan = st.Plan(N, K)
+    plan.prepare_attractive(c3["P"], c3["idx"])
+    # an embedding with structure: 60 steps of the GPU loop from the seeded start
+    y = torch.from_numpy(c3["y0"]).cuda()
+    gains, old = torch.ones_like(y), torch.zeros_like(y)
+    plan.iterate_(None, None, y, gains, old, 0, 60, eta=200.0)
+    y_h, gains_h, old_h = y.cpu().numpy(), gains.cpu().numpy(), old.cpu().numpy()
+    attr = plan.attractive(None, None, y).cpu().numpy()
+    assert rel_l2(attr, oracle.attractive(P_h, idx_h, y_h)) <= 1e-4
+    rep, z = plan.repulsive(y)
+    rep_o, z_o = oracle.repulsive(y_h)
+    assert rel_l2(rep.cpu().numpy(), rep_o) <= 1e-4
+    assert abs(float(z) - z_o) <= 1e-5 * abs(z_o)
+    # three fused steps against three oracle steps from the same state
+    plan.iterate_(None, None, y, gains, old, 60, 63, eta=200.0)
+    y_o, _ = oracle.iterate(P_h, idx_h, y_h, 3, step_begin=60, eta=200.0, gains=gains_h, old_forces=old_h)
+    assert rel_l2(y.cpu().numpy(), y_o) <= 1e-4
+    plan.close()
