@@ -115,10 +115,14 @@ __global__ __launch_bounds__(256) void update_vec4_kernel(float *__restrict__ em
         const float4 ny = make_float4(ey.x + uy.x, ey.y + uy.y, ey.z + uy.z, ey.w + uy.w);
         emb4[i] = nx;
         emb4[n4 + i] = ny;
-        attr4[i] = zero;
-        attr4[n4 + i] = zero;
-        rep4[i] = zero;
-        rep4[n4 + i] = zero;
+        // The reference clears the force arrays here (src/kernels/apply_forces.cu:48-51); the stage-level
+        // call keeps that, the fused loop does not need it: both force kernels overwrite every element.
+        if (!FUSED) {
+            attr4[i] = zero;
+            attr4[n4 + i] = zero;
+            rep4[i] = zero;
+            rep4[n4 + i] = zero;
+        }
         old4[i] = ux;
         old4[n4 + i] = uy;
         gains4[i] = gx;
