@@ -33,6 +33,9 @@ def main():
     ap.add_argument("--points", type=int, default=None, help="override the point count of the workload")
     ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end fit through pymodule_tsne")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="run the repulsive chain and the attractive kernel one after the other (TSNE_OVERLAP=0): "
+                         "per-kernel durations in a trace then are those of kernels running alone")
     ap.add_argument("--cpu-steps", type=int, default=20, help="gradient steps of the CPU baseline sample")
     ap.add_argument("--cpu-knn-rows", type=int, default=512, help="query rows of the CPU baseline's kNN sample")
     ap.add_argument("--calibrate", action="store_true",
@@ -41,6 +44,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X per process, no collectives); run with --gpus 1")
+    if args.no_overlap:
+        os.environ["TSNE_OVERLAP"] = "0"  # read once by the library, at its first gradient step
 
     import numpy as np
     import torch
@@ -144,9 +149,9 @@ def main():
                "fit_seconds_extrapolated": n / (knn_rows / knn_cpu_s) + 1000.0 / (args.cpu_steps / cpu_s)}
 
     # HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes whose
-    # summary sits in profiles/bench_c3_1M_hbm_counters.txt (424126 x 2 KiB fetched + 7826 x 1 KiB written);
+    # summary sits in profiles/bench_c3_1M_hbm_counters.txt (429636 x 2 KiB fetched + 7826 x 1 KiB written);
     # the counters belong to that exact workload, so other sizes report null.
-    traffic = 876.6e6 if (args.workload == "c3" and n == 1000000 and k == 90) else None
+    traffic = 887.9e6 if (args.workload == "c3" and n == 1000000 and k == 90) else None
     out = {
         "metric": "gradient_iters_per_sec",
         "value": iters_per_s,
