@@ -83,6 +83,10 @@ class Options {
 
     // Written by RunTsne.
     float trained_norm = -1.0;
+    // Objective of the returned embedding on the stored pattern, sum P (ln P + ln(1 + d^2) + ln Z), set by
+    // RunTsne (the reference documents no such output and never evaluates its FunctionalKlDivergence,
+    // src/include/util/thrust_transform_functions.h:26-31).
+    double trained_kl_divergence = -1.0;
     bool trained = false;
 
     int random_seed = 0;

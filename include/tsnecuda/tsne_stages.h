@@ -72,6 +72,13 @@ int tsne_hip_locality_order(const float *points, int num_points, int num_dims, i
 int tsne_hip_gather_rows(const float *rows_in, const int *order, int num_rows, int num_cols, float *rows_out,
                          void *stream);
 
+/* Objective of the embedding the last RunTsne / pymodule_tsne call of this thread returned:
+ * sum over the stored pattern of P (ln P + ln(1 + |y_i - y_j|^2) + ln Z), Z from the same
+ * interpolation scheme as the gradient; negative if no fit has run.  No counterpart in the
+ * reference, which never evaluates a divergence (its FunctionalKlDivergence,
+ * src/include/util/thrust_transform_functions.h:26-31, has no call site). */
+double tsne_hip_last_kl_divergence(void);
+
 /* In-place division of n values by their largest absolute value.
  * Replaces tsnecuda::util::MaxNormalizeDeviceVector (src/util/math_utils.cu:66-74). */
 int tsne_hip_max_normalize(float *values, int64_t n, void *stream);

@@ -29,13 +29,17 @@ def test_c0_fit_objective_within_one_percent(c0_problem):
     with open(os.path.join(GOLDEN, "c0_fit.json")) as f:
         gold = json.load(f)
     Y0 = synthetic.initial_embedding(c["X"].shape[0])
-    emb = TSNE(perplexity=c["fit"]["perplexity"], num_neighbors=c["K"], learning_rate=c["fit"]["learning_rate"],
-               n_iter=1000, perplexity_epsilon=1e-4).fit_transform(c["X"], y=Y0)
+    model = TSNE(perplexity=c["fit"]["perplexity"], num_neighbors=c["K"], learning_rate=c["fit"]["learning_rate"],
+                 n_iter=1000, perplexity_epsilon=1e-4)
+    emb = model.fit_transform(c["X"], y=Y0)
     assert emb.shape == (5000, 2) and emb.dtype == np.float32 and emb.flags["F_CONTIGUOUS"]
     assert np.isfinite(emb).all()
     kl = oracle.kl(c["P"], c["idx"], flat(emb))
     print("KL gpu %.5f oracle %.5f initial %.5f" % (kl, gold["kl_exact_z"], gold["kl_initial"]))
     assert abs(kl - gold["kl_exact_z"]) <= 0.01 * gold["kl_exact_z"]
+    # the library's own evaluation of the same embedding (interpolated Z, its own P) agrees with the
+    # oracle's evaluator (exact Z, oracle P)
+    assert abs(model.kl_divergence_ - kl) <= 2e-3 * kl
     # same overall scale of the layout
     assert 0.8 < (emb.max() - emb.min()) / (gold["extent"][1] - gold["extent"][0]) < 1.25
 

@@ -8,6 +8,8 @@
 // are gathered as interleaved (x, y) pairs with one 8-byte load, and the row
 // sum is a lane reduction, so the only HBM traffic is the 8 bytes per non-zero
 // plus the positions.
+#include <algorithm>
+
 #include "plan.h"
 
 namespace tsnehip {
@@ -139,6 +141,63 @@ int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, fl
         attractive_generic_kernel<64><<<div_up(N, 256 / 64), 256, 0, s>>>(pij, indices, p->yxy, attr, N, K);
     }
 #undef TSNE_ATTR
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+
+namespace {
+
+// sum over the pattern of P ln(P (1 + d^2)); the ln Z term is added by the caller (sum P is the
+// second output).  Double accumulation, one pair of atomics per workgroup.
+__global__ __launch_bounds__(256) void kl_terms_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
+                                                       const float *__restrict__ emb, int N, int K,
+                                                       double *__restrict__ out) {
+    double kl = 0.0, mass = 0.0;
+    const int64_t nnz = (int64_t)N * K;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (int64_t)gridDim.x * blockDim.x) {
+        const float p = pij[e];
+        if (p > 0.0f) {
+            const int i = (int)(e / K), j = idx[e];
+            const float dx = emb[i] - emb[j], dy = emb[N + i] - emb[N + j];
+            kl += (double)p * (log((double)p) + log1p((double)dx * dx + (double)dy * dy));
+            mass += (double)p;
+        }
+    }
+    __shared__ double red[2][256 / kWave];
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) {
+        kl += __shfl_xor(kl, m, kWave);
+        mass += __shfl_xor(mass, m, kWave);
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        red[0][threadIdx.x / kWave] = kl;
+        red[1][threadIdx.x / kWave] = mass;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 1; k < 256 / kWave; ++k) {
+            kl += red[0][k];
+            mass += red[1][k];
+        }
+        atomicAdd(&out[0], kl);
+        atomicAdd(&out[1], mass);
+    }
+}
+
+__global__ void clear_pair_kernel(double *out) {
+    if (threadIdx.x < 2 && blockIdx.x == 0) out[threadIdx.x] = 0.0;
+}
+
+}  // namespace
+
+// out[0] = sum P ln(P (1 + d^2)), out[1] = sum P over the pattern (device doubles).
+int launch_kl_terms(const float *pij, const int *indices, const float *embedding, int N, int K, double *out,
+                    hipStream_t s) {
+    clear_pair_kernel<<<1, 64, 0, s>>>(out);
+    TSNE_LAUNCHED(s);
+    const int blocks = (int)std::min<int64_t>(div_up((int64_t)N * K, 256 * 8), 2048);
+    kl_terms_kernel<<<std::max(blocks, 1), 256, 0, s>>>(pij, indices, embedding, N, K, out);
     TSNE_LAUNCHED(s);
     return 0;
 }

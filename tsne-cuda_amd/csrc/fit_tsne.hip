@@ -68,6 +68,8 @@ struct PhaseClock {
     }
 };
 
+thread_local double g_last_kl = -1.0;
+
 int env_int(const char *name, int fallback) {
     const char *v = std::getenv(name);
     return v ? std::atoi(v) : fallback;
@@ -245,12 +247,8 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     TSNE_OR_DIE(tsne_hip_plan_create(&plan, N, K, n_boxes_per_dim, gpu_opt.device), "plan creation");
     // Re-block the sparse pattern for the LDS-staged attractive kernel; shapes it
     // cannot hold (very large K or N) keep the row-ordered kernel.
+    // (The row-ordered pattern stays: the objective of the final embedding is evaluated on it.)
     const bool blocked = tsnehip::prepare_blocked(plan, d_pij.as<float>(), d_idx.as<int>(), stream) == 0;
-    if (blocked) {
-        hip_or_die(hipStreamSynchronize(stream), "pattern re-blocking");
-        d_pij.release();
-        d_idx.release();
-    }
 
     std::ofstream dump_file;
     if (opt.get_dump_points()) {
@@ -397,12 +395,32 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         hip_or_die(hipMemcpy(h_emb.data(), d_emb.ptr, sizeof(float) * 2 * N, hipMemcpyDeviceToHost), "result copy");
         to_caller(h_emb.data(), dst);
     }
+    // Objective of the final embedding: Z of the final positions from one more
+    // repulsive evaluation (the loop's last Z belongs to the positions before
+    // the last update), the pattern sum from the row-ordered P.
+    {
+        DeviceBuffer d_kl(2 * sizeof(double));
+        float z_final = 0.0f;
+        double terms[2] = {0.0, 0.0};
+        TSNE_OR_DIE(tsnehip::launch_repulsive(plan, d_emb.as<float>(), slot, plan->rep, nullptr, nullptr, stream),
+                    "final normalisation");
+        TSNE_OR_DIE(tsnehip::launch_finish_z(plan, d_norm.as<float>(), stream), "final normalisation");
+        TSNE_OR_DIE(tsnehip::launch_kl_terms(d_pij.as<float>(), d_idx.as<int>(), d_emb.as<float>(), N, K,
+                                             d_kl.as<double>(), stream),
+                    "objective");
+        hip_or_die(hipMemcpy(&z_final, d_norm.ptr, sizeof(float), hipMemcpyDeviceToHost), "objective");
+        hip_or_die(hipMemcpy(terms, d_kl.ptr, sizeof(terms), hipMemcpyDeviceToHost), "objective");
+        opt.trained_kl_divergence = z_final > 0.0f ? terms[0] + terms[1] * std::log((double)z_final) : -1.0;
+        g_last_kl = opt.trained_kl_divergence;
+    }
     tsne_hip_plan_destroy(plan);
     opt.trained = true;
     opt.trained_norm = normalization;
 }
 
 }  // namespace tsnecuda
+
+extern "C" double tsne_hip_last_kl_divergence(void) { return g_last_kl; }
 
 extern "C" void pymodule_tsne(float *result, float *points, ssize_t *dims, float perplexity, float learning_rate,
                               float early_exaggeration, float magnitude_factor, int num_neighbors, int iterations,

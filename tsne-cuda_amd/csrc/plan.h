@@ -101,6 +101,9 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
 // Writes Z = z_sum - N to the device scalar *normalization.
 int launch_finish_z(tsne_hip_plan *p, float *normalization, hipStream_t s);
 int launch_pack_xy(tsne_hip_plan *p, const float *embedding, hipStream_t s);
+// out[0] = sum P ln(P (1 + d^2)), out[1] = sum P over the row-ordered pattern (device doubles).
+int launch_kl_terms(const float *pij, const int *indices, const float *embedding, int N, int K, double *out,
+                    hipStream_t s);
 // One gradient step: repulsive chain, attractive forces (prepared pattern when pij is null), optional
 // normalisation output, update.  The chain overlaps the attractive kernel unless profiling is on or
 // TSNE_OVERLAP=0 is set.

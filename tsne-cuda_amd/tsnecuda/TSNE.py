@@ -31,6 +31,8 @@ def _load_library():
     u8 = np.ctypeslib.ndpointer(np.uint8, flags="ALIGNED, CONTIGUOUS")
     c_int, c_float, c_bool = ctypes.c_int, ctypes.c_float, ctypes.c_bool
     lib.pymodule_tsne.restype = None
+    lib.tsne_hip_last_kl_divergence.restype = ctypes.c_double
+    lib.tsne_hip_last_kl_divergence.argtypes = []
     lib.pymodule_tsne.argtypes = [
         f32_2d_out,                          # result
         f32_2d_c,                            # points
@@ -178,6 +180,9 @@ class TSNE(object):
             self.use_interactive, self.viz_server_, self.viz_timeout,
             self.verbosity, self.print_interval, self.gpu_device,
             self.return_style, self.num_snapshots, self.metric)
+        # Objective of the returned embedding on the stored neighbour pattern (sklearn's attribute name;
+        # the reference sets no such attribute).
+        self.kl_divergence_ = float(self._lib.tsne_hip_last_kl_divergence())
         if store is not None:
             self.embedding = store.transpose(0, 2, 1)
         else:
