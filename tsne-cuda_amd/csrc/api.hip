@@ -101,22 +101,48 @@ static bool overlap_enabled() {
     return on;
 }
 
+// Overlapped form: the side stream carries chain(k), update(k), chain(k+1), ... in order, the
+// caller's stream carries attractive(k), attractive(k+1), ...; update(k) waits for attractive(k)
+// and attractive(k+1) for update(k), one event each way per step.  The side stream is opened
+// (made to wait for the caller's stream) by the first step after a join and closed by launch_join.
 int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
                 float *old_forces, float eta, float momentum, float exaggeration, int slot, float *normalization,
                 hipStream_t s) {
     const bool overlap = overlap_enabled() && !p->profiling && p->side_stream != nullptr;
-    hipStream_t rs = overlap ? p->side_stream : s;
-    if (overlap) {
-        TSNE_TRY(hipEventRecord(p->fork_event, s));
-        TSNE_TRY(hipStreamWaitEvent(rs, p->fork_event, 0));
+    if (!overlap) {
+        if (launch_join(p, s)) return 1;
+        if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, s)) return 1;
+        if (pij ? launch_attractive(p, pij, indices, p->attr, s) : launch_attractive_blocked(p, p->attr, s)) return 1;
+        if (normalization && launch_finish_z(p, normalization, s)) return 1;
+        return launch_update(p, embedding, p->attr, p->rep, gains, old_forces, eta, nullptr, momentum, exaggeration,
+                             slot ^ 1, s);
     }
-    if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, rs)) return 1;
-    if (overlap) TSNE_TRY(hipEventRecord(p->join_event, rs));
+    hipStream_t side = p->side_stream;
+    if (!p->side_open) {
+        TSNE_TRY(hipEventRecord(p->fork_event, s));
+        TSNE_TRY(hipStreamWaitEvent(side, p->fork_event, 0));
+        p->side_open = true;
+    } else {
+        TSNE_TRY(hipStreamWaitEvent(s, p->update_event, 0));  // the previous step's update
+    }
+    if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, side)) return 1;
     if (pij ? launch_attractive(p, pij, indices, p->attr, s) : launch_attractive_blocked(p, p->attr, s)) return 1;
-    if (overlap) TSNE_TRY(hipStreamWaitEvent(s, p->join_event, 0));
-    if (normalization && launch_finish_z(p, normalization, s)) return 1;
-    return launch_update(p, embedding, p->attr, p->rep, gains, old_forces, eta, nullptr, momentum, exaggeration,
-                         slot ^ 1, s);
+    TSNE_TRY(hipEventRecord(p->join_event, s));
+    TSNE_TRY(hipStreamWaitEvent(side, p->join_event, 0));
+    if (normalization && launch_finish_z(p, normalization, side)) return 1;
+    if (launch_update(p, embedding, p->attr, p->rep, gains, old_forces, eta, nullptr, momentum, exaggeration, slot ^ 1,
+                      side))
+        return 1;
+    TSNE_TRY(hipEventRecord(p->update_event, side));
+    return 0;
+}
+
+// Makes stream s wait for everything the overlapped steps put on the side stream.
+int launch_join(tsne_hip_plan *p, hipStream_t s) {
+    if (!p->side_open) return 0;
+    TSNE_TRY(hipStreamWaitEvent(s, p->update_event, 0));
+    p->side_open = false;
+    return 0;
 }
 
 }  // namespace tsnehip
@@ -197,6 +223,7 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     for (hipEvent_t e : p->events) (void)hipEventDestroy(e);
     if (p->fork_event) (void)hipEventDestroy(p->fork_event);
     if (p->join_event) (void)hipEventDestroy(p->join_event);
+    if (p->update_event) (void)hipEventDestroy(p->update_event);
     if (p->side_stream) (void)hipStreamDestroy(p->side_stream);
     release_blocked(p);
     (void)hipFree(p->yxy);
@@ -274,7 +301,8 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
     }
     ok = ok && hipStreamCreateWithFlags(&p->side_stream, hipStreamNonBlocking) == hipSuccess &&
          hipEventCreateWithFlags(&p->fork_event, hipEventDisableTiming) == hipSuccess &&
-         hipEventCreateWithFlags(&p->join_event, hipEventDisableTiming) == hipSuccess;
+         hipEventCreateWithFlags(&p->join_event, hipEventDisableTiming) == hipSuccess &&
+         hipEventCreateWithFlags(&p->update_event, hipEventDisableTiming) == hipSuccess;
     if (!ok) {
         set_error("plan_create: device allocation or initialisation failed: %s",
                   hipGetErrorString(hipGetLastError()));
@@ -353,6 +381,7 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
             return 1;
         slot ^= 1;
     }
+    if (launch_join(plan, s)) return 1;
     return profile_mark(plan, -1, s);
 }
 
