@@ -421,3 +421,36 @@ def test_knn_matrix_sweep_verification_falls_back(stages):
     assert stats[0] == 1 and stats[1] > 0
     assert np.array_equal(idx.cpu().numpy(), idx_o)
     assert np.array_equal(d2.cpu().numpy(), d2_o)
+
+
+def test_iterate_graph_replay_matches_eager(stages, c0_problem, monkeypatch):
+    """Small problems replay a captured graph of two steps.  Replays, with eager
+    work and synchronisations between them, give what the eager loop gives (to
+    the repeatability of the loop itself: its float atomics are unordered)."""
+    c = c0_problem
+    n = c["P"].shape[0]
+    dP, di = dev(c["P"]), dev(c["idx"])
+
+    def run(chunks):
+        plan = stages.Plan(n, c["K"])
+        plan.prepare_attractive(dP, di)
+        y = dev(c["y0"]).clone()
+        gains, old = torch.ones_like(y), torch.zeros_like(y)
+        step = 0
+        for k in chunks:
+            plan.iterate_(None, None, y, gains, old, step, step + k, eta=200.0)
+            step += k
+            torch.cuda.synchronize()
+            _ = (y * 2.0).sum().item()  # eager work between the replays
+        out = y.cpu().numpy()
+        plan.close()
+        return out
+
+    monkeypatch.setenv("TSNE_GRAPH", "0")
+    eager = run([12])
+    monkeypatch.setenv("TSNE_GRAPH", "1")
+    replayed = run([5, 4, 3])  # 2 + 2 + 1 replays of the same graph, odd remainders eager
+    assert np.isfinite(replayed).all()
+    assert rel_l2(replayed, eager) <= 1e-3
+    oracle_y, _ = oracle.iterate(c["P"], c["idx"], c["y0"], 12)
+    assert rel_l2(replayed, oracle_y) <= 1e-3

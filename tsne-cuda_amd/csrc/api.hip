@@ -1,4 +1,5 @@
 // Stage-level C ABI: argument checks, plan lifetime, and the fused gradient loop.
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdlib>
@@ -145,6 +146,57 @@ int launch_join(tsne_hip_plan *p, hipStream_t s) {
     return 0;
 }
 
+// Steps are launch-bound below a few hundred thousand points (nine kernels of a few microseconds each).
+static bool graphs_enabled(const tsne_hip_plan *p) {
+    const char *v = std::getenv("TSNE_GRAPH");  // read on every call: cheap, and lets one process try both
+    const int mode = v ? (v[0] == '0' ? 0 : 1) : -1;
+    if (p->profiling || sync_kernels_enabled() || mode == 0) return false;
+    return mode == 1 || p->num_points <= 262144;
+}
+
+int launch_steps(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
+                 float *old_forces, float eta, float momentum, float exaggeration, int count, int &slot,
+                 hipStream_t s) {
+    if (count >= 2 && s != nullptr && graphs_enabled(p)) {
+        hipGraphExec_t exec = nullptr;
+        for (const auto &g : p->step_graphs)
+            if (g.pij == pij && g.indices == indices && g.embedding == embedding && g.gains == gains &&
+                g.old_forces == old_forces && g.eta == eta && g.momentum == momentum &&
+                g.exaggeration == exaggeration && g.slot == slot)
+                exec = g.exec;
+        if (!exec) {
+            // Capture two steps (the bounds slot is back where it started) including the side stream's part.
+            if (launch_join(p, s)) return 1;
+            hipGraph_t graph = nullptr;
+            TSNE_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+            int rc = launch_step(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot,
+                                 nullptr, s);
+            rc = rc || launch_step(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration,
+                                   slot ^ 1, nullptr, s);
+            rc = rc || launch_join(p, s);
+            const hipError_t end = hipStreamEndCapture(s, &graph);
+            if (rc) {
+                if (graph) (void)hipGraphDestroy(graph);
+                return 1;
+            }
+            TSNE_TRY(end);
+            const hipError_t inst = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+            (void)hipGraphDestroy(graph);
+            TSNE_TRY(inst);
+            p->step_graphs.push_back({pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot,
+                                      exec});
+        }
+        if (launch_join(p, s)) return 1;
+        for (; count >= 2; count -= 2) TSNE_TRY(hipGraphLaunch(exec, s));
+    }
+    for (; count > 0; --count) {
+        if (launch_step(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot, nullptr, s))
+            return 1;
+        slot ^= 1;
+    }
+    return 0;
+}
+
 }  // namespace tsnehip
 
 using namespace tsnehip;
@@ -224,6 +276,10 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     if (p->fork_event) (void)hipEventDestroy(p->fork_event);
     if (p->join_event) (void)hipEventDestroy(p->join_event);
     if (p->update_event) (void)hipEventDestroy(p->update_event);
+    for (auto &g : p->step_graphs) (void)hipGraphExecDestroy(g.exec);
+    if (p->enter_event) (void)hipEventDestroy(p->enter_event);
+    if (p->leave_event) (void)hipEventDestroy(p->leave_event);
+    if (p->loop_stream) (void)hipStreamDestroy(p->loop_stream);
     if (p->side_stream) (void)hipStreamDestroy(p->side_stream);
     release_blocked(p);
     (void)hipFree(p->yxy);
@@ -302,7 +358,10 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
     ok = ok && hipStreamCreateWithFlags(&p->side_stream, hipStreamNonBlocking) == hipSuccess &&
          hipEventCreateWithFlags(&p->fork_event, hipEventDisableTiming) == hipSuccess &&
          hipEventCreateWithFlags(&p->join_event, hipEventDisableTiming) == hipSuccess &&
-         hipEventCreateWithFlags(&p->update_event, hipEventDisableTiming) == hipSuccess;
+         hipEventCreateWithFlags(&p->update_event, hipEventDisableTiming) == hipSuccess &&
+         hipStreamCreateWithFlags(&p->loop_stream, hipStreamNonBlocking) == hipSuccess &&
+         hipEventCreateWithFlags(&p->enter_event, hipEventDisableTiming) == hipSuccess &&
+         hipEventCreateWithFlags(&p->leave_event, hipEventDisableTiming) == hipSuccess;
     if (!ok) {
         set_error("plan_create: device allocation or initialisation failed: %s",
                   hipGetErrorString(hipGetLastError()));
@@ -365,24 +424,37 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
     TSNE_REQUIRE(pij || plan->blocked_ready, "iterate: no pattern given and none prepared");
     TSNE_REQUIRE(step_begin <= step_end, "iterate: step range [%d, %d) is reversed", step_begin, step_end);
     if (step_begin == step_end) return 0;
-    hipStream_t s = (hipStream_t)stream;
+    // The loop runs on the plan's own stream, tied to the caller's stream by an event at either end.
+    hipStream_t caller = (hipStream_t)stream, s = plan->loop_stream;
+    TSNE_TRY(hipEventRecord(plan->enter_event, caller));
+    TSNE_TRY(hipStreamWaitEvent(s, plan->enter_event, 0));
     // Bounds and the interleaved copy of the starting embedding; from then on
     // the update kernel keeps both current.
     int slot = 0;
     if (launch_bounds(plan, embedding, slot, s)) return 1;
     if (launch_pack_xy(plan, embedding, s)) return 1;
-    for (int step = step_begin; step < step_end; ++step) {
-        // Schedule of src/fit_tsne.cu:416-420.
-        const bool late = step >= force_magnify_iters;
-        const float momentum = late ? post_exaggeration_momentum : pre_exaggeration_momentum;
-        const float exaggeration = late ? 1.0f : early_exaggeration;
-        if (launch_step(plan, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot,
-                        (normalization && step == step_end - 1) ? normalization : nullptr, s))
+    // Schedule of src/fit_tsne.cu:416-420: two stretches of constant parameters; the step that reports the
+    // normalisation runs by itself.
+    const int last = normalization ? step_end - 1 : step_end;
+    const int switch_at = std::min(std::max(force_magnify_iters, step_begin), last);
+    if (launch_steps(plan, pij, indices, embedding, gains, old_forces, eta, pre_exaggeration_momentum,
+                     early_exaggeration, switch_at - step_begin, slot, s))
+        return 1;
+    if (launch_steps(plan, pij, indices, embedding, gains, old_forces, eta, post_exaggeration_momentum, 1.0f,
+                     last - switch_at, slot, s))
+        return 1;
+    if (normalization) {
+        const bool late = last >= force_magnify_iters;
+        if (launch_step(plan, pij, indices, embedding, gains, old_forces, eta,
+                        late ? post_exaggeration_momentum : pre_exaggeration_momentum,
+                        late ? 1.0f : early_exaggeration, slot, normalization, s))
             return 1;
-        slot ^= 1;
     }
     if (launch_join(plan, s)) return 1;
-    return profile_mark(plan, -1, s);
+    if (profile_mark(plan, -1, s)) return 1;
+    TSNE_TRY(hipEventRecord(plan->leave_event, s));
+    TSNE_TRY(hipStreamWaitEvent(caller, plan->leave_event, 0));
+    return 0;
 }
 
 int tsne_hip_profile_kernel_count(void) { return kKernelCount; }

@@ -78,6 +78,21 @@ struct tsne_hip_plan {
     hipStream_t side_stream = nullptr;
     hipEvent_t fork_event = nullptr, join_event = nullptr, update_event = nullptr;
     bool side_open = false;  // the side stream holds steps the caller's stream has not joined yet
+    // The fused loop runs on this stream of the plan's own (default priority), tied to the caller's stream
+    // by an event at either end: stream capture needs a stream that is not the legacy default one.
+    hipStream_t loop_stream = nullptr;
+    hipEvent_t enter_event = nullptr, leave_event = nullptr;
+    // Replayable graphs of two consecutive steps (launch-bound problem sizes), one per distinct set of
+    // arguments seen.
+    struct StepGraph {
+        const float *pij;
+        const int *indices;
+        float *embedding, *gains, *old_forces;
+        float eta, momentum, exaggeration;
+        int slot;
+        hipGraphExec_t exec;
+    };
+    std::vector<StepGraph> step_graphs;
 
     // Optional per-kernel timing: an event is recorded before every kernel of
     // the loop and one after the last; a kernel's time is the gap to the next
@@ -111,6 +126,12 @@ int launch_kl_terms(const float *pij, const int *indices, const float *embedding
 int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
                 float *old_forces, float eta, float momentum, float exaggeration, int slot, float *normalization,
                 hipStream_t s);
+// `count` consecutive steps with one set of schedule parameters on stream s, starting with bounds slot
+// `slot` (updated).  Problem sizes whose steps are launch-bound replay a captured graph of two steps
+// (TSNE_GRAPH=0 / 1 forces it off / on); s must not be the legacy default stream then.
+int launch_steps(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
+                 float *old_forces, float eta, float momentum, float exaggeration, int count, int &slot,
+                 hipStream_t s);
 // Makes stream s wait for the steps launch_step left on the side stream (no-op when there are none);
 // needed before anything else reads the loop's arrays.
 int launch_join(tsne_hip_plan *p, hipStream_t s);
