@@ -59,7 +59,7 @@ int tsne_hip_knn_select(const float *points, int num_points, int num_dims, int n
 
 /* Locality ordering of the points: order[new] = old (int32, device, num_points
  * entries) such that points that are close in the input space get close numbers
- * (nearest of up to 256 pivots taken from the data, pivots chained greedily;
+ * (nearest of 64 to 256 pivots taken from the data, pivots chained greedily;
  * deterministic; the identity for fewer than 16384 points).  Nothing in t-SNE
  * depends on the numbering of the points; RunTsne renumbers them this way on
  * entry and restores the caller's numbering on exit because the attractive-force

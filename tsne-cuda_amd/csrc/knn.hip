@@ -248,23 +248,84 @@ __device__ __forceinline__ int wave_select(u64 *list, int want, int *cnt, u64 *t
     return want;
 }
 
+// Bounding ball of every tile of kCT consecutive points: the centre is the tile's mean, the
+// radius the largest distance of a member to it, inflated by 1e-3 (far more than the fp32
+// rounding of the sums) so that it is an upper bound.  centers_t is D x T (dimension-major).
+// One workgroup of 128 threads per tile; dynamic LDS: D floats.
+__global__ __launch_bounds__(128) void tile_balls_kernel(const float *__restrict__ X, int N, int D, int T,
+                                                         float *__restrict__ centers_t, float *__restrict__ radius) {
+    extern __shared__ float c[];
+    __shared__ float wmax[2];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int first = t * kCT;
+    const int count = min(kCT, N - first);
+    for (int d = tid; d < D; d += 128) {
+        float sum = 0.0f;
+        for (int i = 0; i < count; ++i) sum += X[(size_t)(first + i) * D + d];
+        sum /= (float)count;
+        c[d] = sum;
+        centers_t[(size_t)d * T + t] = sum;
+    }
+    __syncthreads();
+    float d2 = 0.0f;
+    if (tid < count) {
+        const float *x = X + (size_t)(first + tid) * D;
+        for (int d = 0; d < D; ++d) {
+            const float diff = x[d] - c[d];
+            d2 = fmaf(diff, diff, d2);
+        }
+    }
+    d2 = group_max<kWave>(d2);
+    if ((tid & (kWave - 1)) == 0) wmax[tid / kWave] = d2;
+    __syncthreads();
+    if (tid == 0) radius[t] = sqrtf(fmaxf(wmax[0], wmax[1])) * (1.0f + 1e-3f) + 1e-30f;
+}
+
+constexpr int kHomeTiles = 8;  // candidate tiles on either side of the query tile that are always swept
+
+// Whether tile t may hold a point closer than sqrt(tmax) to some point of the tile whose ball is
+// (qcenter, ra): with c, r the balls, every pair of members is at least |c_a - c_t| - r_a - r_t apart
+// (triangle inequality); 1e-3 relative slack on the centre distance, the radii are upper bounds.
+// Anything that is not a number keeps the tile.
+__device__ __forceinline__ bool tile_may_matter(const float *qcenter, float ra, const float *__restrict__ centers_t,
+                                                const float *__restrict__ radius, int D, int T, int t, float tmax) {
+    float d2 = 0.0f;
+    for (int d = 0; d < D; ++d) {
+        const float diff = qcenter[d] - centers_t[(size_t)d * T + t];
+        d2 = fmaf(diff, diff, d2);
+    }
+    const float lb = sqrtf(d2) * (1.0f - 1e-3f) - (ra + radius[t]);
+    return !(lb > 0.0f && lb * lb > tmax);
+}
+
 // ---------------------------------------------------------------------------
 // VALU sweep.  qlist == nullptr: queries are 0..N-1; otherwise the nq listed ones.
+// Sweeping all queries with tile balls given (bitmap_words > 0), the candidate tiles are visited in
+// two phases as in the matrix sweep: the query tile's neighbourhood in the numbering first, then
+// only the tiles whose ball may hold a point below the largest k-th distance found so far.  The
+// distances here are the canonical ones, so a skipped tile is strictly farther than every threshold.
+// Dynamic LDS: cap keys, then D floats (the query tile's ball centre), then the visit bitmap.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict__ Xt, int N, int Npad, int D, int K,
                                                         int cap, u64 *__restrict__ lists, int num_qtiles,
                                                         const int *__restrict__ qlist, int nq,
-                                                        int *__restrict__ out_idx, float *__restrict__ out_d) {
+                                                        int *__restrict__ out_idx, float *__restrict__ out_d,
+                                                        const float *__restrict__ centers_t,
+                                                        const float *__restrict__ radius, int bitmap_words) {
     __shared__ __attribute__((aligned(16))) float xq[kDC][kQT];
     __shared__ __attribute__((aligned(16))) float xc[kDC][kCT];
     __shared__ u64 thr[kQT];
     __shared__ int cnt[kQT];
     __shared__ int qid[kQT];
     extern __shared__ u64 sortbuf[];
+    float *qcenter = reinterpret_cast<float *>(sortbuf + cap);
+    unsigned int *bitmap = reinterpret_cast<unsigned int *>(qcenter + D);
+    __shared__ float tmax_part[kQT / kWave];
 
     const int tid = threadIdx.x;
     const int tq = tid >> 4, tc = tid & 15;
     const int want = K - 1;
+    const int T = (N + kCT - 1) / kCT;
     u64 *list = lists + (size_t)blockIdx.x * kQT * cap;
 
     for (int qt = blockIdx.x; qt < num_qtiles; qt += gridDim.x) {
@@ -275,7 +336,7 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
             qid[tid] = slot < nq ? (qlist ? qlist[slot] : slot) : -1;
         }
         __syncthreads();
-        for (int c0 = 0; c0 < N; c0 += kCT) {
+        auto process = [&](int c0) {
             float acc[4][8];
 #pragma unroll
             for (int a = 0; a < 4; ++a)
@@ -332,6 +393,44 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
                 for (int ql = 0; ql < kQT; ++ql)
                     if (cnt[ql] > cap - kCT) compact_query(list, cap, want, cnt, thr, ql, sortbuf, tid);
             }
+        };
+        const bool prune = bitmap_words > 0 && qlist == nullptr;
+        const int bt = (qt * kQT) / kCT;  // the ball tile this query tile lies in
+        const int h0 = prune ? max(bt - kHomeTiles, 0) : 0, h1 = prune ? min(bt + kHomeTiles, T - 1) : T - 1;
+        for (int ct = h0; ct <= h1; ++ct) process(ct * kCT);
+        if (prune && (h0 > 0 || h1 < T - 1)) {
+            // Thresholds from what the neighbourhood held, then the tiles that may still matter.
+            for (int ql = 0; ql < kQT; ++ql)
+                if (qid[ql] >= 0) compact_query(list, cap, want, cnt, thr, ql, sortbuf, tid);
+            for (int w = tid; w < bitmap_words; w += 256) bitmap[w] = 0u;
+            for (int d = tid; d < D; d += 256) qcenter[d] = centers_t[(size_t)d * T + bt];
+            if (tid < kQT) {
+                float v = -INFINITY;
+                if (qid[tid] >= 0) {
+                    const u64 t = thr[tid];
+                    v = t == ~0ull ? INFINITY : key_distance(t);
+                    v += 1e-5f * fabsf(v) + 1e-30f;
+                }
+                v = group_max<kWave>(v);
+                if ((tid & (kWave - 1)) == 0) tmax_part[tid / kWave] = v;
+            }
+            __syncthreads();
+            float tmax = tmax_part[0];
+#pragma unroll
+            for (int w = 1; w < kQT / kWave; ++w) tmax = fmaxf(tmax, tmax_part[w]);
+            const float ra = radius[bt];
+            for (int t = tid; t < T; t += 256)
+                if ((t < h0 || t > h1) && tile_may_matter(qcenter, ra, centers_t, radius, D, T, t, tmax))
+                    atomicOr(&bitmap[t >> 5], 1u << (t & 31));
+            __syncthreads();
+            for (int w = 0; w < bitmap_words; ++w) {
+                unsigned int word = bitmap[w];
+                while (word) {
+                    const int t = w * 32 + __ffs((int)word) - 1;
+                    word &= word - 1u;
+                    process(t * kCT);
+                }
+            }
         }
         // Final ordering and output: self first, then the K-1 best others.
         for (int ql = 0; ql < kQT; ++ql) {
@@ -353,41 +452,6 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
         }
     }
 }
-
-// Bounding ball of every tile of kCT consecutive points: the centre is the tile's mean, the
-// radius the largest distance of a member to it, inflated by 1e-3 (far more than the fp32
-// rounding of a sum over at most 128 dimensions) so that it is an upper bound.
-// centers_t is D x T (dimension-major).  One workgroup of 128 threads per tile; D <= 128.
-__global__ __launch_bounds__(128) void tile_balls_kernel(const float *__restrict__ X, int N, int D, int T,
-                                                         float *__restrict__ centers_t, float *__restrict__ radius) {
-    __shared__ float c[128];
-    __shared__ float wmax[2];
-    const int t = blockIdx.x, tid = threadIdx.x;
-    const int first = t * kCT;
-    const int count = min(kCT, N - first);
-    for (int d = tid; d < D; d += 128) {
-        float sum = 0.0f;
-        for (int i = 0; i < count; ++i) sum += X[(size_t)(first + i) * D + d];
-        sum /= (float)count;
-        c[d] = sum;
-        centers_t[(size_t)d * T + t] = sum;
-    }
-    __syncthreads();
-    float d2 = 0.0f;
-    if (tid < count) {
-        const float *x = X + (size_t)(first + tid) * D;
-        for (int d = 0; d < D; ++d) {
-            const float diff = x[d] - c[d];
-            d2 = fmaf(diff, diff, d2);
-        }
-    }
-    d2 = group_max<kWave>(d2);
-    if ((tid & (kWave - 1)) == 0) wmax[tid / kWave] = d2;
-    __syncthreads();
-    if (tid == 0) radius[t] = sqrtf(fmaxf(wmax[0], wmax[1])) * (1.0f + 1e-3f) + 1e-30f;
-}
-
-constexpr int kHomeTiles = 8;  // candidate tiles on either side of the query tile that are always swept
 
 struct SweepArgs {
     const float4 *Xp;
@@ -635,17 +699,9 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
                 __syncthreads();
                 const float tmax = fmaxf(tmax_part[0], tmax_part[1]);
                 const float ra = args.radius[qt];
-                for (int t = tid; t < T; t += 256) {
-                    if (t >= h0 && t <= h1) continue;
-                    float d2 = 0.0f;
-                    for (int d = 0; d < D; ++d) {
-                        const float diff = qcenter[d] - args.centers_t[(size_t)d * T + t];
-                        d2 = fmaf(diff, diff, d2);
-                    }
-                    const float lb = sqrtf(d2) * (1.0f - 1e-3f) - (ra + args.radius[t]);
-                    const bool skip = lb > 0.0f && lb * lb > tmax;  // false for NaN: visit
-                    if (!skip) atomicOr(&bitmap[t >> 5], 1u << (t & 31));
-                }
+                for (int t = tid; t < T; t += 256)
+                    if ((t < h0 || t > h1) && tile_may_matter(qcenter, ra, args.centers_t, args.radius, D, T, t, tmax))
+                        atomicOr(&bitmap[t >> 5], 1u << (t & 31));
                 __syncthreads();
                 nxt = next_tile();
                 if (nxt >= 0) {
@@ -817,18 +873,29 @@ int valu_cap(int K) {
 }
 
 // VALU sweep over all points (qlist == nullptr) or over the nq listed queries.
-int run_valu_sweep(const float *Xt, int N, int Npad, int D, int K, const int *qlist, int nq, int cus, int *indices,
-                   float *sq_dist, hipStream_t s) {
+int run_valu_sweep(const float *points, const float *Xt, int N, int Npad, int D, int K, const int *qlist, int nq,
+                   int cus, int *indices, float *sq_dist, hipStream_t s) {
     const int cap = valu_cap(K);
     const int num_qtiles = div_up(nq, kQT);
     const int grid = std::min(num_qtiles, cus * 3);
-    DeviceMem lists;
-    if (!lists.alloc(sizeof(u64) * (size_t)grid * kQT * cap)) {
+    // Tile balls for skipping far-away candidate tiles: only when all queries are swept and the
+    // neighbourhood that is always swept does not cover everything anyway.
+    const int T = div_up(N, kCT);
+    const bool prune = qlist == nullptr && T > 2 * kHomeTiles + 1;
+    const int bitmap_words = prune ? div_up(T, 32) : 0;
+    DeviceMem lists, centers, radius;
+    if (!lists.alloc(sizeof(u64) * (size_t)grid * kQT * cap) ||
+        (prune && (!centers.alloc(sizeof(float) * (size_t)D * T) || !radius.alloc(sizeof(float) * T)))) {
         set_error("knn: out of device memory for the candidate lists");
         return 1;
     }
-    knn_sweep_kernel<<<grid, 256, sizeof(u64) * cap, s>>>(Xt, N, Npad, D, K, cap, lists.as<u64>(), num_qtiles, qlist,
-                                                          nq, indices, sq_dist);
+    if (prune) {
+        tile_balls_kernel<<<T, 128, sizeof(float) * D, s>>>(points, N, D, T, centers.as<float>(), radius.as<float>());
+        TSNE_TRY(hipGetLastError());
+    }
+    const size_t lds = sizeof(u64) * cap + (prune ? sizeof(float) * D + sizeof(unsigned int) * bitmap_words : 0);
+    knn_sweep_kernel<<<grid, 256, lds, s>>>(Xt, N, Npad, D, K, cap, lists.as<u64>(), num_qtiles, qlist, nq, indices,
+                                            sq_dist, centers.as<float>(), radius.as<float>(), bitmap_words);
     TSNE_TRY(hipGetLastError());
     TSNE_TRY(hipStreamSynchronize(s));
     return 0;
@@ -896,7 +963,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     };
     if (!use_mfma) {
         if (build_transposed()) return 1;
-        return run_valu_sweep(Xt.as<float>(), N, Npad, D, K, nullptr, N, cus, indices, sq_dist, s);
+        return run_valu_sweep(points, Xt.as<float>(), N, Npad, D, K, nullptr, N, cus, indices, sq_dist, s);
     }
 
     const int S4 = (ksteps + 3) / 4;
@@ -916,7 +983,8 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm, S4,
                                                                           Npad, Xp.as<float4>());
     TSNE_TRY(hipGetLastError());
-    tile_balls_kernel<<<num_tiles, 128, 0, s>>>(points, N, D, num_tiles, centers.as<float>(), radius.as<float>());
+    tile_balls_kernel<<<num_tiles, 128, sizeof(float) * D, s>>>(points, N, D, num_tiles, centers.as<float>(),
+                                                               radius.as<float>());
     TSNE_TRY(hipGetLastError());
     SweepArgs args;
     args.Xp = Xp.as<float4>();
@@ -954,7 +1022,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     }
     if (failed > 0) {
         if (build_transposed()) return 1;
-        return run_valu_sweep(Xt.as<float>(), N, Npad, D, K, fail_list.as<int>(), failed, cus, indices, sq_dist, s);
+        return run_valu_sweep(points, Xt.as<float>(), N, Npad, D, K, fail_list.as<int>(), failed, cus, indices, sq_dist, s);
     }
     return 0;
 }

@@ -109,8 +109,10 @@ struct Scratch {
 
 int locality_pivot_count(int N) {
     if (N < 16384) return 0;  // too few points for the ordering to matter
-    int m = 8;
-    while (m * 2 <= N / 4096 && m * 2 <= kMaxPivots) m *= 2;
+    // At least 64: every cluster of the data should own a pivot (with 10 equal clusters the chance
+    // that one of them is missed by 64 random draws is 0.1 %).
+    int m = 64;
+    while (m * 2 <= N / 2048 && m * 2 <= kMaxPivots) m *= 2;
     return m;
 }
 
