@@ -488,7 +488,7 @@ struct SweepArgs {
 // (+inf when fewer than `want` candidates exist), both without the |q|^2 term.
 // ---------------------------------------------------------------------------
 template <int KSTEPS>
-__global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_kernel(const SweepArgs args) {
+__global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_kernel(const SweepArgs args) {
     const float4 *__restrict__ Xp = args.Xp;
     const int N = args.N, D = args.D, Dnorm = args.Dnorm, want = args.want, cap = args.cap;
     const int num_qtiles = args.num_qtiles;
@@ -500,8 +500,8 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
     constexpr int kLoadsPerThread = kTileFloat4 / 256;    // == S4
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     float4 *a_lds = reinterpret_cast<float4 *>(lds_raw);
-    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + 2 * kTileFloat4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
-    unsigned int *bitmap = reinterpret_cast<unsigned int *>(reinterpret_cast<u64 *>(a_lds + 2 * kTileFloat4) + 4 * (size_t)cap);
+    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + kTileFloat4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
+    unsigned int *bitmap = reinterpret_cast<unsigned int *>(reinterpret_cast<u64 *>(a_lds + kTileFloat4) + 4 * (size_t)cap);
     __shared__ u64 thr[kMQ];
     __shared__ int cnt[kMQ];
     __shared__ float qcenter[128];
@@ -552,7 +552,7 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
                 }
             }
         }
-        int buf = 0;
+        const int buf = 0;  // one LDS tile: the next tile waits in registers until this one has been read
         // One tile: compute it from LDS buffer `buf` while the next one travels through registers.
         auto process = [&](int ct, int next_ct) {
             const int c0 = ct * kCT;
@@ -641,9 +641,8 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 2 : 1)) void knn_mfma_sweep_ke
             }
             __syncthreads();  // all waves are done with tile `buf`
             if (next_ct >= 0) {
-                stash(buf ^ 1);
+                stash(buf);
                 __syncthreads();
-                buf ^= 1;
             }
         };
 
@@ -837,7 +836,7 @@ template <int KSTEPS>
 int launch_mfma_sweep(const SweepArgs &args, int grid, hipStream_t s) {
     constexpr int S4 = (KSTEPS + 3) / 4;
     // two tiles + a sort buffer per wave + the visit bitmap
-    const size_t lds = sizeof(float4) * 2 * 4 * S4 * 64 + sizeof(u64) * 4 * args.cap + sizeof(unsigned int) * args.bitmap_words;
+    const size_t lds = sizeof(float4) * 4 * S4 * 64 + sizeof(u64) * 4 * args.cap + sizeof(unsigned int) * args.bitmap_words;
     TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_sweep_kernel<KSTEPS>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     knn_mfma_sweep_kernel<KSTEPS><<<grid, 256, lds, s>>>(args);
@@ -939,7 +938,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     const int mcap = next_pow2(want + kCT) < 256 ? 256 : next_pow2(want + kCT);
     const int num_tiles = div_up(N, kCT);
     const int bitmap_words = div_up(num_tiles, 32);
-    const size_t mfma_lds = sizeof(float4) * 2 * 4 * ((ksteps + 3) / 4) * 64 + sizeof(u64) * 4 * mcap +
+    const size_t mfma_lds = sizeof(float4) * 4 * ((ksteps + 3) / 4) * 64 + sizeof(u64) * 4 * mcap +
                             sizeof(unsigned int) * bitmap_words;
     const bool mfma_fits = ksteps <= kMfmaMaxSteps && mcap <= 4096 && mfma_lds <= 150 * 1024;
     bool use_mfma = mode == 2 || (mode == 0 && mfma_fits && N >= 8192);
@@ -969,7 +968,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     const int S4 = (ksteps + 3) / 4;
     DeviceMem Xp, norms, lists, cand, tau, scal, fail_list, centers, radius;
     const int num_qtiles = div_up(N, kMQ);
-    const int grid = std::min(num_qtiles, cus * 2);
+    const int grid = std::min(num_qtiles, cus * (ksteps <= 28 ? 3 : 2));
     if (!Xp.alloc(sizeof(float4) * (size_t)Npad * S4 * 2) || !norms.alloc(sizeof(float) * Npad) ||
         !lists.alloc(sizeof(u64) * (size_t)grid * kMQ * mcap) || !cand.alloc(sizeof(int) * (size_t)N * want) ||
         !tau.alloc(sizeof(float) * N) || !scal.alloc(4 * sizeof(int)) || !fail_list.alloc(sizeof(int) * N) ||
