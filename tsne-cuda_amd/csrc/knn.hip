@@ -754,17 +754,30 @@ __global__ __launch_bounds__(256) void knn_rerank_kernel(const float *__restrict
             if (j >= 0) {
                 const float *xj = X + (size_t)j * D;
                 float acc = 0.0f;
-                for (int d = 0; d < D; ++d) {
-                    const float df = xq[d] - xj[d];
-                    acc = fmaf(df, df, acc);
+                if ((D & 1) == 0 && (reinterpret_cast<uintptr_t>(X) & 7) == 0) {
+                    // rows are 8-byte aligned: two dimensions per load, the same fma chain
+                    const float2 *q2 = reinterpret_cast<const float2 *>(xq);
+                    const float2 *j2 = reinterpret_cast<const float2 *>(xj);
+                    for (int d = 0; d < D / 2; ++d) {
+                        const float2 a = q2[d], b = j2[d];
+                        const float d0 = a.x - b.x, d1 = a.y - b.y;
+                        acc = fmaf(d0, d0, acc);
+                        acc = fmaf(d1, d1, acc);
+                    }
+                } else {
+                    for (int d = 0; d < D; ++d) {
+                        const float df = xq[d] - xj[d];
+                        acc = fmaf(df, df, acc);
+                    }
                 }
                 key = pack_key(acc, j);
             }
         }
         keys[c] = key;
     }
-    __syncthreads();
-    // Bitonic sort of each wave's keys; all four waves run the same schedule.
+    // Bitonic sort of each wave's own keys: no workgroup barrier, a wave's LDS operations execute in
+    // order and the wavefront fences only keep the compiler from reordering them.
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     for (int k = 2; k <= sort_n; k <<= 1) {
         for (int j = k >> 1; j > 0; j >>= 1) {
             for (int t = lane; t < sort_n / 2; t += kWave) {
@@ -777,7 +790,7 @@ __global__ __launch_bounds__(256) void knn_rerank_kernel(const float *__restrict
                     keys[hi] = a;
                 }
             }
-            __syncthreads();
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         }
     }
     if (!live) return;
