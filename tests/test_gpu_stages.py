@@ -367,7 +367,11 @@ def test_iterate_with_prepared_pattern(stages, c0_problem):
 @pytest.mark.parametrize("n,d,k", [
     (3000, 50, 90),    # the benchmark's shape at small N
     (700, 7, 20),      # odd dimension count, fewer candidates than the K' margin wants
-    (1500, 126, 33),   # the largest dimension count the matrix sweep takes
+    (1500, 126, 33),   # the largest dimension count one wave's registers hold
+    (1500, 127, 33),   # the first that is cut into chunks (3 chunks, the norm row opens the last one)
+    (2200, 190, 40),   # 3 chunks, the last one full but for the norm row's partner
+    (1200, 784, 50),   # config c1's dimension count (13 chunks)
+    (900, 1024, 30),   # config c2's (17 chunks: the norm row has a chunk of its own)
     (40, 3, 40),       # K == N, a single partial tile
     (2500, 33, 300),   # wide neighbour lists
 ])
@@ -391,23 +395,64 @@ def test_knn_tile_skipping_is_exact(stages, scale, d):
     """On locality-ordered points both sweeps skip candidate tiles by their
     bounding balls.  Well separated clusters (most tiles skipped), touching
     clusters (the bound decides tile by tile) and one blob (nothing to skip) all
-    give the oracle's rows bit for bit, and the two sweeps agree wherever the
-    matrix sweep exists (up to 126 dimensions)."""
+    give the oracle's rows bit for bit, and the two sweeps agree (beyond 126
+    dimensions the matrix sweep is the chunked one)."""
     from tsnecuda import synthetic
     n, k = 60000, 40
     X = synthetic.gaussian_clusters(n, d=d, clusters=7, center_scale=scale, seed=int(scale * 10) + d)
     dX = dev(X)
     Xs = stages.gather_rows(dX, stages.locality_order(dX))
     idx_v, d2_v, _ = stages.knn_select(Xs, k, 1)
-    if d <= 126:
-        idx, d2, stats = stages.knn_select(Xs, k, 2)
-        assert stats[0] == 1
-        assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
+    idx, d2, stats = stages.knn_select(Xs, k, 2)
+    assert stats[0] == 1
+    assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
     Xs_h = Xs.cpu().numpy()
     for first in (0, n // 3, n - 96):
         idx_o, d2_o = oracle.knn(Xs_h, k, rows=(first, first + 96))
         assert np.array_equal(idx_v[first:first + 96].cpu().numpy(), idx_o)
         assert np.array_equal(d2_v[first:first + 96].cpu().numpy(), d2_o)
+
+
+def test_knn_chunked_sweep_calibrates_its_margin(stages):
+    """Pixel-like vectors in 784 dimensions: a query's neighbour distances lie so
+    close together that the default margin between neighbour K and candidate K'
+    cannot be verified; the chunked sweep finds that out on a sample of query
+    tiles, widens K' and then verifies (nearly) every query.  Results are the
+    vector sweep's and the oracle's, bit for bit."""
+    from tsnecuda import synthetic
+    n, k = 20000, 45
+    X = synthetic.pixel_like(n=n, d=784)
+    dX = dev(X)
+    Xs = stages.gather_rows(dX, stages.locality_order(dX))
+    idx, d2, stats = stages.knn_select(Xs, k, 0)
+    assert stats[0] == 1 and stats[1] <= n // 100
+    idx_v, d2_v, _ = stages.knn_select(Xs, k, 1)
+    assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
+    Xs_h = Xs.cpu().numpy()
+    for first in (0, n // 2, n - 32):
+        idx_o, d2_o = oracle.knn(Xs_h, k, rows=(first, first + 32))
+        assert np.array_equal(idx[first:first + 32].cpu().numpy(), idx_o)
+        assert np.array_equal(d2[first:first + 32].cpu().numpy(), d2_o)
+
+
+def test_knn_chunked_sweep_gives_up_on_unverifiable_data(stages):
+    """200 dimensions, far from the origin, tiny mutual distances: no margin
+    verifies.  Left to choose, kNN notices on the sample and runs the vector
+    sweep; forced onto the matrix sweep, every query is repaired by the vector
+    sweep afterwards.  Both are exact."""
+    rng = np.random.default_rng(5)
+    n, d, k = 9000, 200, 20
+    base = rng.standard_normal((1, d)).astype(np.float32) * 300.0
+    X = (base + rng.standard_normal((n, d)).astype(np.float32) * 1e-2).astype(np.float32)
+    idx_a, d2_a, stats_a = stages.knn_select(dev(X), k, 0)
+    assert stats_a[0] == 0
+    idx_m, d2_m, stats_m = stages.knn_select(dev(X), k, 2)
+    assert stats_m[0] == 1 and stats_m[1] > n // 2
+    assert torch.equal(idx_a, idx_m) and torch.equal(d2_a, d2_m)
+    for first in (0, n - 48):
+        idx_o, d2_o = oracle.knn(X, k, rows=(first, first + 48))
+        assert np.array_equal(idx_a[first:first + 48].cpu().numpy(), idx_o)
+        assert np.array_equal(d2_a[first:first + 48].cpu().numpy(), d2_o)
 
 
 def test_knn_matrix_sweep_verification_falls_back(stages):

@@ -28,6 +28,19 @@
 //    >= tau - g for a rigorous rounding bound g, and the query passes when its
 //    K-th canonical distance is below that.  Queries that do not pass are redone
 //    by the VALU sweep, so the result is exact either way.
+//
+//  * Chunked MFMA sweep (more than 126 dimensions): the same products, but the
+//    queries no longer fit a wave's registers, so both operands stream in chunks
+//    of 64 dimensions (candidates through LDS, queries straight into registers
+//    from a pre-scaled packed copy) while the 32 x 128 results of a wave
+//    accumulate in registers.  With hundreds of dimensions a query's neighbour
+//    distances lie close together and the rounding bound g grows, so the margin
+//    K' - K is first tried on a sample of query tiles and doubled until the
+//    sample verifies (or the vector sweep is taken instead); the query tiles of
+//    the few queries that still fail are swept once more with twice the margin
+//    before the vector sweep gets what is left.  Sweeps of few query tiles split
+//    every tile's candidates over several workgroups; a merge kernel reduces
+//    their lists to what a single list would have kept.
 #include "common.h"
 
 #include <algorithm>
@@ -102,7 +115,8 @@ __global__ __launch_bounds__(256) void norms_kernel(const float *__restrict__ X,
 // k-step = dimension / 2.  Dimension Dnorm carries |x|^2, padding is zero.
 __global__ __launch_bounds__(256) void pack_points_kernel(const float *__restrict__ X,
                                                           const float *__restrict__ norms, int N, int D, int Dnorm,
-                                                          int S4, int Npad, float4 *__restrict__ Xp) {
+                                                          int S4, int Npad, float4 *__restrict__ Xp,
+                                                          bool query_side) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // one float4 of Xp per thread
     const int64_t total = (int64_t)Npad * S4 * 2;
     if (t >= total) return;
@@ -118,8 +132,8 @@ __global__ __launch_bounds__(256) void pack_points_kernel(const float *__restric
         const int d = 2 * (4 * s4 + c) + h;
         v[c] = 0.0f;
         if (i < N) {
-            if (d < D) v[c] = X[(size_t)i * D + d];
-            else if (d == Dnorm) v[c] = norms[i];
+            if (d < D) v[c] = query_side ? -2.0f * X[(size_t)i * D + d] : X[(size_t)i * D + d];
+            else if (d == Dnorm) v[c] = query_side ? 1.0f : norms[i];
         }
     }
     Xp[t] = make_float4(v[0], v[1], v[2], v[3]);
@@ -466,6 +480,17 @@ struct SweepArgs {
     int bitmap_words;        // ceil(T / 32)
     int trigger;             // a list longer than this is compacted after the tile (<= cap - kCT)
     unsigned long long *tiles_swept;  // statistics: (query tile, candidate tile) pairs computed
+    const float4 *Bp;  // chunked sweep only: query-side packed copy (-2 x_d, 1 in the |c|^2 row)
+    int n_chunks;      // chunked sweep only: chunks of kChunkSteps k-steps per point
+    // Chunked sweep only.  The num_qtiles query tiles are qtile_list[i], or first + i step without a list.
+    // Every query tile is swept by `parts` workgroups, part p taking the candidate tiles t with t % parts == p.
+    // One part writes cand / tau directly (row i * kMQ + query in tile); several parts write the keys they
+    // keep (all bits set where a part has fewer) to row (i * kMQ + query in tile) * parts + p of part_keys,
+    // and knn_merge_parts_kernel picks the `want` best of a query's parts afterwards.
+    const int *qtile_list;
+    int qtile_first, qtile_step;
+    int parts;
+    u64 *part_keys;
 };
 
 // ---------------------------------------------------------------------------
@@ -730,6 +755,291 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
 }
 
 // ---------------------------------------------------------------------------
+// MFMA sweep for more dimensions than one wave's registers hold (more than 126).
+// The k-steps are cut into chunks of kChunkSteps (64 dimensions).  Per candidate tile and chunk the
+// workgroup keeps the chunk of the tile in LDS (32 KB, layout [block (4)][step group (8)][lane (64)]
+// float4, copied verbatim from the packed points), every wave loads the same chunk of its 32 queries
+// from the packed query-side copy (already scaled: -2 q_d, 1 in the |c|^2 row) and the products of
+// all four candidate blocks accumulate over the chunks in 64 registers.  The next chunk of the tile
+// (or the first of the next tile) and of the queries travel through registers meanwhile.  Visiting
+// order, tile skipping, filter, lists and output are those of the kernel above.
+// Dynamic LDS: one tile chunk, one sort buffer (cap keys) per wave, the visit bitmap, D floats
+// (centre of the query tile's ball).
+// ---------------------------------------------------------------------------
+constexpr int kChunkSteps = 32;
+constexpr int kChunkS4 = kChunkSteps / 4;            // float4 per lane, block and chunk
+constexpr int kChunkFloat4 = 4 * kChunkS4 * 64;      // float4 per tile chunk
+
+__global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const SweepArgs args) {
+    const int N = args.N, D = args.D, want = args.want, cap = args.cap;
+    const int num_qtiles = args.num_qtiles, n_chunks = args.n_chunks;
+    u64 *__restrict__ lists = args.lists;
+    int *__restrict__ cand = args.cand;
+    float *__restrict__ tau = args.tau;
+    const size_t tile_stride = (size_t)n_chunks * kChunkFloat4;  // float4 per packed tile
+    const size_t block_stride = (size_t)n_chunks * kChunkS4 * 64;  // float4 per 32-point block of a tile
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    v4f *a_lds = reinterpret_cast<v4f *>(lds_raw);
+    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + kChunkFloat4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
+    unsigned int *bitmap = reinterpret_cast<unsigned int *>(reinterpret_cast<u64 *>(a_lds + kChunkFloat4) + 4 * (size_t)cap);
+    float *qcenter = reinterpret_cast<float *>(bitmap + args.bitmap_words);
+    __shared__ u64 thr[kMQ];
+    __shared__ int cnt[kMQ];
+    __shared__ unsigned int hist_all[4][kWave];
+    __shared__ float tmax_part[2];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int qn = lane & 31, kh = lane >> 5;
+    u64 *list = lists + (size_t)blockIdx.x * kMQ * cap;
+
+    // Chunk c of a candidate tile: global -> registers -> LDS.  Element e = 256 r + tid of the chunk is
+    // float4 (e % 512) of block e / 512 = r / 2.
+    v4f stage[kChunkS4];
+    auto fetch = [&](int tile, int c) {
+        const v4f *src = reinterpret_cast<const v4f *>(args.Xp) + (size_t)tile * tile_stride + (size_t)c * (kChunkS4 * 64) + tid;
+#pragma unroll
+        for (int r = 0; r < kChunkS4; ++r) stage[r] = src[(size_t)(r >> 1) * block_stride + (r & 1) * 256];
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int r = 0; r < kChunkS4; ++r) a_lds[r * 256 + tid] = stage[r];
+    };
+    const int num_ctiles = (N + kCT - 1) / kCT;
+
+    const int P = args.parts;
+    for (int w = blockIdx.x; w < num_qtiles * P; w += gridDim.x) {
+        const int qi = w / P, part = w - qi * P;
+        const int qt = args.qtile_list ? args.qtile_list[qi] : args.qtile_first + qi * args.qtile_step;
+        const int q0 = qt * kMQ;
+        const int q = q0 + wave * 32 + qn;  // this lane's query (>= N in the last tile: padded zeros)
+        if (tid < kMQ) {
+            thr[tid] = ~0ull;
+            cnt[tid] = 0;
+        }
+        // This wave's block of the query-side copy.
+        const v4f *bsrc = reinterpret_cast<const v4f *>(args.Bp) + (size_t)qt * tile_stride + (size_t)wave * block_stride + lane;
+        v4f bcur[kChunkS4], bnext[kChunkS4];
+#pragma unroll
+        for (int s4 = 0; s4 < kChunkS4; ++s4) bcur[s4] = bsrc[s4 * 64];
+
+        // One tile: its first chunk is in LDS and the queries' first chunk in bcur on entry; the same holds
+        // for next_ct on exit.
+        auto process = [&](int ct, int next_ct) {
+            const int c0 = ct * kCT;
+            v16f acc[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+            for (int c = 0; c < n_chunks; ++c) {
+                const bool last = c + 1 == n_chunks;
+                if (!last) fetch(ct, c + 1);
+                else if (next_ct >= 0) fetch(next_ct, 0);
+                {
+                    const v4f *bn = bsrc + (size_t)(last ? 0 : c + 1) * (kChunkS4 * 64);
+#pragma unroll
+                    for (int s4 = 0; s4 < kChunkS4; ++s4) bnext[s4] = bn[s4 * 64];
+                }
+#pragma unroll
+                for (int s4 = 0; s4 < kChunkS4; ++s4) {
+                    v4f x[4];
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) x[b] = a_lds[(b * kChunkS4 + s4) * 64 + lane];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+#pragma unroll
+                        for (int b = 0; b < 4; ++b)
+                            acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(x[b][k], bcur[s4][k], acc[b], 0, 0, 0);
+                }
+                if (!last) {
+                    __syncthreads();  // all waves have read this chunk
+                    stash();
+                    __syncthreads();
+#pragma unroll
+                    for (int s4 = 0; s4 < kChunkS4; ++s4) bcur[s4] = bnext[s4];
+                }
+            }
+            const u64 limit = thr[wave * 32 + qn];
+            // ~0 is "no threshold yet": its distance field does not decode to a number.
+            const float limit_d = limit == ~0ull ? INFINITY : key_distance(limit);
+            // Never +inf: excluded elements are raised to +inf and must fail the test also while the query
+            // has no threshold yet (a part can hold fewer than `want` real candidates, so nothing would
+            // push them out of the list later).
+            const float lim = q < N ? fminf(limit_d, 3.4028234663852886e38f) : -INFINITY;
+            const bool edge_tile = c0 + kCT > N || (unsigned int)(q0 - c0) < (unsigned int)kCT;
+#pragma unroll
+            for (int cb = 0; cb < 4; cb += 2) {
+                v16f &acc0 = acc[cb], &acc1 = acc[cb + 1];
+                // Register v of lane l holds candidate row 8*(v/4) + 4*(l/32) + v%4 of the block, query column l%32.
+                float best = min3(acc0[0], acc0[1], acc0[2]);
+#pragma unroll
+                for (int v = 3; v + 1 < 16; v += 2) best = min3(best, acc0[v], acc0[v + 1]);
+                best = min3(best, acc0[15], acc1[0]);
+#pragma unroll
+                for (int v = 1; v + 1 < 16; v += 2) best = min3(best, acc1[v], acc1[v + 1]);
+                best = fminf(best, acc1[15]);
+                if (best <= limit_d) {
+                    const int jbase = c0 + cb * 32 + 4 * kh;  // element (half, v) is candidate jbase + 32 half + 8 (v / 4) + v % 4
+                    // Candidates beyond N (last tile) and the query itself (its own tile) are raised to +inf.
+                    if (edge_tile) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            const int j = jbase + 8 * (e >> 2) + (e & 3);
+                            if (j >= N || j == q) acc0[e] = INFINITY;
+                            if (j + 32 >= N || j + 32 == q) acc1[e] = INFINITY;
+                        }
+                    }
+                    // Count, reserve the list slots with one LDS atomic, then store the keys.
+                    int n = 0;
+#pragma unroll
+                    for (int e = 0; e < 32; ++e) n += ((e < 16 ? acc0[e & 15] : acc1[e & 15]) <= lim) ? 1 : 0;
+                    if (n != 0) {
+                        const int slot = atomicAdd(&cnt[wave * 32 + qn], n);
+                        u64 *dst = list + (size_t)(wave * 32 + qn) * cap + slot;
+                        float lim2 = lim;
+                        asm volatile("" : "+v"(lim2));  // compare again rather than keep 32 lane masks alive
+#pragma unroll
+                        for (int e = 0; e < 32; ++e) {
+                            const float dist = e < 16 ? acc0[e & 15] : acc1[e & 15];
+                            if (dist <= lim2) *dst++ = pack_key(dist, jbase + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
+                        }
+                    }
+                }
+            }
+            // Lists that a further tile could overflow are compacted by their own wave, right away.
+            {
+                u64 crowded = __ballot(cnt[wave * 32 + qn] > args.trigger) & 0xffffffffull;  // lanes l, l+32 share a query
+                while (crowded) {
+                    const int ql = wave * 32 + (__ffsll((long long)crowded) - 1);
+                    crowded &= crowded - 1;
+                    wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
+                }
+            }
+            __syncthreads();  // all waves are done with the tile's last chunk
+            if (next_ct >= 0) {
+                stash();
+                __syncthreads();
+            }
+#pragma unroll
+            for (int s4 = 0; s4 < kChunkS4; ++s4) bcur[s4] = bnext[s4];
+        };
+
+        // Phase 1: the query tile's neighbourhood; phase 2: the tiles the bitmap keeps.
+        const int T = num_ctiles;
+        const int h0 = max(qt - kHomeTiles * P, 0), h1 = min(qt + kHomeTiles * P, T - 1);  // >= kHomeTiles tiles of every part
+        int word_idx = -1;
+        unsigned int cur_word = 0u;
+        auto next_tile = [&]() -> int {
+            while (cur_word == 0u) {
+                ++word_idx;
+                if (word_idx >= args.bitmap_words) return -1;
+                cur_word = bitmap[word_idx];
+            }
+            const int b = __ffs((int)cur_word) - 1;
+            cur_word &= cur_word - 1u;
+            return word_idx * 32 + b;
+        };
+        int cur = h0 + (part - h0 % P + P) % P;  // this part's first tile of the neighbourhood
+        fetch(cur, 0);
+        __syncthreads();  // the previous query tile's last reads of the LDS chunk
+        stash();
+        __syncthreads();
+        bool home = true;
+        unsigned int swept = 0;
+        while (cur >= 0) {
+            ++swept;
+            int nxt = home ? (cur + P <= h1 ? cur + P : -1) : next_tile();
+            process(cur, nxt);
+            if (nxt < 0 && home && (h0 > 0 || h1 < T - 1)) {
+                home = false;
+                for (int b = 0; b < 32; ++b) {
+                    const int ql = wave * 32 + b;
+                    if (q0 + ql < N)
+                        wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
+                }
+                for (int w = tid; w < args.bitmap_words; w += 256) bitmap[w] = 0u;
+                for (int d = tid; d < D; d += 256) qcenter[d] = args.centers_t[(size_t)d * T + qt];
+                __syncthreads();
+                if (tid < kMQ) {
+                    // Largest squared distance any query of the tile would still accept (rounded up).
+                    float v = -INFINITY;
+                    if (q0 + tid < N) {
+                        const u64 t = thr[tid];
+                        v = t == ~0ull ? INFINITY : key_distance(t) + args.norms[q0 + tid];
+                        v += 1e-5f * fabsf(v) + 1e-30f;
+                    }
+                    v = group_max<kWave>(v);
+                    if (lane == 0) tmax_part[wave] = v;
+                }
+                __syncthreads();
+                const float tmax = fmaxf(tmax_part[0], tmax_part[1]);
+                const float ra = args.radius[qt];
+                for (int t = tid; t < T; t += 256)
+                    if ((t < h0 || t > h1) && t % P == part &&
+                        tile_may_matter(qcenter, ra, args.centers_t, args.radius, D, T, t, tmax))
+                        atomicOr(&bitmap[t >> 5], 1u << (t & 31));
+                __syncthreads();
+                nxt = next_tile();
+                if (nxt >= 0) {
+                    fetch(nxt, 0);
+                    stash();  // the barrier that ended the last tile freed the LDS chunk
+                    __syncthreads();
+                }
+            }
+            cur = nxt;
+        }
+        if (tid == 0) atomicAdd(args.tiles_swept, (unsigned long long)swept);
+        // Final ordering and output, every wave for its own 32 queries.
+        for (int b = 0; b < 32; ++b) {
+            const int ql = wave * 32 + b;
+            const int qq = q0 + ql;
+            if (qq >= N) break;
+            const int n = wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
+            const size_t row = (size_t)qi * kMQ + ql;
+            if (P == 1) {
+                for (int e = lane; e < want; e += kWave)
+                    cand[row * want + e] = e < n ? key_index(list[(size_t)ql * cap + e]) : -1;
+                if (lane == 0) tau[row] = thr[ql] == ~0ull ? INFINITY : key_distance(thr[ql]);
+            } else {
+                u64 *dst = args.part_keys + (row * P + part) * want;
+                for (int e = lane; e < want; e += kWave) dst[e] = e < n ? list[(size_t)ql * cap + e] : ~0ull;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        }
+        __syncthreads();  // before the next query tile re-initialises thr / cnt and the LDS chunk
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Merge of the parts of the chunked sweep: the `want` best keys of a query's parts * want, exactly what
+// a single list would have kept (every part kept its own `want` best), and their threshold.  One wave
+// per query row, four rows per workgroup.  Dynamic LDS: 4 x parts * want keys.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void knn_merge_parts_kernel(u64 *__restrict__ part_keys, int parts, int want,
+                                                              int n_rows, int *__restrict__ cand,
+                                                              float *__restrict__ tau) {
+    extern __shared__ u64 merge_buf[];
+    __shared__ unsigned int hist_all[4][kWave];
+    __shared__ u64 thr[4];
+    __shared__ int cnt[4];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + wave;
+    if (row >= n_rows) return;  // no workgroup barrier below
+    const int total = parts * want;
+    u64 *list = part_keys + (size_t)row * total;
+    if (lane == 0) {
+        thr[wave] = ~0ull;
+        cnt[wave] = total;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    // The filler keys sort last; a threshold with all distance bits set means "fewer than `want` candidates".
+    wave_select(list, want, &cnt[wave], &thr[wave], merge_buf + (size_t)wave * total, hist_all[wave], lane);
+    for (int e = lane; e < want; e += kWave) cand[(size_t)row * want + e] = key_index(list[e]);
+    if (lane == 0) tau[row] = (thr[wave] >> 32) == 0xffffffffull ? INFINITY : key_distance(thr[wave]);
+}
+
+// ---------------------------------------------------------------------------
 // Re-rank: canonical distances of a query's candidates, sort by (distance,
 // index), verify, write.  One wave per query, four queries per workgroup.
 // Dynamic LDS: 4 x sort_n keys.
@@ -740,21 +1050,57 @@ __global__ __launch_bounds__(256) void knn_rerank_kernel(const float *__restrict
                                                          const float *__restrict__ tau,
                                                          const float *__restrict__ max_norm,
                                                          int *__restrict__ out_idx, float *__restrict__ out_d,
-                                                         int *__restrict__ fail_count, int *__restrict__ fail_list) {
+                                                         int *__restrict__ fail_count, int *__restrict__ fail_list,
+                                                         const int *__restrict__ qtile_list, int qtile_first,
+                                                         int qtile_step, int n_slots) {
     extern __shared__ u64 keys_all[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int q = blockIdx.x * 4 + wave;
+    // Query slot w belongs to query tile qtile_list[w / kMQ], or first + (w / kMQ) step without a list
+    // (all queries: first 0, step 1).  cand holds `want` candidates per slot, tau one threshold.
+    const int w = blockIdx.x * 4 + wave;
+    const int wt = w < n_slots ? w / kMQ : 0;
+    const int q = (qtile_list ? qtile_list[wt] : qtile_first + wt * qtile_step) * kMQ + (w % kMQ);
     u64 *keys = keys_all + (size_t)wave * sort_n;
-    const bool live = q < N;
+    const bool live = w < n_slots && q < N;
     const float *xq = X + (size_t)(live ? q : 0) * D;
     for (int c = lane; c < sort_n; c += kWave) {
         u64 key = ~0ull;
         if (live && c < want) {
-            const int j = cand[(size_t)q * want + c];
+            const int j = cand[(size_t)w * want + c];
             if (j >= 0) {
                 const float *xj = X + (size_t)j * D;
                 float acc = 0.0f;
-                if ((D & 1) == 0 && (reinterpret_cast<uintptr_t>(X) & 7) == 0) {
+                if ((D & 3) == 0 && D >= 64 && (reinterpret_cast<uintptr_t>(X) & 15) == 0) {
+                    // Long rows, 16-byte aligned: 128 bytes of the candidate's row per lane and step, so that a
+                    // cache line is used whole by the load that fetches it (the lanes walk 64 different rows);
+                    // the same fma chain.
+                    const v4f *q4 = reinterpret_cast<const v4f *>(xq);
+                    const v4f *j4 = reinterpret_cast<const v4f *>(xj);
+                    const int n4 = D / 4;
+                    int d4 = 0;
+                    for (; d4 + 8 <= n4; d4 += 8) {
+                        v4f b[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) b[u] = j4[d4 + u];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) {
+                            const v4f a = q4[d4 + u];
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) {
+                                const float df = a[k] - b[u][k];
+                                acc = fmaf(df, df, acc);
+                            }
+                        }
+                    }
+                    for (; d4 < n4; ++d4) {
+                        const v4f a = q4[d4], b = j4[d4];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const float df = a[k] - b[k];
+                            acc = fmaf(df, df, acc);
+                        }
+                    }
+                } else if ((D & 1) == 0 && (reinterpret_cast<uintptr_t>(X) & 7) == 0) {
                     // rows are 8-byte aligned: two dimensions per load, the same fma chain
                     const float2 *q2 = reinterpret_cast<const float2 *>(xq);
                     const float2 *j2 = reinterpret_cast<const float2 *>(xj);
@@ -800,7 +1146,7 @@ __global__ __launch_bounds__(256) void knn_rerank_kernel(const float *__restrict
     // a relative error of (D + 2) 2^-24 of itself; a factor of four covers the matrix unit's
     // accumulation order and the rounding of the stored norms.
     const float kth = key_distance(keys[K - 2]);
-    const float t = tau[q];
+    const float t = tau[w];
     bool pass = isinf(t) && t > 0.0f;
     if (!pass) {
         const double nq = norms[q], nmax = *max_norm;
@@ -946,14 +1292,27 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     // Matrix-instruction sweep geometry.
     const int Dnorm = (D + 1) & ~1;        // |x|^2 row: first even row after the real dimensions
     int ksteps = (Dnorm + 2) / 2;          // k-steps incl. the augmented pair
-    if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
-    const int want = std::min(N - 1, (K - 1) + std::max(32, (K - 1) / 2));  // K' candidates kept per query
-    const int mcap = next_pow2(want + kCT) < 256 ? 256 : next_pow2(want + kCT);
+    const bool chunked = ksteps > kMfmaMaxSteps;  // more dimensions than one wave's registers hold
+    const int n_chunks = chunked ? div_up(ksteps, kChunkSteps) : 0;
+    if (chunked) ksteps = n_chunks * kChunkSteps;
+    else if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
     const int num_tiles = div_up(N, kCT);
     const int bitmap_words = div_up(num_tiles, 32);
-    const size_t mfma_lds = sizeof(float4) * 4 * ((ksteps + 3) / 4) * 64 + sizeof(u64) * 4 * mcap +
-                            sizeof(unsigned int) * bitmap_words;
-    const bool mfma_fits = ksteps <= kMfmaMaxSteps && mcap <= 4096 && mfma_lds <= 150 * 1024;
+    // Room for the candidates kept, as many again and one more tile where that fits: a list that is
+    // nearly full right after a selection would be selected again after every tile.
+    auto list_cap = [](int want) {
+        int cap = next_pow2(2 * want + kCT);
+        if (cap > 4096) cap = next_pow2(want + kCT);
+        return cap < 256 ? 256 : cap;
+    };
+    auto sweep_lds = [&](int want) -> size_t {
+        const size_t tile = chunked ? sizeof(float4) * kChunkFloat4 + sizeof(float) * D
+                                    : sizeof(float4) * 4 * ((ksteps + 3) / 4) * 64;
+        return tile + sizeof(u64) * 4 * list_cap(want) + sizeof(unsigned int) * bitmap_words;
+    };
+    auto sweep_fits = [&](int want) { return list_cap(want) <= 4096 && sweep_lds(want) <= 150 * 1024; };
+    int want = std::min(N - 1, (K - 1) + std::max(32, (K - 1) / 2));  // K' candidates kept per query
+    const bool mfma_fits = sweep_fits(want);
     bool use_mfma = mode == 2 || (mode == 0 && mfma_fits && N >= 8192);
     if (mode == 2 && !mfma_fits) {
         set_error("knn: the matrix-instruction sweep does not fit %d dimensions / %d neighbours", D, K);
@@ -979,12 +1338,11 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     }
 
     const int S4 = (ksteps + 3) / 4;
-    DeviceMem Xp, norms, lists, cand, tau, scal, fail_list, centers, radius;
+    DeviceMem Xp, Bp, norms, scal, fail_list, centers, radius;
     const int num_qtiles = div_up(N, kMQ);
-    const int grid = std::min(num_qtiles, cus * (ksteps <= 28 ? 3 : 2));
     if (!Xp.alloc(sizeof(float4) * (size_t)Npad * S4 * 2) || !norms.alloc(sizeof(float) * Npad) ||
-        !lists.alloc(sizeof(u64) * (size_t)grid * kMQ * mcap) || !cand.alloc(sizeof(int) * (size_t)N * want) ||
-        !tau.alloc(sizeof(float) * N) || !scal.alloc(4 * sizeof(int)) || !fail_list.alloc(sizeof(int) * N) ||
+        (chunked && !Bp.alloc(sizeof(float4) * (size_t)Npad * S4 * 2)) ||
+        !scal.alloc(4 * sizeof(int)) || !fail_list.alloc(sizeof(int) * N) ||
         !centers.alloc(sizeof(float) * (size_t)D * num_tiles) || !radius.alloc(sizeof(float) * num_tiles)) {
         set_error("knn: out of device memory for the candidate buffers");
         return 1;
@@ -993,44 +1351,151 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     norms_kernel<<<div_up(Npad, 256), 256, 0, s>>>(points, N, D, Npad, norms.as<float>(), scal.as<float>());
     TSNE_TRY(hipGetLastError());
     pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm, S4,
-                                                                          Npad, Xp.as<float4>());
+                                                                          Npad, Xp.as<float4>(), false);
     TSNE_TRY(hipGetLastError());
+    if (chunked) {
+        pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm,
+                                                                              S4, Npad, Bp.as<float4>(), true);
+        TSNE_TRY(hipGetLastError());
+    }
     tile_balls_kernel<<<num_tiles, 128, sizeof(float) * D, s>>>(points, N, D, num_tiles, centers.as<float>(),
                                                                radius.as<float>());
     TSNE_TRY(hipGetLastError());
-    SweepArgs args;
-    args.Xp = Xp.as<float4>();
-    args.N = N;
-    args.D = D;
-    args.Dnorm = Dnorm;
-    args.want = want;
-    args.cap = mcap;
-    args.lists = lists.as<u64>();
-    args.num_qtiles = num_qtiles;
-    args.cand = cand.as<int>();
-    args.tau = tau.as<float>();
-    args.norms = norms.as<float>();
-    args.centers_t = centers.as<float>();
-    args.radius = radius.as<float>();
-    args.bitmap_words = bitmap_words;
-    args.trigger = mcap - kCT;  // as late as possible: a later selection costs the same and sees more candidates
-    args.tiles_swept = reinterpret_cast<unsigned long long *>(scal.as<int>() + 2);
-    if (dispatch_mfma_sweep(ksteps, args, grid, s)) return 1;
-    const int sort_n = next_pow2(want) < 64 ? 64 : next_pow2(want);
-    knn_rerank_kernel<<<div_up(N, 4), 256, sizeof(u64) * 4 * sort_n, s>>>(
-        points, norms.as<float>(), N, D, K, want, sort_n, cand.as<int>(), tau.as<float>(), scal.as<float>(), indices,
-        sq_dist, scal.as<int>() + 1, fail_list.as<int>());
-    TSNE_TRY(hipGetLastError());
-    int host_scal[4] = {0, 0, 0, 0};
-    TSNE_TRY(hipMemcpyAsync(host_scal, scal.p, sizeof(host_scal), hipMemcpyDeviceToHost, s));
-    TSNE_TRY(hipStreamSynchronize(s));
-    const int failed = host_scal[1];
+
+    // Sweep + re-rank of `count` query tiles: those of tile_list (device), or first, first + step, ... without a
+    // list.  Keeps `keep` candidates per query and part.  failed = queries of those tiles whose verification
+    // failed (listed in fail_list), swept = tile pairs computed.
+    auto sweep_and_rerank = [&](int keep, const int *tile_list, int first, int step, int count, int &failed,
+                                unsigned long long &swept) -> int {
+        const int cap = list_cap(keep);
+        // One workgroup sweeps a query tile against all its candidate tiles, which takes long with hundreds
+        // of dimensions, and the tiles differ in how many candidate tiles they can skip: unless there are
+        // several query tiles per workgroup slot to even that out, the chunked kernel splits every tile's
+        // candidates over up to 8 workgroups.
+        const int slots = cus * (!chunked && ksteps <= 28 ? 3 : 2);
+        int parts = 1;
+        if (chunked)
+            while (parts < 8 && count * parts < 3 * slots && parts * 2 * keep <= 2048) parts *= 2;
+        const int grid = std::min(count * parts, slots);
+        const size_t n_slots = (size_t)(tile_list || step != 1 ? count * kMQ : N);
+        DeviceMem lists, cand, tau, part_keys;
+        if (!lists.alloc(sizeof(u64) * (size_t)grid * kMQ * cap) || !cand.alloc(sizeof(int) * n_slots * keep) ||
+            !tau.alloc(sizeof(float) * n_slots) ||
+            (parts > 1 && !part_keys.alloc(sizeof(u64) * n_slots * parts * keep))) {
+            set_error("knn: out of device memory for the candidate lists");
+            return 1;
+        }
+        TSNE_TRY(hipMemsetAsync(scal.as<int>() + 1, 0, 3 * sizeof(int), s));
+        SweepArgs args;
+        args.Xp = Xp.as<float4>();
+        args.N = N;
+        args.D = D;
+        args.Dnorm = Dnorm;
+        args.want = keep;
+        args.cap = cap;
+        args.lists = lists.as<u64>();
+        args.num_qtiles = count;
+        args.cand = cand.as<int>();
+        args.tau = tau.as<float>();
+        args.norms = norms.as<float>();
+        args.centers_t = centers.as<float>();
+        args.radius = radius.as<float>();
+        args.bitmap_words = bitmap_words;
+        args.trigger = cap - kCT;  // as late as possible: a later selection costs the same and sees more candidates
+        args.tiles_swept = reinterpret_cast<unsigned long long *>(scal.as<int>() + 2);
+        args.Bp = Bp.as<float4>();
+        args.n_chunks = n_chunks;
+        args.qtile_list = tile_list;
+        args.qtile_first = first;
+        args.qtile_step = step;
+        args.parts = parts;
+        args.part_keys = part_keys.as<u64>();
+        if (chunked) {
+            const size_t lds = sweep_lds(keep);
+            TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_chunked_sweep_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            knn_mfma_chunked_sweep_kernel<<<grid, 256, lds, s>>>(args);
+            TSNE_TRY(hipGetLastError());
+        } else if (dispatch_mfma_sweep(ksteps, args, grid, s)) {
+            return 1;
+        }
+        if (parts > 1) {
+            // rows of a partial last tile are merged too: the sweep left them unwritten, the re-rank skips them
+            const size_t lds = sizeof(u64) * 4 * parts * keep;
+            TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_merge_parts_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            knn_merge_parts_kernel<<<div_up((int)n_slots, 4), 256, lds, s>>>(part_keys.as<u64>(), parts, keep,
+                                                                            (int)n_slots, cand.as<int>(),
+                                                                            tau.as<float>());
+            TSNE_TRY(hipGetLastError());
+        }
+        const int sort_n = next_pow2(keep) < 64 ? 64 : next_pow2(keep);
+        TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_rerank_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)(sizeof(u64) * 4 * sort_n)));
+        knn_rerank_kernel<<<div_up((int)n_slots, 4), 256, sizeof(u64) * 4 * sort_n, s>>>(
+            points, norms.as<float>(), N, D, K, keep, sort_n, cand.as<int>(), tau.as<float>(), scal.as<float>(),
+            indices, sq_dist, scal.as<int>() + 1, fail_list.as<int>(), tile_list, first, step, (int)n_slots);
+        TSNE_TRY(hipGetLastError());
+        int host_scal[4] = {0, 0, 0, 0};
+        TSNE_TRY(hipMemcpyAsync(host_scal, scal.p, sizeof(host_scal), hipMemcpyDeviceToHost, s));
+        TSNE_TRY(hipStreamSynchronize(s));
+        failed = host_scal[1];
+        std::memcpy(&swept, host_scal + 2, sizeof(swept));
+        return 0;
+    };
+
+    int failed = 0;
+    unsigned long long swept = 0;
+    // The verification needs the distance gap between neighbour K and candidate K' to exceed the rounding
+    // bound of the approximate distances, which grows with the dimension count and with the points'
+    // distance from the origin.  With many dimensions the neighbour distances of a query lie close
+    // together, so the chunked sweep first tries its margin on a sample of query tiles and doubles K'
+    // while more than a tenth of the sample fails; data that no margin verifies goes to the vector sweep.
+    if (chunked && num_qtiles >= 64) {
+        const int sample_tiles = 16, step = num_qtiles / sample_tiles;
+        bool verified = false;
+        for (int attempt = 0; attempt < 3 && !verified; ++attempt) {
+            if (sweep_and_rerank(want, nullptr, step / 2, step, sample_tiles, failed, swept)) return 1;
+            if (failed * 10 <= sample_tiles * kMQ) {
+                verified = true;
+            } else {
+                const int wider = std::min(N - 1, 2 * want);
+                if (wider == want || !sweep_fits(wider)) break;
+                want = wider;
+            }
+        }
+        if (!verified && mode == 0) {
+            if (build_transposed()) return 1;
+            return run_valu_sweep(points, Xt.as<float>(), N, Npad, D, K, nullptr, N, cus, indices, sq_dist, s);
+        }
+    }
+    if (sweep_and_rerank(want, nullptr, 0, 1, num_qtiles, failed, swept)) return 1;
     if (stats) {
         stats[0] = 1;
         stats[1] = failed;
-        unsigned long long swept = 0;
-        std::memcpy(&swept, host_scal + 2, sizeof(swept));
         stats[2] = (int)((1000.0 * (double)swept) / ((double)num_tiles * (double)num_tiles) + 0.5);
+    }
+    // The chunked sweep takes the tiles of the few queries that failed once more with twice the margin
+    // (a vector sweep of one query tile over all points in hundreds of dimensions takes as long as the
+    // whole matrix sweep); what fails again, and every failure of the register-resident sweep, goes to
+    // the vector sweep.
+    if (failed > 0 && chunked && failed * 10 <= N) {
+        const int wider = std::min(N - 1, 2 * want);
+        if (wider != want && sweep_fits(wider)) {
+            std::vector<int> queries(failed), tiles;
+            TSNE_TRY(hipMemcpy(queries.data(), fail_list.p, sizeof(int) * (size_t)failed, hipMemcpyDeviceToHost));
+            for (int q : queries) tiles.push_back(q / kMQ);
+            std::sort(tiles.begin(), tiles.end());
+            tiles.erase(std::unique(tiles.begin(), tiles.end()), tiles.end());
+            DeviceMem tile_list;
+            if (!tile_list.alloc(sizeof(int) * tiles.size())) {
+                set_error("knn: out of device memory for the retry list");
+                return 1;
+            }
+            TSNE_TRY(hipMemcpy(tile_list.p, tiles.data(), sizeof(int) * tiles.size(), hipMemcpyHostToDevice));
+            unsigned long long swept_again = 0;
+            if (sweep_and_rerank(wider, tile_list.as<int>(), 0, 1, (int)tiles.size(), failed, swept_again)) return 1;
+        }
     }
     if (failed > 0) {
         if (build_transposed()) return 1;
