@@ -372,6 +372,7 @@ def test_iterate_with_prepared_pattern(stages, c0_problem):
     (2200, 190, 40),   # 3 chunks, the last one full but for the norm row's partner
     (1200, 784, 50),   # config c1's dimension count (13 chunks)
     (900, 1024, 30),   # config c2's (17 chunks: the norm row has a chunk of its own)
+    (745, 864, 126),   # six candidate tiles: fewer than the workgroups a query tile could be split over
     (40, 3, 40),       # K == N, a single partial tile
     (2500, 33, 300),   # wide neighbour lists
 ])

@@ -201,12 +201,21 @@ __device__ __forceinline__ int wave_select(u64 *list, int want, int *cnt, u64 *t
     const int n = *cnt;
     if (n < want) return n;
     unsigned int lo = ~0u, hi = 0u;
-    for (int e = lane; e < n; e += kWave) {
-        const u64 key = list[e];
-        buf[e] = key;
-        const unsigned int bits = (unsigned int)(key >> 32);
-        lo = min(lo, bits);
-        hi = max(hi, bits);
+    // Four loads in flight: the list comes from global memory and a load at a time would cost its latency each.
+    for (int e0 = lane; e0 < n; e0 += 4 * kWave) {
+        u64 key[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) key[u] = list[min(e0 + u * kWave, n - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = e0 + u * kWave;
+            if (e < n) {
+                buf[e] = key[u];
+                const unsigned int bits = (unsigned int)(key[u] >> 32);
+                lo = min(lo, bits);
+                hi = max(hi, bits);
+            }
+        }
     }
 #pragma unroll
     for (int m = kWave / 2; m > 0; m >>= 1) {
@@ -309,6 +318,31 @@ __device__ __forceinline__ bool tile_may_matter(const float *qcenter, float ra, 
         d2 = fmaf(diff, diff, d2);
     }
     const float lb = sqrtf(d2) * (1.0f - 1e-3f) - (ra + radius[t]);
+    return !(lb > 0.0f && lb * lb > tmax);
+}
+
+// The same test for hundreds of dimensions: eight loads in flight and two partial sums (any summation
+// order will do, the slack covers the rounding).
+__device__ __forceinline__ bool tile_may_matter_wide(const float *qcenter, float ra, const float *__restrict__ centers_t,
+                                                     const float *__restrict__ radius, int D, int T, int t, float tmax) {
+    float s0 = 0.0f, s1 = 0.0f;
+    int d = 0;
+    for (; d + 8 <= D; d += 8) {
+        float c[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) c[u] = centers_t[(size_t)(d + u) * T + t];
+#pragma unroll
+        for (int u = 0; u < 8; u += 2) {
+            const float e0 = qcenter[d + u] - c[u], e1 = qcenter[d + u + 1] - c[u + 1];
+            s0 = fmaf(e0, e0, s0);
+            s1 = fmaf(e1, e1, s1);
+        }
+    }
+    for (; d < D; ++d) {
+        const float diff = qcenter[d] - centers_t[(size_t)d * T + t];
+        s0 = fmaf(diff, diff, s0);
+    }
+    const float lb = sqrtf(s0 + s1) * (1.0f - 1e-3f) - (ra + radius[t]);
     return !(lb > 0.0f && lb * lb > tmax);
 }
 
@@ -941,9 +975,10 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
             return word_idx * 32 + b;
         };
         int cur = h0 + (part - h0 % P + P) % P;  // this part's first tile of the neighbourhood
-        fetch(cur, 0);
+        if (cur > h1) cur = -1;  // fewer tiles than parts: nothing for this part, its lists stay empty
+        if (cur >= 0) fetch(cur, 0);
         __syncthreads();  // the previous query tile's last reads of the LDS chunk
-        stash();
+        if (cur >= 0) stash();
         __syncthreads();
         bool home = true;
         unsigned int swept = 0;
@@ -977,7 +1012,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                 const float ra = args.radius[qt];
                 for (int t = tid; t < T; t += 256)
                     if ((t < h0 || t > h1) && t % P == part &&
-                        tile_may_matter(qcenter, ra, args.centers_t, args.radius, D, T, t, tmax))
+                        tile_may_matter_wide(qcenter, ra, args.centers_t, args.radius, D, T, t, tmax))
                         atomicOr(&bitmap[t >> 5], 1u << (t & 31));
                 __syncthreads();
                 nxt = next_tile();
@@ -1375,7 +1410,8 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         const int slots = cus * (!chunked && ksteps <= 28 ? 3 : 2);
         int parts = 1;
         if (chunked)
-            while (parts < 8 && count * parts < 3 * slots && parts * 2 * keep <= 2048) parts *= 2;
+            while (parts < 8 && count * parts < 3 * slots && parts * 2 * keep <= 2048 && parts * 2 <= num_tiles)
+                parts *= 2;
         const int grid = std::min(count * parts, slots);
         const size_t n_slots = (size_t)(tile_list || step != 1 ? count * kMQ : N);
         DeviceMem lists, cand, tau, part_keys;
