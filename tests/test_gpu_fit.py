@@ -120,7 +120,8 @@ def test_renumbering_is_invisible_to_the_caller(monkeypatch):
     (16385, 7, 30, 3),    # just above the renumbering threshold, odd count (scalar update kernel)
     (20001, 3, 90, 1),    # one blob: nothing for the kNN sweep to skip
     (8192, 126, 16, 4),   # smallest matrix-sweep problem, largest matrix-sweep dimension
-    (8195, 127, 16, 4),   # one dimension more: vector sweep
+    (8195, 127, 16, 4),   # one dimension more: chunked matrix sweep
+    (17000, 300, 30, 5),  # chunked matrix sweep on renumbered points, margin tried on a sample of query tiles
     (40000, 50, 40, 6),   # several column partitions and strips, clustered
 ])
 def test_whole_pipeline_against_the_oracle(n, d, k, clusters):
