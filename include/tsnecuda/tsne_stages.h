@@ -46,10 +46,12 @@ int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neig
 
 /* tsne_hip_knn with an explicit choice of the distance sweep: 0 = choose by
  * shape (what tsne_hip_knn does), 1 = vector-ALU sweep, 2 = matrix-instruction
- * (MFMA) candidate sweep followed by an exact re-rank and verification (at most
- * 126 dimensions).  Results are identical whichever sweep runs.  stats (host
- * pointer to three ints, may be NULL): [0] = 1 if the matrix sweep ran,
- * [1] = queries the verification sent back to the vector sweep, [2] = per
+ * (MFMA) candidate sweep followed by an exact re-rank and verification (up to
+ * 126 dimensions the queries stay in registers; beyond, both operands stream in
+ * chunks of 64 dimensions).  Results are identical whichever sweep runs.  stats
+ * (host pointer to three ints, may be NULL): [0] = 1 if the matrix sweep ran,
+ * [1] = queries that failed the verification of the sweep over all query tiles
+ * (they are swept again with a wider margin or by the vector sweep), [2] = per
  * mille of the (query tile, candidate tile) pairs the matrix sweep computed (it
  * skips candidate tiles whose bounding ball lies beyond every threshold of the
  * query tile, which pays on locality-ordered points).  Same reference
