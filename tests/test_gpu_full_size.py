@@ -104,3 +104,27 @@ def test_forces_and_fused_steps(c3):
     y_o, _ = oracle.iterate(P_h, idx_h, y_h, 3, step_begin=60, eta=200.0, gains=gains_h, old_forces=old_h)
     assert rel_l2(y.cpu().numpy(), y_o) <= 1e-4
     plan.close()
+
+
+def test_blocked_attractive_with_more_than_1024_column_partitions():
+    """4.5 M points are 1099 column partitions of 4096: the re-blocking's scans
+    give every thread several partition slots.  A pattern without any locality
+    (every strip references every partition, most runs far shorter than a work
+    item) against the row-ordered kernel and, on its first and last rows, the
+    oracle."""
+    from tsnecuda import stages
+    n, k = 4500000, 6
+    g = torch.Generator(device="cuda").manual_seed(1)
+    idx = torch.randint(0, n, (n, k), generator=g, device="cuda", dtype=torch.int32)
+    idx[:, 0] = torch.arange(n, device="cuda", dtype=torch.int32)
+    P = torch.rand((n, k), generator=g, device="cuda", dtype=torch.float32) * 1e-6
+    P[:, 0] = 0.0
+    y = torch.randn(2 * n, generator=g, device="cuda", dtype=torch.float32) * 20.0
+    plan = stages.Plan(n, k)
+    plan.prepare_attractive(P, idx)
+    blocked = plan.attractive(None, None, y)
+    by_rows = plan.attractive(P, idx, y)
+    assert rel_l2(blocked.cpu().numpy(), by_rows.cpu().numpy()) <= 1e-6
+    want = oracle.attractive(P.cpu().numpy(), idx.cpu().numpy(), y.cpu().numpy())
+    assert rel_l2(blocked.cpu().numpy(), want) <= 1e-4
+    plan.close()

@@ -42,8 +42,7 @@ constexpr int kStripMax = 3968;     // rows per strip: 31 KB of positions + 62 K
                                     // repulsive chain that run beside this one
 constexpr double kRoundMagic = 6755399441055744.0;  // 1.5 * 2^52: adding it rounds a double to an integer
 constexpr int kBlock = 1024;
-constexpr int kMaxParts = 1024;
-static_assert(kBlock == kMaxParts, "the partition scan uses one thread per slot");
+constexpr int kMaxParts = 4096;     // column partitions: up to 16.7 M points
 constexpr int kPrefetch = 4;        // entries per thread in one work item
 constexpr int kStreamThreads = 768; // force kernel: waves 0-11 stream entries ...
 constexpr int kLoadThreads = kBlock - kStreamThreads;  // ... waves 12-15 stage the partitions
@@ -53,14 +52,45 @@ constexpr int kPadItems = 4;        // empty records after a strip's last item: 
 // ---------------------------------------------------------------------------
 // Re-blocking: one workgroup per strip.  Histogram of the strip's entries over
 // the partitions, exclusive scan, then a scatter that ranks entries inside a
-// partition with LDS atomics.
+// partition with LDS atomics.  A thread owns kSlotsPerThread consecutive
+// partition slots in the scans.
 // ---------------------------------------------------------------------------
+constexpr int kSlotsPerThread = kMaxParts / kBlock;
+static_assert(kMaxParts % kBlock == 0, "the partition scans give every thread the same number of slots");
+
+// Exclusive prefix sums over all kMaxParts slots (thread t holds slots t * kSlotsPerThread ...); returns the
+// total.  scan: kBlock words of LDS.  Ends with the LDS array free for reuse.
+__device__ __forceinline__ unsigned int scan_slots(const unsigned int (&value)[kSlotsPerThread],
+                                                   unsigned int (&before)[kSlotsPerThread], unsigned int *scan,
+                                                   int tid) {
+    unsigned int mine = 0u;
+#pragma unroll
+    for (int i = 0; i < kSlotsPerThread; ++i) {
+        before[i] = mine;
+        mine += value[i];
+    }
+    scan[tid] = mine;
+    __syncthreads();
+    for (int off = 1; off < kBlock; off <<= 1) {  // inclusive Hillis-Steele scan of the per-thread sums
+        const unsigned int add = tid >= off ? scan[tid - off] : 0u;
+        __syncthreads();
+        scan[tid] += add;
+        __syncthreads();
+    }
+    const unsigned int base = scan[tid] - mine;
+    const unsigned int total = scan[kBlock - 1];
+#pragma unroll
+    for (int i = 0; i < kSlotsPerThread; ++i) before[i] += base;
+    __syncthreads();
+    return total;
+}
+
 __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
                                                          int N, int K, int strip_rows, int max_items,
                                                          int seg_stride, float *__restrict__ ent_p,
                                                          unsigned int *__restrict__ seg, float *__restrict__ p_max) {
     __shared__ unsigned int cursor[kMaxParts];
-    __shared__ unsigned int scan[kMaxParts];
+    __shared__ unsigned int scan[kBlock];
     const int tid = threadIdx.x;
     const int strip = blockIdx.x;
     const int row0 = strip * strip_rows;
@@ -71,57 +101,42 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
     __syncthreads();
     for (unsigned int e = tid; e < count; e += kBlock) atomicAdd(&cursor[idx[base + e] / kPartPoints], 1u);
     __syncthreads();
-    // Inclusive Hillis-Steele scan over kMaxParts == kBlock slots.
-    unsigned int mine = cursor[tid];
-    scan[tid] = mine;
-    __syncthreads();
-    for (int off = 1; off < kMaxParts; off <<= 1) {
-        const unsigned int add = tid >= off ? scan[tid - off] : 0u;
-        __syncthreads();
-        scan[tid] += add;
-        __syncthreads();
-    }
-    const unsigned int first = scan[tid] - mine;
-    cursor[tid] = first;
-    __syncthreads();
+    unsigned int mine[kSlotsPerThread], first[kSlotsPerThread];
+#pragma unroll
+    for (int i = 0; i < kSlotsPerThread; ++i) mine[i] = cursor[tid * kSlotsPerThread + i];
+    scan_slots(mine, first, scan, tid);
+#pragma unroll
+    for (int i = 0; i < kSlotsPerThread; ++i) cursor[tid * kSlotsPerThread + i] = first[i];
     // Work list of the strip: every referenced partition contributes ceil(entries / kItemEntries) items
     // (runs of at most kItemEntries entries that share the partition); a second scan, over the item counts.
-    const unsigned int items = (mine + kItemEntries - 1u) / kItemEntries;
-    scan[tid] = items;
-    __syncthreads();
-    for (int off = 1; off < kMaxParts; off <<= 1) {
-        const unsigned int add = tid >= off ? scan[tid - off] : 0u;
-        __syncthreads();
-        scan[tid] += add;
-        __syncthreads();
-    }
+    unsigned int items[kSlotsPerThread], item_slot[kSlotsPerThread];
+#pragma unroll
+    for (int i = 0; i < kSlotsPerThread; ++i) items[i] = (mine[i] + kItemEntries - 1u) / kItemEntries;
+    const unsigned int n_items_total = scan_slots(items, item_slot, scan, tid);
     // Layout of a strip's list: {item count, fresh count, -, -}, then one record per item
     // {first entry, end entry, partition, 1 if the item opens the partition}, kPadItems empty records,
     // then the partitions in the order they are opened.
     unsigned int *hdr = seg + (size_t)strip * seg_stride;
     uint4 *records = reinterpret_cast<uint4 *>(hdr + 4);
     unsigned int *fresh_parts = hdr + 4 + 4 * (max_items + kPadItems);
-    for (unsigned int it = 0; it < items; ++it) {
-        const unsigned int slot = scan[tid] - items + it;
-        const unsigned int b = first + it * kItemEntries;
-        records[slot] = make_uint4(b, min(first + mine, b + kItemEntries), (unsigned int)tid, it == 0 ? 1u : 0u);
-    }
-    const unsigned int n_items_total = scan[kMaxParts - 1];
+#pragma unroll
+    for (int i = 0; i < kSlotsPerThread; ++i)
+        for (unsigned int it = 0; it < items[i]; ++it) {
+            const unsigned int b = first[i] + it * kItemEntries;
+            records[item_slot[i] + it] = make_uint4(b, min(first[i] + mine[i], b + kItemEntries),
+                                                    (unsigned int)(tid * kSlotsPerThread + i), it == 0 ? 1u : 0u);
+        }
     if (tid < kPadItems) records[n_items_total + tid] = make_uint4(count, count, 0u, 0u);
     if (tid == 0) hdr[0] = n_items_total;
-    __syncthreads();
     // Third scan, over the "referenced at all" flags: the order in which partitions are opened.
-    const unsigned int flag = mine > 0u ? 1u : 0u;
-    scan[tid] = flag;
-    __syncthreads();
-    for (int off = 1; off < kMaxParts; off <<= 1) {
-        const unsigned int add = tid >= off ? scan[tid - off] : 0u;
-        __syncthreads();
-        scan[tid] += add;
-        __syncthreads();
-    }
-    if (flag) fresh_parts[scan[tid] - 1u] = (unsigned int)tid;
-    if (tid == kMaxParts - 1) hdr[1] = scan[tid];
+    unsigned int flag[kSlotsPerThread], order[kSlotsPerThread];
+#pragma unroll
+    for (int i = 0; i < kSlotsPerThread; ++i) flag[i] = mine[i] > 0u ? 1u : 0u;
+    const unsigned int n_fresh = scan_slots(flag, order, scan, tid);
+#pragma unroll
+    for (int i = 0; i < kSlotsPerThread; ++i)
+        if (flag[i]) fresh_parts[order[i]] = (unsigned int)(tid * kSlotsPerThread + i);
+    if (tid == 0) hdr[1] = n_fresh;
     // Entries are visited neighbour slot by neighbour slot, so that neighbouring positions of a
     // partition's run belong to different rows: a wave of the force kernel then spreads its LDS
     // atomics over many accumulators even when most neighbours of a row share one partition.
