@@ -79,7 +79,7 @@ def main():
     order, order_s = timed(lambda: stages.locality_order(dX))
     dXs, gather_s = timed(lambda: stages.gather_rows(dX, order))
     del dX
-    (idx, d2), knn_s = timed(lambda: stages.knn(dXs, k))
+    (idx, d2, knn_stats), knn_s = timed(lambda: stages.knn_select(dXs, k, 0))  # 0: what tsne_hip_knn does
     del dXs
     order_h = order.cpu().numpy().astype(np.int64)
     y0 = np.concatenate([y0[:n][order_h], y0[n:][order_h]])
@@ -110,6 +110,35 @@ def main():
     attr_ms = kernels_us["attractive_kernel"] * 1e-3  # profiling slot of whichever attractive kernel ran
     attr_bytes = 8.0 * n * k + 16.0 * n  # P and index streams; read positions, write forces
     achieved = attr_bytes / (attr_ms * 1e-3) / 1e9
+
+    # ---- every phase against its roofline -----------------------------------
+    # Algorithmic bytes per launch of the loop's kernels (G = 390 interpolation nodes per side, four charge
+    # planes; the transposed spectra are 2 plane pairs x 1024 x 512 complex).
+    G2, spectra = 390.0 * 390.0, 2 * 1024 * 512 * 8.0
+    loop_bytes = {
+        "tile_count_kernel": 8.0 * n,                       # positions in
+        "tile_scatter_kernel": 16.0 * n,                    # positions in, positions grouped by tile out
+        "spread_kernel": 8.0 * n + 16.0 * G2,               # grouped positions in, node charges out
+        "conv_rows_forward_kernel": 16.0 * G2 + spectra,    # node charges in, row spectra out
+        "conv_columns_kernel": 2.0 * spectra,               # row spectra in, convolved columns out
+        "conv_rows_inverse_kernel": spectra + 16.0 * G2,    # in, node potentials out
+        "gather_forces_kernel": 16.0 * n + 16.0 * G2,       # positions and node potentials in, forces out
+        "attractive_kernel": attr_bytes,
+        "update_kernel": 72.0 * n,                          # 5 arrays of 2N in, 4 out (incl. the packed copy)
+    }
+    phase_rooflines = {
+        name: {"bound": "hbm", "bytes": b, "achieved": b / (kernels_us[name] * 1e-6) / 1e9, "unit": "GB/s",
+               "frac": b / (kernels_us[name] * 1e-6) / 1e9 / HBM_PEAK_GBS}
+        for name, b in loop_bytes.items() if kernels_us.get(name)}
+    if knn_stats[0] == 1:
+        # Flop the matrix sweep executed: 2 x 128 x 128 x (padded dimensions) per tile pair it did not skip.
+        ksteps = (((d + 1) & ~1) + 2) // 2
+        ksteps = -(-ksteps // 32) * 32 if ksteps > 64 else (-(-ksteps // 4) * 4 if ksteps > 32 else ksteps)
+        tiles = -(-n // 128)
+        flop = 2.0 * 128 * 128 * (2 * ksteps) * tiles * tiles * knn_stats[2] / 1000.0
+        phase_rooflines["knn"] = {"bound": "mfma", "flop": flop, "achieved": flop / knn_s / 1e12, "unit": "TFLOP/s",
+                                  "frac": flop / knn_s / 1e12 / 157.3, "tile_pairs_per_mille": knn_stats[2],
+                                  "note": "fp32 matrix peak; time of the whole kNN call (sweep, re-rank, packing)"}
 
     if args.calibrate:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda").normal_()
@@ -182,6 +211,7 @@ def main():
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "bytes_per_launch": attr_bytes, "ms_per_launch": attr_ms},
         "kernels_us": kernels_us,
+        "phase_rooflines": phase_rooflines,
         "cpu_baseline": cpu,
         "final_Z": float(z.item()),
     }

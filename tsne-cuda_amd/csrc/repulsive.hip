@@ -359,7 +359,7 @@ __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__
                                                      const int *__restrict__ num_chunks, const LoopScalars *sc,
                                                      int slot, int n_boxes, LagrangeConsts lc,
                                                      float *__restrict__ w) {
-    constexpr int kTileNodes = kTileBoxes * kInterp;  // 30
+    constexpr int kTileNodes = kTileBoxes * kInterp;  // 21
     __shared__ unsigned long long acc[kTileNodes * kTileNodes * kTerms];
     if ((int)blockIdx.x >= *num_chunks) return;
     const int4 ch = chunks[blockIdx.x];
