@@ -56,6 +56,7 @@ struct tsne_hip_plan {
     int4 *chunks = nullptr;        // (tile, first point, count, -) per spreading workgroup
     int *num_chunks = nullptr;  // [0] chunks of the current step, [1] ticket counter of the tile count kernel
     int max_chunks = 0;
+    int spread_grid = 512;         // workgroups of the spreading kernel (two per CU)
     float4 *node_charges = nullptr;     // n_nodes^2, one float4 (4 terms) per node
     float4 *node_potentials = nullptr;  // n_nodes^2
     float2 *row_spectra = nullptr;      // 2 plane pairs x kFft x kNodePad (transposed)

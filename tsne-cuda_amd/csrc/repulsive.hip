@@ -352,56 +352,104 @@ __device__ __forceinline__ void add_fixed(unsigned long long *dst, float v, doub
 
 // LDS float atomic adds cost ~190 clocks per wave instruction on gfx950 while
 // 64-bit integer LDS atomics are about 25x faster, so the private tile is kept
-// in 64-bit fixed point (which also makes a chunk's sums independent of the
-// order of the additions) and converted to fp32 when it is flushed.
+// in 64-bit fixed point (which also makes the sums independent of the order of
+// the additions) and converted to fp32 when it is flushed.
+//
+// A workgroup takes a contiguous range of the chunk list (the chunks are in tile
+// order): while it spreads one chunk the points of the next are already on their
+// way, consecutive chunks of one tile share the LDS tile, and the tile goes to
+// global memory (float atomics: neighbouring workgroups may hold parts of the same
+// tile) when the tile changes, after kChunksPerFlush chunks (the fixed-point sums
+// have room for 8192 contributions per node), and at the end of the range.
+constexpr int kChunksPerFlush = 4;
+static_assert(kChunkPoints == 2 * kSpreadThreads, "a thread spreads two points of a chunk");
+static_assert(kChunksPerFlush * kChunkPoints <= 4096, "a node's fixed-point sum must stay below 2^62");
+
 __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__restrict__ tile_xy,
                                                      const int4 *__restrict__ chunks,
                                                      const int *__restrict__ num_chunks, const LoopScalars *sc,
                                                      int slot, int n_boxes, LagrangeConsts lc,
                                                      float *__restrict__ w) {
     constexpr int kTileNodes = kTileBoxes * kInterp;  // 21
-    __shared__ unsigned long long acc[kTileNodes * kTileNodes * kTerms];
-    if ((int)blockIdx.x >= *num_chunks) return;
-    const int4 ch = chunks[blockIdx.x];
+    constexpr int kPlane = kTileNodes * kTileNodes;
+    __shared__ unsigned long long acc[kTerms * kPlane];
+    const int nc = *num_chunks;
+    const int c0 = (int)((long long)blockIdx.x * nc / gridDim.x);
+    const int c1 = (int)((long long)(blockIdx.x + 1) * nc / gridDim.x);
+    if (c0 >= c1) return;
+    const int tid = threadIdx.x;
+    for (int e = tid; e < kTerms * kPlane; e += kSpreadThreads) acc[e] = 0ull;
     const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
-    const int bx0 = (ch.x % tiles_per_dim) * kTileBoxes;
-    const int by0 = (ch.x / tiles_per_dim) * kTileBoxes;
-    for (int e = threadIdx.x; e < kTileNodes * kTileNodes * kTerms; e += kSpreadThreads) acc[e] = 0ull;
-    __syncthreads();
+    const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
     const SpreadScales fx = spread_scales(sc, slot);
-    for (int p = threadIdx.x; p < ch.z; p += kSpreadThreads) {
-        const float2 pt = tile_xy[ch.y + p];
-        const float x = pt.x, y = pt.y;
-        int bx, by;
-        float Lx[kInterp], Ly[kInterp];
-        bin_and_weights(x, bd, n_boxes, lc, bx, Lx);
-        bin_and_weights(y, bd, n_boxes, lc, by, Ly);
-        const float q3 = x * x + y * y;
-        const int nx = (bx - bx0) * kInterp, ny = (by - by0) * kInterp;
+    // Unconditional, clamped loads: a chunk holds at least one point.
+    auto fetch = [&](const int4 &ch, float2 (&pt)[2]) {
 #pragma unroll
-        for (int a = 0; a < kInterp; ++a) {
+        for (int u = 0; u < 2; ++u) pt[u] = tile_xy[ch.y + min(tid + u * kSpreadThreads, ch.z - 1)];
+    };
+    int4 ch = chunks[c0];
+    float2 pt[2];
+    fetch(ch, pt);
+    __syncthreads();  // the tile is zero
+    int cur_tile = ch.x, in_tile = 0;
+    for (int c = c0; c < c1; ++c) {
+        const bool last = c + 1 == c1;
+        int4 next_ch = ch;
+        float2 next_pt[2] = {pt[0], pt[1]};
+        if (!last) {
+            next_ch = chunks[c + 1];
+            fetch(next_ch, next_pt);
+        }
+        const int bx0 = (cur_tile % tiles_per_dim) * kTileBoxes;
+        const int by0 = (cur_tile / tiles_per_dim) * kTileBoxes;
 #pragma unroll
-            for (int b = 0; b < kInterp; ++b) {
-                const float lw = Lx[a] * Ly[b];
-                unsigned long long *dst = acc + ((nx + a) * kTileNodes + (ny + b)) * kTerms;
-                add_fixed(dst + 0, lw, fx.to_fixed[0]);
-                add_fixed(dst + 1, lw * x, fx.to_fixed[1]);
-                add_fixed(dst + 2, lw * y, fx.to_fixed[2]);
-                add_fixed(dst + 3, lw * q3, fx.to_fixed[3]);
+        for (int u = 0; u < 2; ++u) {
+            if (tid + u * kSpreadThreads < ch.z) {
+                const float x = pt[u].x, y = pt[u].y;
+                int bx, by;
+                float Lx[kInterp], Ly[kInterp];
+                bin_and_weights(x, bd, n_boxes, lc, bx, Lx);
+                bin_and_weights(y, bd, n_boxes, lc, by, Ly);
+                const float q3 = x * x + y * y;
+                const int nx = (bx - bx0) * kInterp, ny = (by - by0) * kInterp;
+#pragma unroll
+                for (int a = 0; a < kInterp; ++a) {
+#pragma unroll
+                    for (int b = 0; b < kInterp; ++b) {
+                        const float lw = Lx[a] * Ly[b];
+                        // One plane per term: the lanes of an atomic instruction all add to the same term, and
+                        // with the four terms of a node side by side they would only ever meet an eighth of the
+                        // LDS banks.
+                        unsigned long long *dst = acc + (nx + a) * kTileNodes + (ny + b);
+                        add_fixed(dst + 0 * kPlane, lw, fx.to_fixed[0]);
+                        add_fixed(dst + 1 * kPlane, lw * x, fx.to_fixed[1]);
+                        add_fixed(dst + 2 * kPlane, lw * y, fx.to_fixed[2]);
+                        add_fixed(dst + 3 * kPlane, lw * q3, fx.to_fixed[3]);
+                    }
+                }
             }
         }
-    }
-    __syncthreads();
-    const int G = n_boxes * kInterp;
-    for (int e = threadIdx.x; e < kTileNodes * kTileNodes * kTerms; e += kSpreadThreads) {
-        const long long v = (long long)acc[e];
-        if (v != 0) {
-            const int node = e / kTerms, t = e % kTerms;
-            const int gx = bx0 * kInterp + node / kTileNodes, gy = by0 * kInterp + node % kTileNodes;
-            if (gx < G && gy < G)
-                atomicAdd(w + ((size_t)gx * G + gy) * kTerms + t, (float)((double)v * fx.from_fixed[t]));
+        ++in_tile;
+        if (last || next_ch.x != cur_tile || in_tile == kChunksPerFlush) {
+            __syncthreads();
+            for (int e = tid; e < kTerms * kPlane; e += kSpreadThreads) {
+                const long long v = (long long)acc[e];
+                if (v != 0) {
+                    acc[e] = 0ull;
+                    const int node = e % kPlane, t = e / kPlane;
+                    const int gx = bx0 * kInterp + node / kTileNodes, gy = by0 * kInterp + node % kTileNodes;
+                    if (gx < G && gy < G)
+                        atomicAdd(w + ((size_t)gx * G + gy) * kTerms + t, (float)((double)v * fx.from_fixed[t]));
+                }
+            }
+            if (!last) __syncthreads();
+            cur_tile = next_ch.x;
+            in_tile = 0;
         }
+        ch = next_ch;
+        pt[0] = next_pt[0];
+        pt[1] = next_pt[1];
     }
 }
 
@@ -688,8 +736,9 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     tile_scatter_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_cursor, p->tile_xy);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelSpread, s)) return 1;
-    // Upper bound on the number of chunks; surplus workgroups exit at once.
-    const int spread_blocks = N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1;
+    // Resident workgroups share the chunk list (its length is only known on the device; with fewer chunks
+    // than workgroups the surplus ones exit at once).
+    const int spread_blocks = std::min(N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1, p->spread_grid);
     spread_kernel<<<spread_blocks, kSpreadThreads, 0, s>>>(p->tile_xy, p->chunks, p->num_chunks, p->scalars, slot, nb,
                                                 p->lagrange, reinterpret_cast<float *>(p->node_charges));
     TSNE_LAUNCHED(s);
