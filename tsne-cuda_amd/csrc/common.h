@@ -75,11 +75,13 @@ __device__ __forceinline__ float group_max(float v) {
 struct LoopScalars {
     unsigned int min_enc[2];  // ordered-uint encoding of the smallest coordinate
     unsigned int max_enc[2];  // ... and of the largest
-    float z_sum;              // sum_i z_i of the current step (Z = z_sum - N)
     float sumsq;              // scratch for the gradient-norm reduction
     float vmax;               // largest probability of the re-blocked pattern (fixed-point scale)
-    float pad;
+    // sum_i z_i of the current step in kZParts partial sums (Z = their sum - N): a thousand workgroups each
+    // end with one atomic add, and atomics on a single address are performed one after the other.
+    float z_part[16];
 };
+constexpr int kZParts = 16;
 
 }  // namespace tsnehip
 

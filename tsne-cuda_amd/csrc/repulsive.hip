@@ -201,6 +201,33 @@ __device__ __forceinline__ int tile_of(float x, float y, const Bounds &bd, int n
     return (box_of(y, bd, n_boxes) / kTileBoxes) * tiles_per_dim + box_of(x, bd, n_boxes) / kTileBoxes;
 }
 
+// hist[t] += 1 for every active lane of the wave; returns the value the lane's own increment found (its
+// rank).  Neighbouring points of the locality-ordered numbering lie close together in the embedding too,
+// so most lanes of a wave name the same one or two tiles: 64 LDS atomics on one address would be
+// performed one after the other.  Up to four groups of at least eight lanes that share a tile are
+// therefore counted by one lane each (ballot + population count); whatever is left adds on its own.
+__device__ __forceinline__ int wave_tile_add(int *hist, int t, bool active) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    unsigned long long remaining = __ballot(active);
+    int rank = 0;
+    for (int round = 0; round < 4 && remaining; ++round) {
+        const int leader = __builtin_amdgcn_readfirstlane(__ffsll((long long)remaining) - 1);
+        const int tl = __builtin_amdgcn_readlane(t, leader);
+        const bool mine = active && t == tl && ((remaining >> lane) & 1ull);
+        const unsigned long long group = __ballot(mine);
+        const int members = __popcll(group);
+        if (members < 8) break;
+        int first = 0;
+        if (lane == leader) first = atomicAdd(&hist[tl], members);
+        first = __builtin_amdgcn_readlane(first, leader);
+        if (mine) rank = first + __popcll(group & below);
+        remaining &= ~group;
+    }
+    if ((remaining >> lane) & 1ull) rank = atomicAdd(&hist[t], 1);
+    return rank;
+}
+
 // Exclusive scan of the tile counts and of the chunk counts by one workgroup of 1024
 // threads: write cursors, every tile cut into chunks of at most kChunkPoints points.
 // Two tiles per thread (kMaxTiles <= 2 * 1024).  Leaves the counters at zero for the
@@ -259,8 +286,8 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
     __shared__ int last;
     const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
     const int n_tiles = tiles_per_dim * tiles_per_dim;
+    if (blockIdx.x == 0 && threadIdx.x < kZParts) sc->z_part[threadIdx.x] = 0.0f;
     if (blockIdx.x == 0 && threadIdx.x == 0) {
-        sc->z_sum = 0.0f;
         if (next_slot >= 0) {
             sc->min_enc[next_slot] = 0xffffffffu;
             sc->max_enc[next_slot] = 0u;
@@ -269,8 +296,13 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
     for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;
     __syncthreads();
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x)
-        atomicAdd(&hist[tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim)], 1);
+    // (whole waves enter the loop body together: the bound is rounded up to the wave)
+    for (int i0 = blockIdx.x * blockDim.x + (threadIdx.x & ~(kWave - 1)); i0 < N; i0 += gridDim.x * blockDim.x) {
+        const int i = i0 + (threadIdx.x & (kWave - 1));
+        const bool active = i < N;
+        const int t = active ? tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim) : 0;
+        wave_tile_add(hist, t, active);
+    }
     __syncthreads();
     // The counters live where device-scope atomics are performed, so no cache maintenance is needed
     // to publish them (a device-wide fence would write back and invalidate the L2 of every XCD, once
@@ -304,19 +336,25 @@ __global__ __launch_bounds__(1024) void tile_scatter_kernel(const float *__restr
     for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;
     __syncthreads();
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x)
-        atomicAdd(&hist[tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim)], 1);
+    for (int i0 = blockIdx.x * blockDim.x + (threadIdx.x & ~(kWave - 1)); i0 < N; i0 += gridDim.x * blockDim.x) {
+        const int i = i0 + (threadIdx.x & (kWave - 1));
+        const bool active = i < N;
+        const int t = active ? tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim) : 0;
+        wave_tile_add(hist, t, active);
+    }
     __syncthreads();
     for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) {
         base[b] = hist[b] ? atomicAdd(&tile_cursor[b], hist[b]) : 0;
         hist[b] = 0;
     }
     __syncthreads();
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
-        const float x = emb[i], y = emb[N + i];
-        const int t = tile_of(x, y, bd, n_boxes, tiles_per_dim);
-        const int r = atomicAdd(&hist[t], 1);
-        tile_xy[base[t] + r] = make_float2(x, y);
+    for (int i0 = blockIdx.x * blockDim.x + (threadIdx.x & ~(kWave - 1)); i0 < N; i0 += gridDim.x * blockDim.x) {
+        const int i = i0 + (threadIdx.x & (kWave - 1));
+        const bool active = i < N;
+        const float x = active ? emb[i] : 0.0f, y = active ? emb[N + i] : 0.0f;
+        const int t = active ? tile_of(x, y, bd, n_boxes, tiles_per_dim) : 0;
+        const int r = wave_tile_add(hist, t, active);
+        if (active) tile_xy[base[t] + r] = make_float2(x, y);
     }
 }
 
@@ -687,12 +725,16 @@ __global__ __launch_bounds__(256) void gather_forces_kernel(const float *__restr
         float t = 0.0f;
 #pragma unroll
         for (int k = 0; k < 256 / kWave; ++k) t += partial[k];
-        atomicAdd(&sc->z_sum, t);
+        atomicAdd(&sc->z_part[blockIdx.x % kZParts], t);
     }
 }
 
 __global__ void finish_z_kernel(const LoopScalars *sc, int N, float *out) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) *out = sc->z_sum - (float)N;  // src/kernels/rep_forces.cu:54
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        float z = 0.0f;
+        for (int k = 0; k < kZParts; ++k) z += sc->z_part[k];
+        *out = z - (float)N;  // src/kernels/rep_forces.cu:54
+    }
 }
 
 }  // namespace
@@ -719,7 +761,7 @@ int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_
 }
 
 // All kernels of one repulsive-force evaluation.  Expects the bounds of
-// `embedding` in `slot`; leaves sum_i z_i in scalars->z_sum and resets the other
+// `embedding` in `slot`; leaves sum_i z_i in scalars->z_part and resets the other
 // bounds slot.  charges_out (optional) receives a copy of the node charges.
 int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *rep, float *point_potentials,
                      float *charges_out, hipStream_t s) {

@@ -31,10 +31,13 @@ template <bool FUSED>
 __global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, float *__restrict__ attr,
                                                      float *__restrict__ rep, float *__restrict__ gains,
                                                      float *__restrict__ old, int N, float eta,
-                                                     const float *__restrict__ z_ptr, float z_offset, float momentum,
+                                                     const float *__restrict__ z_ptr, int z_count, float z_offset,
+                                                     float momentum,
                                                      float exaggeration, float2 *__restrict__ yxy, LoopScalars *sc,
                                                      int next_slot) {
-    const float normalization = *z_ptr - z_offset;
+    float z_total = 0.0f;
+    for (int k = 0; k < z_count; ++k) z_total += z_ptr[k];  // same order in every thread
+    const float normalization = z_total - z_offset;
     float lo = INFINITY, hi = -INFINITY;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
         float gx = gains[i], gy = gains[N + i];
@@ -87,10 +90,13 @@ template <bool FUSED>
 __global__ __launch_bounds__(256) void update_vec4_kernel(float *__restrict__ emb, float *__restrict__ attr,
                                                           float *__restrict__ rep, float *__restrict__ gains,
                                                           float *__restrict__ old, int N, float eta,
-                                                          const float *__restrict__ z_ptr, float z_offset,
+                                                          const float *__restrict__ z_ptr, int z_count,
+                                                          float z_offset,
                                                           float momentum, float exaggeration,
                                                           float2 *__restrict__ yxy, LoopScalars *sc, int next_slot) {
-    const float normalization = *z_ptr - z_offset;
+    float z_total = 0.0f;
+    for (int k = 0; k < z_count; ++k) z_total += z_ptr[k];  // same order in every thread
+    const float normalization = z_total - z_offset;
     float lo = INFINITY, hi = -INFINITY;
     const int n4 = N / 4;
     float4 *emb4 = reinterpret_cast<float4 *>(emb), *attr4 = reinterpret_cast<float4 *>(attr);
@@ -179,13 +185,14 @@ __global__ __launch_bounds__(256) void sum_squares_kernel(const float *__restric
 
 }  // namespace
 
-// normalization == nullptr: Z is taken from the loop scalars (z_sum - N).
+// normalization == nullptr: Z is taken from the loop scalars (sum of z_part - N).
 // next_slot >= 0: also refresh the (x, y) copy and accumulate the new bounds.
 int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, float *gains, float *old_forces,
                   float eta, const float *normalization, float momentum, float exaggeration, int next_slot,
                   hipStream_t s) {
     const int N = p->num_points;
-    const float *z_ptr = normalization ? normalization : &p->scalars->z_sum;
+    const float *z_ptr = normalization ? normalization : p->scalars->z_part;
+    const int z_count = normalization ? 1 : kZParts;
     const float z_offset = normalization ? 0.0f : (float)N;
     if (profile_mark(p, kKernelUpdate, s)) return 1;
     auto aligned16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
@@ -193,11 +200,11 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
         aligned16(old_forces)) {
         const int blocks = std::min(div_up(N / 4, 256), 512);  // few workgroups: one pair of same-address atomics each
         if (next_slot >= 0) {
-            update_vec4_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr,
+            update_vec4_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count,
                                                             z_offset, momentum, exaggeration, p->yxy, p->scalars,
                                                             next_slot);
         } else {
-            update_vec4_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr,
+            update_vec4_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count,
                                                              z_offset, momentum, exaggeration, nullptr, nullptr, 0);
         }
         TSNE_LAUNCHED(s);
@@ -205,10 +212,10 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
     }
     const int blocks = std::min(div_up(N, 256), 2048);
     if (next_slot >= 0) {
-        update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_offset,
+        update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count, z_offset,
                                                    momentum, exaggeration, p->yxy, p->scalars, next_slot);
     } else {
-        update_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_offset,
+        update_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count, z_offset,
                                                     momentum, exaggeration, nullptr, nullptr, 0);
     }
     TSNE_LAUNCHED(s);
