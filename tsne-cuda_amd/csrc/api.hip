@@ -286,6 +286,8 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     (void)hipFree(p->tile_xy);
     (void)hipFree(p->tile_count);
     (void)hipFree(p->tile_cursor);
+    (void)hipFree(p->point_code);
+    (void)hipFree(p->wg_tile_base);
     (void)hipFree(p->chunks);
     (void)hipFree(p->num_chunks);
     (void)hipFree(p->node_charges);
@@ -331,6 +333,8 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
               hipMalloc(&p->tile_xy, sizeof(float2) * N) == hipSuccess &&
               hipMalloc(&p->tile_count, sizeof(int) * kMaxTiles) == hipSuccess &&
               hipMalloc(&p->tile_cursor, sizeof(int) * kMaxTiles) == hipSuccess &&
+              hipMalloc(&p->point_code, sizeof(unsigned int) * N) == hipSuccess &&
+              hipMalloc(&p->wg_tile_base, sizeof(int) * (size_t)kSortBlocks * kMaxTiles) == hipSuccess &&
               hipMalloc(&p->chunks, sizeof(int4) * p->max_chunks) == hipSuccess &&
               hipMalloc(&p->num_chunks, 2 * sizeof(int)) == hipSuccess &&
               hipMalloc(&p->node_charges, sizeof(float4) * G2) == hipSuccess &&

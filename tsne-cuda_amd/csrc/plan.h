@@ -17,6 +17,7 @@ constexpr int kTileBoxes = 7;     // boxes per side of a spreading tile (21 x 21
                                   // two spreading workgroups fit beside the attractive kernel workgroup of a CU)
 constexpr int kMaxTiles = 25 * 25;  // ceil(kMaxBoxes / kTileBoxes)^2
 constexpr int kChunkPoints = 1024;  // points one workgroup spreads into its private LDS tile
+constexpr int kSortBlocks = 256;    // most workgroups of the tile count / scatter kernels
 
 // Lagrange node positions inside a box and the basis denominators, formed in
 // fp32 exactly as the reference does on the host (src/fit_tsne.cu:303-321).
@@ -52,7 +53,9 @@ struct tsne_hip_plan {
     float2 *yxy = nullptr;         // N interleaved (x, y) pairs for the neighbour gathers
     float2 *tile_xy = nullptr;     // N positions grouped by spreading tile (rebuilt every step)
     int *tile_count = nullptr;     // points per tile
-    int *tile_cursor = nullptr;    // running write position per tile during the scatter
+    int *tile_cursor = nullptr;    // first position of every tile's run in tile_xy
+    unsigned int *point_code = nullptr;  // N: (tile << 22 | rank among its workgroup's points of that tile), by the count kernel
+    int *wg_tile_base = nullptr;   // kSortBlocks x kMaxTiles: where a workgroup's points start inside a tile's run
     int4 *chunks = nullptr;        // (tile, first point, count, -) per spreading workgroup
     int *num_chunks = nullptr;  // [0] chunks of the current step, [1] ticket counter of the tile count kernel
     int max_chunks = 0;

@@ -201,6 +201,9 @@ __device__ __forceinline__ int tile_of(float x, float y, const Bounds &bd, int n
     return (box_of(y, bd, n_boxes) / kTileBoxes) * tiles_per_dim + box_of(x, bd, n_boxes) / kTileBoxes;
 }
 
+constexpr int kRankBits = 22;  // a point's code: tile << kRankBits | rank (a workgroup counts fewer than 4 M points)
+static_assert(kMaxTiles <= (1 << (32 - kRankBits)), "tile numbers must fit the code's upper bits");
+
 // hist[t] += 1 for every active lane of the wave; returns the value the lane's own increment found (its
 // rank).  Neighbouring points of the locality-ordered numbering lie close together in the embedding too,
 // so most lanes of a wave name the same one or two tiles: 64 LDS atomics on one address would be
@@ -280,7 +283,9 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
                                                          int slot, int next_slot, int n_boxes,
                                                          int *__restrict__ tile_count,
                                                          int *__restrict__ tile_cursor, int4 *__restrict__ chunks,
-                                                         int *__restrict__ num_chunks, int *__restrict__ ticket) {
+                                                         int *__restrict__ num_chunks, int *__restrict__ ticket,
+                                                         unsigned int *__restrict__ point_code,
+                                                         int *__restrict__ wg_tile_base) {
     __shared__ int hist[kMaxTiles];
     __shared__ int pts[1024], chk[1024];
     __shared__ int last;
@@ -301,7 +306,9 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
         const int i = i0 + (threadIdx.x & (kWave - 1));
         const bool active = i < N;
         const int t = active ? tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim) : 0;
-        wave_tile_add(hist, t, active);
+        const int rank = wave_tile_add(hist, t, active);
+        // The scatter kernel needs no histogram of its own: tile and rank travel with the point.
+        if (active) point_code[i] = ((unsigned int)t << kRankBits) | (unsigned int)rank;
     }
     __syncthreads();
     // The counters live where device-scope atomics are performed, so no cache maintenance is needed
@@ -310,8 +317,8 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
     // taken after all of this workgroup's atomics have returned.
     for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) {
         if (hist[b]) {
-            const int before = atomicAdd(&tile_count[b], hist[b]);
-            asm volatile("" ::"v"(before));
+            // what the counter held before: where this workgroup's points start inside the tile's run
+            wg_tile_base[(size_t)blockIdx.x * kMaxTiles + b] = atomicAdd(&tile_count[b], hist[b]);
         }
     }
     __syncthreads();
@@ -322,39 +329,22 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
     if (threadIdx.x == 0) *ticket = 0;
 }
 
-// Same point-to-workgroup assignment as tile_count_kernel: the workgroup
-// reserves a run per tile with one global atomic, then ranks its points inside
-// the run with LDS atomics.
-__global__ __launch_bounds__(1024) void tile_scatter_kernel(const float *__restrict__ emb, int N,
-                                                           const LoopScalars *sc, int slot, int n_boxes,
-                                                           int *__restrict__ tile_cursor,
+// Same point-to-workgroup assignment as tile_count_kernel, which left every point's tile and its rank
+// among the workgroup's points of that tile: position = start of the tile's run + start of the
+// workgroup's part of it + rank.  A streaming pass without atomics.
+__global__ __launch_bounds__(1024) void tile_scatter_kernel(const float *__restrict__ emb, int N, int n_tiles,
+                                                           const int *__restrict__ tile_cursor,
+                                                           const unsigned int *__restrict__ point_code,
+                                                           const int *__restrict__ wg_tile_base,
                                                            float2 *__restrict__ tile_xy) {
-    __shared__ int hist[kMaxTiles];
     __shared__ int base[kMaxTiles];
-    const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
-    const int n_tiles = tiles_per_dim * tiles_per_dim;
-    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;
+    // (entries of wg_tile_base for tiles this workgroup has no point in are never read)
+    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x)
+        base[b] = tile_cursor[b] + wg_tile_base[(size_t)blockIdx.x * kMaxTiles + b];
     __syncthreads();
-    const Bounds bd = load_bounds(sc, slot, n_boxes);
-    for (int i0 = blockIdx.x * blockDim.x + (threadIdx.x & ~(kWave - 1)); i0 < N; i0 += gridDim.x * blockDim.x) {
-        const int i = i0 + (threadIdx.x & (kWave - 1));
-        const bool active = i < N;
-        const int t = active ? tile_of(emb[i], emb[N + i], bd, n_boxes, tiles_per_dim) : 0;
-        wave_tile_add(hist, t, active);
-    }
-    __syncthreads();
-    for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) {
-        base[b] = hist[b] ? atomicAdd(&tile_cursor[b], hist[b]) : 0;
-        hist[b] = 0;
-    }
-    __syncthreads();
-    for (int i0 = blockIdx.x * blockDim.x + (threadIdx.x & ~(kWave - 1)); i0 < N; i0 += gridDim.x * blockDim.x) {
-        const int i = i0 + (threadIdx.x & (kWave - 1));
-        const bool active = i < N;
-        const float x = active ? emb[i] : 0.0f, y = active ? emb[N + i] : 0.0f;
-        const int t = active ? tile_of(x, y, bd, n_boxes, tiles_per_dim) : 0;
-        const int r = wave_tile_add(hist, t, active);
-        if (active) tile_xy[base[t] + r] = make_float2(x, y);
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
+        const unsigned int code = point_code[i];
+        tile_xy[base[code >> kRankBits] + (int)(code & ((1u << kRankBits) - 1u))] = make_float2(emb[i], emb[N + i]);
     }
 }
 
@@ -769,13 +759,15 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     const int tiles_per_dim = (nb + kTileBoxes - 1) / kTileBoxes;
     // Few, large workgroups: every workgroup ends with one global atomic per tile counter, and
     // same-address atomics serialise (about a thousand per counter cost ~20 us).
-    const int sort_blocks = std::min(div_up(N, 1024 * 4), 256);
+    const int sort_blocks = std::min(div_up(N, 1024 * 4), kSortBlocks);
     if (profile_mark(p, kKernelTileCount, s)) return 1;
     tile_count_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, slot ^ 1, nb, p->tile_count,
-                                                   p->tile_cursor, p->chunks, p->num_chunks, p->num_chunks + 1);
+                                                   p->tile_cursor, p->chunks, p->num_chunks, p->num_chunks + 1,
+                                                   p->point_code, p->wg_tile_base);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelTileScatter, s)) return 1;
-    tile_scatter_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, nb, p->tile_cursor, p->tile_xy);
+    tile_scatter_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, tiles_per_dim * tiles_per_dim, p->tile_cursor,
+                                                     p->point_code, p->wg_tile_base, p->tile_xy);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelSpread, s)) return 1;
     // Resident workgroups share the chunk list (its length is only known on the device; with fewer chunks
