@@ -116,8 +116,8 @@ def main():
     # planes; the transposed spectra are 2 plane pairs x 1024 x 512 complex).
     G2, spectra = 390.0 * 390.0, 2 * 1024 * 512 * 8.0
     loop_bytes = {
-        "tile_count_kernel": 8.0 * n,                       # positions in
-        "tile_scatter_kernel": 16.0 * n,                    # positions in, positions grouped by tile out
+        "tile_count_kernel": 12.0 * n,                      # positions in, (tile, rank) codes out
+        "tile_scatter_kernel": 20.0 * n,                    # positions and codes in, positions grouped by tile out
         "spread_kernel": 8.0 * n + 16.0 * G2,               # grouped positions in, node charges out
         "conv_rows_forward_kernel": 16.0 * G2 + spectra,    # node charges in, row spectra out
         "conv_columns_kernel": 2.0 * spectra,               # row spectra in, convolved columns out
