@@ -1139,7 +1139,22 @@ __global__ __launch_bounds__(256) void knn_rerank_kernel(const float *__restrict
                     // rows are 8-byte aligned: two dimensions per load, the same fma chain
                     const float2 *q2 = reinterpret_cast<const float2 *>(xq);
                     const float2 *j2 = reinterpret_cast<const float2 *>(xj);
-                    for (int d = 0; d < D / 2; ++d) {
+                    const int n2 = D / 2;
+                    int d = 0;
+                    // eight loads (64 bytes of the candidate's row) in flight per lane
+                    for (; d + 8 <= n2; d += 8) {
+                        float2 b[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) b[u] = j2[d + u];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) {
+                            const float2 a = q2[d + u];
+                            const float d0 = a.x - b[u].x, d1 = a.y - b[u].y;
+                            acc = fmaf(d0, d0, acc);
+                            acc = fmaf(d1, d1, acc);
+                        }
+                    }
+                    for (; d < n2; ++d) {
                         const float2 a = q2[d], b = j2[d];
                         const float d0 = a.x - b.x, d1 = a.y - b.y;
                         acc = fmaf(d0, d0, acc);
