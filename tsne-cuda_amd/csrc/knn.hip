@@ -195,8 +195,12 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 // of LDS.  Afterwards list[0, min(n, want)) holds the entries kept (in no particular order), *cnt their
 // number, and *thr is lowered to (distance of the want-th smallest, all index bits set) when n >= want.
 // Returns the number of entries kept.
+// With slack > 0 the selection may stop early: once the histogram bin that holds the want-th smallest
+// has few enough entries that keeping all of them stays within want + slack, everything up to the
+// bin's upper edge is kept and that edge becomes the threshold.  A compaction in the middle of a sweep
+// only needs some threshold below which everything was kept; the last one of a query passes slack = 0.
 __device__ __forceinline__ int wave_select(u64 *list, int want, int *cnt, u64 *thr, u64 *buf, unsigned int *hist,
-                                           int lane) {
+                                           int lane, int slack = 0) {
     __threadfence_block();  // this wave's appends to the list are complete
     const int n = *cnt;
     if (n < want) return n;
@@ -243,6 +247,30 @@ __device__ __forceinline__ int wave_select(u64 *list, int want, int *cnt, u64 *t
         const int b = __ffsll((long long)__ballot(incl >= rank)) - 1;  // some lane qualifies: the last one holds all matches
         rank -= __shfl(incl - c, b, kWave);
         prefix = (prefix << w) | (unsigned int)b;
+        if (slack > 0 && shift > 0) {
+            const int kept = (want - rank) + __shfl(c, b, kWave);  // below the bin + the whole bin
+            if (kept <= want + slack) {
+                // Keep everything up to the upper edge of the bin.
+                const u64 edge = (u64)lo + ((((u64)prefix + 1ull) << shift) - 1ull);
+                const unsigned int dedge = edge > 0xffffffffull ? 0xffffffffu : (unsigned int)edge;
+                int base = 0;
+                const u64 below_lanes = (1ull << lane) - 1ull;
+                for (int e0 = 0; e0 < n; e0 += kWave) {
+                    const int e = e0 + lane;
+                    const u64 key = e < n ? buf[e] : 0ull;
+                    const bool keep = e < n && (unsigned int)(key >> 32) <= dedge;
+                    const u64 m = __ballot(keep);
+                    if (keep) list[base + __popcll(m & below_lanes)] = key;
+                    base += __popcll(m);
+                }
+                if (lane == 0) {
+                    *cnt = base;
+                    *thr = ((u64)dedge << 32) | 0xffffffffull;
+                }
+                __threadfence_block();
+                return base;
+            }
+        }
     }
     const unsigned int dstar = lo + prefix;
     // Keep everything below dstar and the first `rank` entries equal to it.
@@ -525,6 +553,7 @@ struct SweepArgs {
     int qtile_first, qtile_step;
     int parts;
     u64 *part_keys;
+    int select_slack;  // entries beyond `want` a compaction in mid-sweep may keep (see wave_select)
 };
 
 // ---------------------------------------------------------------------------
@@ -695,7 +724,8 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                 while (crowded) {
                     const int ql = wave * 32 + (__ffsll((long long)crowded) - 1);
                     crowded &= crowded - 1;
-                    wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
+                    wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane,
+                                args.select_slack);
                 }
             }
             __syncthreads();  // all waves are done with tile `buf`
@@ -947,7 +977,8 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                 while (crowded) {
                     const int ql = wave * 32 + (__ffsll((long long)crowded) - 1);
                     crowded &= crowded - 1;
-                    wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
+                    wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane,
+                                args.select_slack);
                 }
             }
             __syncthreads();  // all waves are done with the tile's last chunk
@@ -1453,6 +1484,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         args.radius = radius.as<float>();
         args.bitmap_words = bitmap_words;
         args.trigger = cap - kCT;  // as late as possible: a later selection costs the same and sees more candidates
+        args.select_slack = (cap - kCT - keep) / 4;
         args.tiles_swept = reinterpret_cast<unsigned long long *>(scal.as<int>() + 2);
         args.Bp = Bp.as<float4>();
         args.n_chunks = n_chunks;
