@@ -37,8 +37,8 @@ def main():
                     help="run the repulsive chain and the attractive kernel one after the other (TSNE_OVERLAP=0): "
                          "per-kernel durations in a trace then are those of kernels running alone")
     ap.add_argument("--fit-repeats", type=int, default=3, help="end-to-end fits timed (the median is reported)")
-    ap.add_argument("--cpu-steps", type=int, default=20, help="gradient steps of the CPU baseline sample")
-    ap.add_argument("--cpu-knn-rows", type=int, default=512, help="query rows of the CPU baseline's kNN sample")
+    ap.add_argument("--cpu-steps", type=int, default=150, help="gradient steps of the CPU baseline sample")
+    ap.add_argument("--cpu-knn-rows", type=int, default=4096, help="query rows of the CPU baseline's kNN sample")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 10 plain 256 MiB device copies (known traffic, to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
