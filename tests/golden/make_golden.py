@@ -9,7 +9,8 @@ checks in tests/test_oracle.py.
   small256.npz   256 x 16 points, K = 16: neighbours, P, forces and one update
                  step from a fixed embedding (a few hundred KB at most)
   c0_fit.json    config c0 (5000 x 50, K = 90, perplexity 30): objective value
-                 of the oracle's 1000-step fit from the seeded initial embedding
+                 and trustworthiness of the oracle's 1000-step fit from the seeded
+                 initial embedding
 
 Run from the repository root:  python tests/golden/make_golden.py
 """
@@ -25,6 +26,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tsne-cuda_amd"))
 
 import oracle  # noqa: E402
+from sklearn.manifold import trustworthiness  # noqa: E402
 from tsnecuda import synthetic  # noqa: E402
 
 
@@ -60,6 +62,10 @@ def c0_fit():
         "z_final_interpolated": z,
         "extent": [float(y.min()), float(y.max())],
         "p_sum": float(P.astype(np.float64).sum()),
+        # fraction of each point's 12 nearest embedding neighbours that are also near in the input space
+        # (sklearn's definition, an independent implementation)
+        "trustworthiness_k12": float(trustworthiness(X, np.stack([y[:X.shape[0]], y[X.shape[0]:]], axis=1),
+                                                     n_neighbors=12)),
     }
     with open(os.path.join(HERE, "c0_fit.json"), "w") as f:
         json.dump(out, f, indent=1)

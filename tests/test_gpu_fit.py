@@ -42,6 +42,11 @@ def test_c0_fit_objective_within_one_percent(c0_problem):
     assert abs(model.kl_divergence_ - kl) <= 2e-3 * kl
     # same overall scale of the layout
     assert 0.8 < (emb.max() - emb.min()) / (gold["extent"][1] - gold["extent"][0]) < 1.25
+    # and the same neighbourhood preservation, by an implementation that shares nothing with this build
+    from sklearn.manifold import trustworthiness
+    t = trustworthiness(c["X"], emb, n_neighbors=12)
+    print("trustworthiness gpu %.4f oracle %.4f" % (t, gold["trustworthiness_k12"]))
+    assert abs(t - gold["trustworthiness_k12"]) <= 0.01
 
 
 def test_fit_is_repeatable_for_a_given_start(c0_problem):
