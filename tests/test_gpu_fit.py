@@ -146,3 +146,26 @@ def test_whole_pipeline_against_the_oracle(n, d, k, clusters):
     got = flat(emb)
     assert np.isfinite(got).all()
     assert np.linalg.norm(got - y_o) <= 2e-3 * np.linalg.norm(y_o)
+
+
+def test_command_line_program(tmp_path):
+    """`tsne` on its built-in two-cluster data set (src/exe/main.cu:172-213):
+    runs RunTsne with the given options, prints the reference's progress and
+    timing lines, and dumps every step when asked to."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tsne-cuda_amd", "tsnecuda", "tsne")
+    out = subprocess.run([exe, "-k", "600", "--dim=8", "-n", "30", "-u", "20", "--perplexity", "8", "-d"],
+                         capture_output=True, text=True, cwd=tmp_path, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert "Starting TSNE calculation with 600 points." in out.stdout
+    assert "[Step 0] Avg. Gradient Norm:" in out.stdout and "_time_knn:" in out.stdout
+    lines = (tmp_path / "dump_ys.txt").read_text().split("\n")
+    assert lines[0] == "600 2"
+    body = np.array([[float(v) for v in l.split()] for l in lines[1:] if l])
+    assert body.shape == (30 * 600, 2) and np.isfinite(body).all()
+    # two well separated clusters of 300 points: after 30 exaggerated steps each half is closer to its own
+    # centroid than to the other's
+    last = body[-600:]
+    a, b = last[:300].mean(0), last[300:].mean(0)
+    own = np.linalg.norm(last[:300] - a, axis=1) < np.linalg.norm(last[:300] - b, axis=1)
+    assert own.mean() > 0.95

@@ -113,3 +113,88 @@ def test_synthetic_generators_are_deterministic():
     assert 0.0 < u.min() and u.max() < 1.0 and abs(u.mean() - 0.5) < 5e-3
     z = synthetic.normal(0, 0, 200000)
     assert abs(z.mean()) < 1e-2 and abs(z.std() - 1.0) < 1e-2
+
+
+def _load(fn, path):
+    lib = ctypes.CDLL(LIB)
+    f = getattr(lib, fn)
+    f.restype = ctypes.POINTER(ctypes.c_float)
+    f.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_int)]
+    dims = (ctypes.c_int * 2)()
+    ptr = f(str(path).encode(), dims)
+    if not ptr:
+        return None
+    out = np.ctypeslib.as_array(ptr, shape=(dims[0], dims[1])).copy()
+    lib.tsnecuda_free_points.argtypes = [ctypes.POINTER(ctypes.c_float)]
+    lib.tsnecuda_free_points(ptr)
+    return out
+
+
+def test_mnist_reader(tmp_path, capfd):
+    """idx3-ubyte: big-endian magic 2051, count, rows, columns, one byte per
+    pixel; values / 255, one image per row (src/util/data_utils.cu:12-79)."""
+    rng = np.random.default_rng(0)
+    pixels = rng.integers(0, 256, size=(1234, 7, 5), dtype=np.uint8)  # more images than one read batch
+    path = tmp_path / "images.idx3-ubyte"
+    with open(path, "wb") as f:
+        f.write(np.array([2051, 1234, 7, 5], dtype=">i4").tobytes())
+        f.write(pixels.tobytes())
+    got = _load("tsnecuda_load_mnist", path)
+    assert got.shape == (1234, 35) and got.dtype == np.float32
+    assert np.array_equal(got, pixels.reshape(1234, 35).astype(np.float32) / np.float32(255.0))
+    assert "Num Images: 1234" in capfd.readouterr().out
+    # wrong magic number, truncated file, missing file: no data
+    bad = tmp_path / "labels.idx1-ubyte"
+    bad.write_bytes(np.array([2049, 10, 1, 1], dtype=">i4").tobytes() + bytes(10))
+    assert _load("tsnecuda_load_mnist", bad) is None
+    short = tmp_path / "short.idx3-ubyte"
+    short.write_bytes(np.array([2051, 100, 7, 5], dtype=">i4").tobytes() + bytes(99 * 35))
+    assert _load("tsnecuda_load_mnist", short) is None
+    assert _load("tsnecuda_load_mnist", tmp_path / "missing") is None
+    err = capfd.readouterr().err
+    assert "Magic number: 2049" in err and "ends after 99 of 100" in err and "cannot read" in err
+
+
+def test_cifar_readers(tmp_path):
+    """CIFAR-10: five files of 10000 records (1 label byte + 3072 pixels);
+    CIFAR-100: one file of 50000 records with 2 label bytes
+    (src/util/data_utils.cu:81-159)."""
+    rng = np.random.default_rng(1)
+    pixels = rng.integers(0, 256, size=(50000, 3072), dtype=np.uint8)
+    want = pixels.astype(np.float32) / np.float32(255.0)
+    for b in range(5):
+        rec = np.concatenate([rng.integers(0, 10, size=(10000, 1), dtype=np.uint8), pixels[b * 10000:(b + 1) * 10000]],
+                             axis=1)
+        (tmp_path / ("data_batch_%d.bin" % (b + 1))).write_bytes(rec.tobytes())
+    got = _load("tsnecuda_load_cifar10", tmp_path)
+    assert got.shape == (50000, 3072) and np.array_equal(got, want)
+    rec = np.concatenate([rng.integers(0, 100, size=(50000, 2), dtype=np.uint8), pixels], axis=1)
+    (tmp_path / "train.bin").write_bytes(rec.tobytes())
+    got = _load("tsnecuda_load_cifar100", tmp_path / "train.bin")
+    assert got.shape == (50000, 3072) and np.array_equal(got, want)
+    (tmp_path / "data_batch_5.bin").unlink()
+    assert _load("tsnecuda_load_cifar10", tmp_path) is None
+
+
+def test_command_line_options(capfd):
+    """The `tsne` program takes the reference's option letters and names
+    (src/exe/main.cu:25-40); parsing needs no GPU."""
+    import subprocess
+    exe = os.path.join(ROOT, "tsne-cuda_amd", "tsnecuda", "tsne")
+    assert os.path.exists(exe), "build first: make -C tsne-cuda_amd"
+    out = subprocess.run([exe, "--help"], capture_output=True, text=True)
+    assert out.returncode == 0
+    for line in ("-l, --learning-rate arg", "-p, --perplexity arg", "-e, --early-ex arg", "-s, --data arg",
+                 "-k, --num-points arg", "-u, --nearest-neighbors arg", "-n, --num-steps arg", "-i, --viz",
+                 "-d, --dump", "-m, --magnitude-factor arg", "-t, --init arg", "-f, --fname arg",
+                 "-c, --connection arg", "-q, --dim arg", "-j, --device arg", "-h, --help"):
+        assert line in out.stdout, line
+    assert "(default: 50.0)" in out.stdout and "(default: 32)" in out.stdout
+    bad = subprocess.run([exe, "--no-such-option"], capture_output=True, text=True)
+    assert bad.returncode != 0 and "does not exist" in bad.stderr
+    bad = subprocess.run([exe, "-n", "many"], capture_output=True, text=True)
+    assert bad.returncode != 0 and "failed to parse" in bad.stderr
+    unknown = subprocess.run([exe, "-s", "imagenet"], capture_output=True, text=True)
+    assert unknown.returncode == 0 and "Dataset not recognized..." in unknown.stdout
+    missing = subprocess.run([exe, "--data=mnist", "-f", "/nonexistent/file"], capture_output=True, text=True)
+    assert missing.returncode != 0 and "cannot read" in missing.stderr
