@@ -12,7 +12,9 @@ checks in tests/test_oracle.py.
                  and trustworthiness of the oracle's 1000-step fit from the seeded
                  initial embedding
 
-Run from the repository root:  python tests/golden/make_golden.py
+  c1_fit.json, c2_fit.json   the same for configs c1 and c2 (trustworthiness on a fixed subsample)
+
+Run from the repository root:  python tests/golden/make_golden.py [small] [c0] [c1] [c2]
 """
 import json
 import os
@@ -72,6 +74,42 @@ def c0_fit():
     print(out)
 
 
+def subsample(n, m=4000):
+    """The m points on which the larger configs' trustworthiness is evaluated (the full pairwise matrix of
+    60000 points does not fit a test)."""
+    return np.sort(np.random.default_rng(0).choice(n, size=m, replace=False))
+
+
+def larger_fit(name):
+    """Configs c1 (60000 x 784) and c2 (50000 x 1024): objective and subsample trustworthiness of the
+    oracle's 1000-step fit; a few minutes of CPU time each."""
+    X, fit = synthetic.make_config(name)
+    n = X.shape[0]
+    Y0 = synthetic.initial_embedding(n)
+    y0 = np.concatenate([Y0[:, 0], Y0[:, 1]])
+    y, z, idx, P = oracle.fit(X, y0, fit["num_neighbors"], fit["perplexity"], eps=1e-4, iterations=1000,
+                              eta=fit["learning_rate"])
+    sub = subsample(n)
+    emb = np.stack([y[:n], y[n:]], axis=1)
+    out = {
+        "config": "%s: %d x %d, K=%d, perplexity %g, lr %g, 1000 steps, exaggeration 12 for 250, VECTOR init seed 1"
+                  % (name, n, X.shape[1], fit["num_neighbors"], fit["perplexity"], fit["learning_rate"]),
+        "kl_exact_z": oracle.kl(P, idx, y),
+        "kl_initial": oracle.kl(P, idx, y0),
+        "extent": [float(y.min()), float(y.max())],
+        "trustworthiness_k12_subsample4000": float(trustworthiness(X[sub], emb[sub], n_neighbors=12)),
+    }
+    with open(os.path.join(HERE, "%s_fit.json" % name), "w") as f:
+        json.dump(out, f, indent=1)
+    print(out)
+
+
 if __name__ == "__main__":
-    small_case()
-    c0_fit()
+    which = sys.argv[1:] or ["small", "c0", "c1", "c2"]
+    if "small" in which:
+        small_case()
+    if "c0" in which:
+        c0_fit()
+    for name in ("c1", "c2"):
+        if name in which:
+            larger_fit(name)

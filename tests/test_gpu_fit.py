@@ -49,6 +49,38 @@ def test_c0_fit_objective_within_one_percent(c0_problem):
     assert abs(t - gold["trustworthiness_k12"]) <= 0.01
 
 
+@pytest.mark.parametrize("name", ["c1", "c2"])
+def test_larger_configs_objective_within_one_percent(name):
+    """Configs c1 (60000 x 784 pixel-like) and c2 (50000 x 1024 feature-like), 1000
+    steps from the seeded start: the objective of the final embedding (exact Z,
+    evaluated by the oracle on the neighbours and P of the GPU stages, which are
+    compared with the oracle's elsewhere) within 1 % of the oracle's own run, and
+    the trustworthiness of a fixed 4000-point subsample within 0.02 of it
+    (tests/golden/c1_fit.json, c2_fit.json)."""
+    from sklearn.manifold import trustworthiness
+    from tsnecuda import TSNE, stages, synthetic
+    with open(os.path.join(GOLDEN, "%s_fit.json" % name)) as f:
+        gold = json.load(f)
+    X, fit = synthetic.make_config(name)
+    n, k = X.shape[0], fit["num_neighbors"]
+    Y0 = synthetic.initial_embedding(n)
+    model = TSNE(perplexity=fit["perplexity"], num_neighbors=k, learning_rate=fit["learning_rate"], n_iter=1000,
+                 perplexity_epsilon=1e-4)
+    emb = model.fit_transform(X, y=Y0)
+    assert emb.shape == (n, 2) and np.isfinite(emb).all()
+    idx, d2 = stages.knn(torch.from_numpy(X).cuda(), k)
+    P = stages.symmetrize(stages.perplexity(stages.max_normalize_(d2), fit["perplexity"], 1e-4), idx)
+    kl = oracle.kl(P.cpu().numpy(), idx.cpu().numpy(), flat(emb))
+    sub = np.sort(np.random.default_rng(0).choice(n, size=4000, replace=False))  # as tests/golden/make_golden.py
+    t = trustworthiness(X[sub], emb[sub], n_neighbors=12)
+    print("%s: KL gpu %.5f oracle %.5f (library's own %.5f), trustworthiness gpu %.4f oracle %.4f"
+          % (name, kl, gold["kl_exact_z"], model.kl_divergence_, t, gold["trustworthiness_k12_subsample4000"]))
+    assert abs(kl - gold["kl_exact_z"]) <= 0.01 * gold["kl_exact_z"]
+    assert abs(model.kl_divergence_ - kl) <= 5e-3 * kl
+    assert abs(t - gold["trustworthiness_k12_subsample4000"]) <= 0.02
+    assert 0.8 < (emb.max() - emb.min()) / (gold["extent"][1] - gold["extent"][0]) < 1.25
+
+
 def test_fit_is_repeatable_for_a_given_start(c0_problem):
     """Two short fits from the same start agree closely.  Not bitwise: the
     charge spreading and the Z reduction use floating-point atomics, and the
