@@ -182,6 +182,14 @@ def main():
                "knn_query_rows_per_s": knn_rows / knn_cpu_s,
                "fit_seconds_extrapolated": n / (knn_rows / knn_cpu_s) + 1000.0 / (args.cpu_steps / cpu_s)}
 
+    # The CPU oracle's own 1000-step fit of the same configuration from the same start (a fixture: the fit
+    # takes an hour of CPU time at 1M points), for the objective of the GPU fit to stand beside.
+    oracle_kl = None
+    gold_path = os.path.join(ROOT, "tests", "golden", "%s_fit.json" % args.workload)
+    if args.points is None and os.path.exists(gold_path):
+        with open(gold_path) as f:
+            oracle_kl = json.load(f).get("kl_exact_z")
+
     # HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes whose
     # summary sits in profiles/bench_c3_1M_hbm_counters.txt (423464 x 2 KiB fetched + 7826 x 1 KiB written);
     # the counters belong to that exact workload, so other sizes report null.
@@ -204,6 +212,7 @@ def main():
         "fit_seconds": fit_s,
         "fit_seconds_runs": fit_runs,
         "fit_kl_divergence": kl_final,
+        "fit_kl_divergence_oracle": oracle_kl,
         "phases_s": {"locality_order": order_s + gather_s, "knn": knn_s, "max_normalize": norm_s, "perplexity": perp_s, "symmetrize": sym_s,
                      "reblock_pattern": reblock_s,
                      "gradient_loop_%d_steps" % args.steps: loop_s, "data_generation_host": gen_s},

@@ -105,11 +105,11 @@ def larger_fit(name):
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["small", "c0", "c1", "c2"]
+    which = sys.argv[1:] or ["small", "c0", "c1", "c2"]  # c3 (1,000,000 points) only when named: about an hour
     if "small" in which:
         small_case()
     if "c0" in which:
         c0_fit()
-    for name in ("c1", "c2"):
+    for name in ("c1", "c2", "c3"):
         if name in which:
             larger_fit(name)
