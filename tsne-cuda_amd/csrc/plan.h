@@ -13,9 +13,9 @@ constexpr int kTerms = 4;         // charges per point (src/fit_tsne.cu:254)
 constexpr int kFft = 1024;        // padded transform length, >= 2 * 3 * n_boxes - 1
 constexpr int kNodePad = 512;     // leading dimension of the transposed spectra (>= nodes per dim)
 constexpr int kMaxBoxes = 170;    // 3 * 170 = 510 nodes <= kNodePad
-constexpr int kTileBoxes = 7;     // boxes per side of a spreading tile (21 x 21 nodes x 4 terms x 8 B = 14.1 KB of LDS:
-                                  // two spreading workgroups fit beside the attractive kernel workgroup of a CU)
-constexpr int kMaxTiles = 25 * 25;  // ceil(kMaxBoxes / kTileBoxes)^2
+constexpr int kTileBoxes = 5;     // boxes per side of a spreading tile (25 boxes x 21 moments x 8 B = 4.2 KB of LDS;
+                                  // measured alone at 1M points: 4 -> 29 us, 5 -> 28 us, 7 -> 33 us, 10 -> 49 us)
+constexpr int kMaxTiles = 34 * 34;  // ceil(kMaxBoxes / kTileBoxes)^2
 constexpr int kChunkPoints = 1024;  // points one workgroup spreads into its private LDS tile
 constexpr int kSortBlocks = 256;    // most workgroups of the tile count / scatter kernels
 

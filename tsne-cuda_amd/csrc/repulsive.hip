@@ -201,7 +201,7 @@ __device__ __forceinline__ int tile_of(float x, float y, const Bounds &bd, int n
     return (box_of(y, bd, n_boxes) / kTileBoxes) * tiles_per_dim + box_of(x, bd, n_boxes) / kTileBoxes;
 }
 
-constexpr int kRankBits = 22;  // a point's code: tile << kRankBits | rank (a workgroup counts fewer than 4 M points)
+constexpr int kRankBits = 21;  // a point's code: tile << kRankBits | rank (a workgroup counts fewer than 2 M points)
 static_assert(kMaxTiles <= (1 << (32 - kRankBits)), "tile numbers must fit the code's upper bits");
 
 // hist[t] += 1 for every active lane of the wave; returns the value the lane's own increment found (its
@@ -348,30 +348,9 @@ __global__ __launch_bounds__(1024) void tile_scatter_kernel(const float *__restr
     }
 }
 
-// Fixed-point scales of the four charge planes.  With m the largest absolute
-// coordinate and |Lx * Ly| <= 1.875^2 < 4, a contribution to plane t is bounded by
-// B = (4, 4m, 4m, 8m^2); the scale 2^50 / B keeps a contribution below 2^50 and
-// the sum of a chunk's 2048 contributions below 2^61.
-constexpr int kSpreadThreads = 512;  // per chunk of kChunkPoints points: the chunk's critical path sets the kernel time
+constexpr int kSpreadThreads = 512;  // two points of a 1024-point chunk per thread
 
-struct SpreadScales {
-    double to_fixed[kTerms];
-    double from_fixed[kTerms];
-};
-__device__ __forceinline__ SpreadScales spread_scales(const LoopScalars *sc, int slot) {
-    const float lo = ordered_to_float(sc->min_enc[slot]);
-    const float hi = ordered_to_float(sc->max_enc[slot]);
-    double m = fmax(fabs((double)lo), fabs((double)hi));
-    if (!(m > 0.0)) m = 1.0;
-    const double bound[kTerms] = {4.0, 4.0 * m, 4.0 * m, 8.0 * m * m};
-    SpreadScales s;
-#pragma unroll
-    for (int t = 0; t < kTerms; ++t) {
-        s.to_fixed[t] = 1125899906842624.0 / bound[t];  // 2^50 / B
-        s.from_fixed[t] = bound[t] / 1125899906842624.0;
-    }
-    return s;
-}
+// 64-bit fixed-point add of v * scale (|v * scale| < 2^51) to an LDS word.
 __device__ __forceinline__ void add_fixed(unsigned long long *dst, float v, double scale) {
     const double magic = 6755399441055744.0;  // 1.5 * 2^52: adding it rounds a double to an integer
     const double r = fma((double)v, scale, magic);
@@ -381,36 +360,71 @@ __device__ __forceinline__ void add_fixed(unsigned long long *dst, float v, doub
 // LDS float atomic adds cost ~190 clocks per wave instruction on gfx950 while
 // 64-bit integer LDS atomics are about 25x faster, so the private tile is kept
 // in 64-bit fixed point (which also makes the sums independent of the order of
-// the additions) and converted to fp32 when it is flushed.
+// the additions) and converted when it is flushed.
 //
 // A workgroup takes a contiguous range of the chunk list (the chunks are in tile
 // order): while it spreads one chunk the points of the next are already on their
 // way, consecutive chunks of one tile share the LDS tile, and the tile goes to
 // global memory (float atomics: neighbouring workgroups may hold parts of the same
 // tile) when the tile changes, after kChunksPerFlush chunks (the fixed-point sums
-// have room for 8192 contributions per node), and at the end of the range.
+// have room for 8192 contributions of at most 1) and at the end of the range.
 constexpr int kChunksPerFlush = 4;
 static_assert(kChunkPoints == 2 * kSpreadThreads, "a thread spreads two points of a chunk");
-static_assert(kChunksPerFlush * kChunkPoints <= 4096, "a node's fixed-point sum must stay below 2^62");
+static_assert(kChunksPerFlush * kChunkPoints <= 4096, "a box's fixed-point sums must stay below 2^62");
+
+// In-box coordinate of one embedding coordinate: box as in bin_and_weights, t in [0, 1].
+__device__ __forceinline__ void bin_and_coord(float v, const Bounds &bd, int n_boxes, int &box, float &t) {
+#pragma clang fp contract(off)
+    int b = (int)((v - bd.lo) / bd.box_width);
+    b = max(0, b);
+    b = min(n_boxes - 1, b);
+    box = b;
+    const float lower = b * bd.box_width + bd.lo;
+    t = (v - lower) / bd.box_width;
+}
+
+// Lower edge of a box, rounded as the binning rounds it.
+__device__ __forceinline__ float box_lower(int b, const Bounds &bd) {
+#pragma clang fp contract(off)
+    return b * bd.box_width + bd.lo;
+}
+
+// What a point adds to the nine nodes of its box, L_a(u) L_b(v) (1, x, y, x^2 + y^2) with u, v its
+// in-box coordinates, is a polynomial in (u, v): the three Lagrange weights are quadratics in their
+// coordinate and x = x_box + w u, y = y_box + w v (w the box width).  So the 36 node sums of a box follow
+// from the 21 moments sum u^i v^j with (i <= 4, j <= 2) or (i <= 2, j <= 4), and a point costs 21 LDS
+// atomics, not 36; the moments lie in [0, 1], so one fixed-point scale (2^50) serves them all and
+// up to 4096 of them sum below 2^62.  The node sums are formed from the moments in fp64 when the tile is
+// flushed, which is exact to fp64 rounding where the per-point products were rounded to fp32.
+constexpr int kMoments = 21;
+constexpr int kTileBoxes2 = kTileBoxes * kTileBoxes;
+__device__ __forceinline__ constexpr int moment_index(int i, int j) { return j <= 2 ? j * 5 + i : 15 + (j - 3) * 3 + i; }
 
 __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__restrict__ tile_xy,
                                                      const int4 *__restrict__ chunks,
                                                      const int *__restrict__ num_chunks, const LoopScalars *sc,
                                                      int slot, int n_boxes, LagrangeConsts lc,
                                                      float *__restrict__ w) {
-    constexpr int kTileNodes = kTileBoxes * kInterp;  // 21
-    constexpr int kPlane = kTileNodes * kTileNodes;
-    __shared__ unsigned long long acc[kTerms * kPlane];
+    __shared__ unsigned long long acc[kMoments * kTileBoxes2];  // one plane per moment
     const int nc = *num_chunks;
     const int c0 = (int)((long long)blockIdx.x * nc / gridDim.x);
     const int c1 = (int)((long long)(blockIdx.x + 1) * nc / gridDim.x);
     if (c0 >= c1) return;
     const int tid = threadIdx.x;
-    for (int e = tid; e < kTerms * kPlane; e += kSpreadThreads) acc[e] = 0ull;
+    for (int e = tid; e < kMoments * kTileBoxes2; e += kSpreadThreads) acc[e] = 0ull;
     const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
     const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    const SpreadScales fx = spread_scales(sc, slot);
+    const double to_fixed = 1125899906842624.0, from_fixed = 1.0 / 1125899906842624.0;  // 2^50
+    // Monomial coefficients of the Lagrange weights: L_m(t) = (t - s_k)(t - s_l) / denom_m.
+    double coef[kInterp][3];
+#pragma unroll
+    for (int m = 0; m < kInterp; ++m) {
+        const double sk = lc.spacing[(m + 1) % kInterp], sl = lc.spacing[(m + 2) % kInterp], d = lc.denom[m];
+        coef[m][0] = sk * sl / d;
+        coef[m][1] = -(sk + sl) / d;
+        coef[m][2] = 1.0 / d;
+    }
     // Unconditional, clamped loads: a chunk holds at least one point.
     auto fetch = [&](const int4 &ch, float2 (&pt)[2]) {
 #pragma unroll
@@ -434,43 +448,62 @@ __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             if (tid + u * kSpreadThreads < ch.z) {
-                const float x = pt[u].x, y = pt[u].y;
                 int bx, by;
-                float Lx[kInterp], Ly[kInterp];
-                bin_and_weights(x, bd, n_boxes, lc, bx, Lx);
-                bin_and_weights(y, bd, n_boxes, lc, by, Ly);
-                const float q3 = x * x + y * y;
-                const int nx = (bx - bx0) * kInterp, ny = (by - by0) * kInterp;
+                float pu[5], pv[5];
+                pu[0] = pv[0] = 1.0f;
+                bin_and_coord(pt[u].x, bd, n_boxes, bx, pu[1]);
+                bin_and_coord(pt[u].y, bd, n_boxes, by, pv[1]);
 #pragma unroll
-                for (int a = 0; a < kInterp; ++a) {
-#pragma unroll
-                    for (int b = 0; b < kInterp; ++b) {
-                        const float lw = Lx[a] * Ly[b];
-                        // One plane per term: the lanes of an atomic instruction all add to the same term, and
-                        // with the four terms of a node side by side they would only ever meet an eighth of the
-                        // LDS banks.
-                        unsigned long long *dst = acc + (nx + a) * kTileNodes + (ny + b);
-                        add_fixed(dst + 0 * kPlane, lw, fx.to_fixed[0]);
-                        add_fixed(dst + 1 * kPlane, lw * x, fx.to_fixed[1]);
-                        add_fixed(dst + 2 * kPlane, lw * y, fx.to_fixed[2]);
-                        add_fixed(dst + 3 * kPlane, lw * q3, fx.to_fixed[3]);
-                    }
+                for (int k = 2; k < 5; ++k) {
+                    pu[k] = pu[k - 1] * pu[1];
+                    pv[k] = pv[k - 1] * pv[1];
                 }
+                unsigned long long *dst = acc + (bx - bx0) * kTileBoxes + (by - by0);
+#pragma unroll
+                for (int j = 0; j < 5; ++j)
+#pragma unroll
+                    for (int i = 0; i < 5; ++i)
+                        if (j <= 2 || i <= 2)
+                            add_fixed(dst + moment_index(i, j) * kTileBoxes2, pu[i] * pv[j], to_fixed);
             }
         }
         ++in_tile;
         if (last || next_ch.x != cur_tile || in_tile == kChunksPerFlush) {
             __syncthreads();
-            for (int e = tid; e < kTerms * kPlane; e += kSpreadThreads) {
-                const long long v = (long long)acc[e];
-                if (v != 0) {
-                    acc[e] = 0ull;
-                    const int node = e % kPlane, t = e / kPlane;
-                    const int gx = bx0 * kInterp + node / kTileNodes, gy = by0 * kInterp + node % kTileNodes;
-                    if (gx < G && gy < G)
-                        atomicAdd(w + ((size_t)gx * G + gy) * kTerms + t, (float)((double)v * fx.from_fixed[t]));
-                }
+            // One thread per (box, node of the box): five sums over the nine monomial pairs, then the four terms.
+            for (int e = tid; e < kTileBoxes2 * kInterp * kInterp; e += kSpreadThreads) {
+                const int box = e / (kInterp * kInterp), a = (e / kInterp) % kInterp, b = e % kInterp;
+                const unsigned long long *src = acc + box;
+                if (src[0] == 0ull) continue;  // moment (0, 0) is the number of points in the box
+                const int bxl = box / kTileBoxes, byl = box % kTileBoxes;
+                const int gx = (bx0 + bxl) * kInterp + a, gy = (by0 + byl) * kInterp + b;
+                if (gx >= G || gy >= G) continue;
+                double M[kMoments];
+#pragma unroll
+                for (int m = 0; m < kMoments; ++m) M[m] = (double)(long long)src[m * kTileBoxes2] * from_fixed;
+                double s00 = 0.0, s10 = 0.0, s01 = 0.0, s20 = 0.0, s02 = 0.0;
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+#pragma unroll
+                    for (int j = 0; j < 3; ++j) {
+                        const double cc = coef[a][i] * coef[b][j];
+                        s00 += cc * M[moment_index(i, j)];
+                        s10 += cc * M[moment_index(i + 1, j)];
+                        s01 += cc * M[moment_index(i, j + 1)];
+                        s20 += cc * M[moment_index(i + 2, j)];
+                        s02 += cc * M[moment_index(i, j + 2)];
+                    }
+                const double bw = bd.box_width;
+                const double xl = box_lower(bx0 + bxl, bd), yl = box_lower(by0 + byl, bd);
+                float *out = w + ((size_t)gx * G + gy) * kTerms;
+                atomicAdd(out + 0, (float)s00);
+                atomicAdd(out + 1, (float)(xl * s00 + bw * s10));
+                atomicAdd(out + 2, (float)(yl * s00 + bw * s01));
+                atomicAdd(out + 3, (float)((xl * xl + yl * yl) * s00 + 2.0 * bw * (xl * s10 + yl * s01) +
+                                           bw * bw * (s20 + s02)));
             }
+            __syncthreads();
+            for (int e = tid; e < kMoments * kTileBoxes2; e += kSpreadThreads) acc[e] = 0ull;
             if (!last) __syncthreads();
             cur_tile = next_ch.x;
             in_tile = 0;
