@@ -160,6 +160,7 @@ def test_renumbering_is_invisible_to_the_caller(monkeypatch):
     (8195, 127, 16, 4),   # one dimension more: chunked matrix sweep
     (17000, 300, 30, 5),  # chunked matrix sweep on renumbered points, margin tried on a sample of query tiles
     (40000, 50, 40, 6),   # several column partitions and strips, clustered
+    (12000, 10, 1023, 3),  # the neighbour count of the reference's C++ default options
 ])
 def test_whole_pipeline_against_the_oracle(n, d, k, clusters):
     """RunTsne end to end (renumbering, kNN, P, eight gradient steps, numbering

@@ -375,6 +375,7 @@ def test_iterate_with_prepared_pattern(stages, c0_problem):
     (745, 864, 126),   # six candidate tiles: fewer than the workgroups a query tile could be split over
     (40, 3, 40),       # K == N, a single partial tile
     (2500, 33, 300),   # wide neighbour lists
+    (3000, 20, 1023),  # the reference's default neighbour count: the roomier list size no longer fits the LDS
 ])
 def test_knn_matrix_sweep_is_exact(stages, n, d, k):
     """The MFMA candidate sweep + exact re-rank gives the oracle's neighbours bit

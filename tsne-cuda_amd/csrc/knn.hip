@@ -1379,18 +1379,19 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     else if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
     const int num_tiles = div_up(N, kCT);
     const int bitmap_words = div_up(num_tiles, 32);
-    // Room for the candidates kept, as many again and one more tile where that fits: a list that is
-    // nearly full right after a selection would be selected again after every tile.
-    auto list_cap = [](int want) {
+    // Room for the candidates kept, as many again and one more tile where the LDS sort buffers of that
+    // size fit: a list that is nearly full right after a selection would be selected again after every tile.
+    const size_t tile_lds = chunked ? sizeof(float4) * kChunkFloat4 + sizeof(float) * D
+                                    : sizeof(float4) * 4 * ((ksteps + 3) / 4) * 64;
+    auto lds_with = [&](int cap) -> size_t {
+        return tile_lds + sizeof(u64) * 4 * cap + sizeof(unsigned int) * bitmap_words;
+    };
+    auto list_cap = [&](int want) {
         int cap = next_pow2(2 * want + kCT);
-        if (cap > 4096) cap = next_pow2(want + kCT);
+        if (cap > 4096 || lds_with(cap) > 150 * 1024) cap = next_pow2(want + kCT);
         return cap < 256 ? 256 : cap;
     };
-    auto sweep_lds = [&](int want) -> size_t {
-        const size_t tile = chunked ? sizeof(float4) * kChunkFloat4 + sizeof(float) * D
-                                    : sizeof(float4) * 4 * ((ksteps + 3) / 4) * 64;
-        return tile + sizeof(u64) * 4 * list_cap(want) + sizeof(unsigned int) * bitmap_words;
-    };
+    auto sweep_lds = [&](int want) -> size_t { return lds_with(list_cap(want)); };
     auto sweep_fits = [&](int want) { return list_cap(want) <= 4096 && sweep_lds(want) <= 150 * 1024; };
     int want = std::min(N - 1, (K - 1) + std::max(32, (K - 1) / 2));  // K' candidates kept per query
     const bool mfma_fits = sweep_fits(want);
