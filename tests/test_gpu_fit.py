@@ -202,3 +202,16 @@ def test_command_line_program(tmp_path):
     a, b = last[:300].mean(0), last[300:].mean(0)
     own = np.linalg.norm(last[:300] - a, axis=1) < np.linalg.norm(last[:300] - b, axis=1)
     assert own.mean() > 0.95
+
+
+def test_package_smoke_run_with_all_defaults(capfd):
+    """tsnecuda.test(): 5000 x 50 uniform random points (float64 input) with
+    every keyword at its default (perplexity 50, 32 neighbours, Gaussian start,
+    1000 steps), as src/python/tsnecuda/__init__.py:4-7 does."""
+    import tsnecuda
+    tsnecuda.test()
+    out = capfd.readouterr().out
+    assert "[Step 0] Avg. Gradient Norm:" in out and "total_time:" in out
+    # and the same call returns a finite float32 embedding
+    emb = tsnecuda.TSNE().fit_transform(np.random.default_rng(0).random((3000, 20)))
+    assert emb.shape == (3000, 2) and emb.dtype == np.float32 and np.isfinite(emb).all()
