@@ -199,27 +199,44 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 // has few enough entries that keeping all of them stays within want + slack, everything up to the
 // bin's upper edge is kept and that edge becomes the threshold.  A compaction in the middle of a sweep
 // only needs some threshold below which everything was kept; the last one of a query passes slack = 0.
+//
+// HALVES: the list is two regions of `half` entries, each appended to by one of the query's two lanes
+// (entries 0 .. c0-1 of the first, the rest of the *cnt entries in the second); the entries kept go back
+// alternately into the two regions (entry p to region p & 1, position p >> 1), so both keep room.
+template <bool HALVES = false>
 __device__ __forceinline__ int wave_select(u64 *list, int want, int *cnt, u64 *thr, u64 *buf, unsigned int *hist,
-                                           int lane, int slack = 0) {
+                                           int lane, int slack = 0, int half = 0, int c0 = 0) {
     __threadfence_block();  // this wave's appends to the list are complete
     const int n = *cnt;
     if (n < want) return n;
+    auto wr = [&](int p, u64 key) {
+        if (HALVES) list[(p & 1) * half + (p >> 1)] = key;
+        else list[p] = key;
+    };
     unsigned int lo = ~0u, hi = 0u;
     // Four loads in flight: the list comes from global memory and a load at a time would cost its latency each.
-    for (int e0 = lane; e0 < n; e0 += 4 * kWave) {
-        u64 key[4];
+    auto load_run = [&](const u64 *src, int count, u64 *dst) {
+        for (int e0 = lane; e0 < count; e0 += 4 * kWave) {
+            u64 key[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) key[u] = list[min(e0 + u * kWave, n - 1)];
+            for (int u = 0; u < 4; ++u) key[u] = src[min(e0 + u * kWave, count - 1)];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int e = e0 + u * kWave;
-            if (e < n) {
-                buf[e] = key[u];
-                const unsigned int bits = (unsigned int)(key[u] >> 32);
-                lo = min(lo, bits);
-                hi = max(hi, bits);
+            for (int u = 0; u < 4; ++u) {
+                const int e = e0 + u * kWave;
+                if (e < count) {
+                    dst[e] = key[u];
+                    const unsigned int bits = (unsigned int)(key[u] >> 32);
+                    lo = min(lo, bits);
+                    hi = max(hi, bits);
+                }
             }
         }
+    };
+    if (HALVES) {
+        load_run(list, c0, buf);
+        load_run(list + half, n - c0, buf + c0);
+    } else {
+        load_run(list, n, buf);
     }
 #pragma unroll
     for (int m = kWave / 2; m > 0; m >>= 1) {
@@ -260,7 +277,7 @@ __device__ __forceinline__ int wave_select(u64 *list, int want, int *cnt, u64 *t
                     const u64 key = e < n ? buf[e] : 0ull;
                     const bool keep = e < n && (unsigned int)(key >> 32) <= dedge;
                     const u64 m = __ballot(keep);
-                    if (keep) list[base + __popcll(m & below_lanes)] = key;
+                    if (keep) wr(base + __popcll(m & below_lanes), key);
                     base += __popcll(m);
                 }
                 if (lane == 0) {
@@ -283,10 +300,10 @@ __device__ __forceinline__ int wave_select(u64 *list, int want, int *cnt, u64 *t
         const unsigned int bits = (unsigned int)(key >> 32);
         const bool lt = e < n && bits < dstar, eq = e < n && bits == dstar;
         const u64 m_lt = __ballot(lt), m_eq = __ballot(eq);
-        if (lt) list[base_lt + __popcll(m_lt & below)] = key;
+        if (lt) wr(base_lt + __popcll(m_lt & below), key);
         if (eq) {
             const int k = base_eq + __popcll(m_eq & below);
-            if (k < need_eq) list[c_lt + k] = key;
+            if (k < need_eq) wr(c_lt + k, key);
         }
         base_lt += __popcll(m_lt);
         base_eq += __popcll(m_eq);
@@ -592,6 +609,7 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
     unsigned int *bitmap = reinterpret_cast<unsigned int *>(reinterpret_cast<u64 *>(a_lds + kTileFloat4) + 4 * (size_t)cap);
     __shared__ u64 thr[kMQ];
     __shared__ int cnt[kMQ];
+    __shared__ int fill[256];  // entries in each lane's region of its query's list
     __shared__ float qcenter[128];
     __shared__ unsigned int hist_all[4][kWave];
     __shared__ float tmax_part[2];
@@ -624,6 +642,42 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
             thr[tid] = ~0ull;
             cnt[tid] = 0;
         }
+        // A query's list is two regions of cap / 2 entries, one per lane of the pair that shares the query:
+        // a lane appends to its own region with a counter of its own, so an append needs neither a count of
+        // the passing elements nor an atomic to reserve room.
+        const int half = cap >> 1;
+        // The counter is a register; around a selection it passes through LDS (fill[tid]), where the whole
+        // wave can read and set it.
+        int my_n = 0;
+        // Selection over the list of query b of this wave (all lanes take part); returns the caller's updated
+        // counter: the entries kept go back alternately into the two regions.
+        // With fewer than `want` entries nothing is dropped; `spread` then still deals them out alternately,
+        // for a query whose one region fills up while the other stays empty (and for the output pass, which
+        // reads that order).
+        auto select_query = [&](int b, int slack, bool spread) {
+            const int ql = wave * 32 + b;
+            const int c0n = fill[wave * 64 + b], c1n = fill[wave * 64 + b + 32];
+            int kept = c0n + c1n;
+            if (kept < want) {
+                if (!spread) return;
+                u64 *lq = list + (size_t)ql * cap;
+                __threadfence_block();  // this wave's appends to the list are complete
+                for (int e = lane; e < kept; e += kWave) sortbuf[e] = e < c0n ? lq[e] : lq[half + e - c0n];
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                for (int e = lane; e < kept; e += kWave) lq[(e & 1) * half + (e >> 1)] = sortbuf[e];
+                __threadfence_block();
+            } else {
+                if (lane == 0) cnt[ql] = kept;
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                kept = wave_select<true>(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf,
+                                         hist_all[wave], lane, slack, half, c0n);
+            }
+            if (lane == 0) {
+                fill[wave * 64 + b] = (kept + 1) >> 1;
+                fill[wave * 64 + b + 32] = kept >> 1;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        };
         // B operand from the same packed layout (query tiles and candidate tiles coincide: kMQ == kCT):
         // -2 q_d for the real dimensions, 1 for the |c|^2 row, 0 elsewhere.
         float bq[4 * S4];
@@ -684,9 +738,8 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                 for (int v = 1; v + 1 < 16; v += 2) best = min3(best, acc1[v], acc1[v + 1]);
                 best = fminf(best, acc1[15]);
                 // A query meets about K' ln(N / K') passing candidates during the sweep and the 64 lanes
-                // serve different queries, so most block pairs have some lane that passes.  A lane first
-                // counts its passing elements (compare + add-with-carry each), reserves that many list
-                // slots with one LDS atomic and then stores the keys: no atomic round trip per element.
+                // serve different queries, so most block pairs have some lane that passes.  A passing lane
+                // stores its keys one after the other at the end of its own region of the query's list.
                 // The test is on the distance alone; an element that ties with the threshold's distance
                 // but not its index is appended too and sorted out by the next compaction.
                 if (best <= limit_d) {
@@ -702,30 +755,34 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                         }
                     }
                     const float lim = q < N ? limit_d : -INFINITY;
-                    int n = 0;
+                    u64 *const dst0 = list + ((wave * 32 + qn) * cap + kh * half + my_n);
+                    u64 *dst = dst0;
 #pragma unroll
-                    for (int e = 0; e < 32; ++e) n += ((e < 16 ? acc0[e & 15] : acc1[e & 15]) <= lim) ? 1 : 0;
-                    if (n != 0) {
-                        const int slot = atomicAdd(&cnt[wave * 32 + qn], n);
-                        u64 *dst = list + (size_t)(wave * 32 + qn) * cap + slot;
-                        float lim2 = lim;
-                        asm volatile("" : "+v"(lim2));  // compare again rather than keep 32 lane masks alive
-#pragma unroll
-                        for (int e = 0; e < 32; ++e) {
-                            const float dist = e < 16 ? acc0[e & 15] : acc1[e & 15];
-                            if (dist <= lim2) *dst++ = pack_key(dist, jbase + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
+                    for (int e = 0; e < 32; ++e) {
+                        const float dist = e < 16 ? acc0[e & 15] : acc1[e & 15];
+                        if (dist <= lim) {
+                            int jb = jbase;
+                            asm volatile("" : "+v"(jb));  // the index is formed here, not held in 32 registers
+                            *dst++ = pack_key(dist, jb + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
                         }
                     }
+                    my_n += (int)(dst - dst0);
                 }
             }
             // Lists that a further tile could overflow are compacted by their own wave, right away.
             {
-                u64 crowded = __ballot(cnt[wave * 32 + qn] > args.trigger) & 0xffffffffull;  // lanes l, l+32 share a query
-                while (crowded) {
-                    const int ql = wave * 32 + (__ffsll((long long)crowded) - 1);
-                    crowded &= crowded - 1;
-                    wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane,
-                                args.select_slack);
+                // (a region takes at most 64 entries per tile)
+                u64 crowded = __ballot(my_n > half - kCT / 2);
+                crowded = (crowded | (crowded >> 32)) & 0xffffffffull;  // lanes l, l+32 share a query
+                if (crowded) {
+                    fill[tid] = my_n;
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                    while (crowded) {
+                        const int b = __ffsll((long long)crowded) - 1;
+                        crowded &= crowded - 1;
+                        select_query(b, args.select_slack, true);
+                    }
+                    my_n = fill[tid];
                 }
             }
             __syncthreads();  // all waves are done with tile `buf`
@@ -765,11 +822,11 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
             if (nxt < 0 && home && (h0 > 0 || h1 < T - 1)) {
                 home = false;
                 // Thresholds from what the neighbourhood held.
-                for (int b = 0; b < 32; ++b) {
-                    const int ql = wave * 32 + b;
-                    if (q0 + ql < N)
-                        wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
-                }
+                fill[tid] = my_n;
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                for (int b = 0; b < 32; ++b)
+                    if (q0 + wave * 32 + b < N) select_query(b, 0, false);
+                my_n = fill[tid];
                 for (int w = tid; w < args.bitmap_words; w += 256) bitmap[w] = 0u;
                 if (tid < D) qcenter[tid] = args.centers_t[(size_t)tid * T + qt];
                 __syncthreads();
@@ -802,13 +859,17 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
         }
         if (tid == 0) atomicAdd(args.tiles_swept, (unsigned long long)swept);
         // Final ordering and output, every wave for its own 32 queries.
+        fill[tid] = my_n;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         for (int b = 0; b < 32; ++b) {
             const int ql = wave * 32 + b;
             const int qq = q0 + ql;
             if (qq >= N) break;
-            const int n = wave_select(list + (size_t)ql * cap, want, &cnt[ql], &thr[ql], sortbuf, hist_all[wave], lane);
+            select_query(b, 0, true);
+            const int n = fill[wave * 64 + b] + fill[wave * 64 + b + 32];
+            const u64 *lq = list + (size_t)ql * cap;  // entry e of the n kept: region e & 1, position e >> 1
             for (int e = lane; e < want; e += kWave)
-                cand[(size_t)qq * want + e] = e < n ? key_index(list[(size_t)ql * cap + e]) : -1;
+                cand[(size_t)qq * want + e] = e < n ? key_index(lq[(e & 1) * half + (e >> 1)]) : -1;
             // Every candidate that was dropped, by a compaction or by the filter, had a distance >= the
             // threshold of the moment, and thresholds only decrease.
             if (lane == 0) tau[qq] = thr[ql] == ~0ull ? INFINITY : key_distance(thr[ql]);
