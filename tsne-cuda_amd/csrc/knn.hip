@@ -730,13 +730,19 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                 // Register v of lane l holds candidate row 8*(v/4) + 4*(l/32) + v%4 of the block, query column l%32.
                 // Smallest of the lane's 32 values, three operands per instruction (the accumulators are
                 // never signalling NaNs, so the library fminf's quieting moves are left out).
-                float best = min3(acc0[0], acc0[1], acc0[2]);
+                // The minima of the four runs of eight registers are kept: the filter skips a run in which no
+                // lane of the wave has a passing element.
+                float run_min[4];
 #pragma unroll
-                for (int v = 3; v + 1 < 16; v += 2) best = min3(best, acc0[v], acc0[v + 1]);
-                best = min3(best, acc0[15], acc1[0]);
-#pragma unroll
-                for (int v = 1; v + 1 < 16; v += 2) best = min3(best, acc1[v], acc1[v + 1]);
-                best = fminf(best, acc1[15]);
+                for (int g = 0; g < 4; ++g) {
+                    const v16f &a = g < 2 ? acc0 : acc1;
+                    const int o = 8 * (g & 1);
+                    float m = min3(a[o], a[o + 1], a[o + 2]);
+                    m = min3(m, a[o + 3], a[o + 4]);
+                    m = min3(m, a[o + 5], a[o + 6]);
+                    run_min[g] = fminf(m, a[o + 7]);
+                }
+                const float best = fminf(min3(run_min[0], run_min[1], run_min[2]), run_min[3]);
                 // A query meets about K' ln(N / K') passing candidates during the sweep and the 64 lanes
                 // serve different queries, so most block pairs have some lane that passes.  A passing lane
                 // stores its keys one after the other at the end of its own region of the query's list.
@@ -758,12 +764,18 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                     u64 *const dst0 = list + ((wave * 32 + qn) * cap + kh * half + my_n);
                     u64 *dst = dst0;
 #pragma unroll
-                    for (int e = 0; e < 32; ++e) {
-                        const float dist = e < 16 ? acc0[e & 15] : acc1[e & 15];
-                        if (dist <= lim) {
-                            int jb = jbase;
-                            asm volatile("" : "+v"(jb));  // the index is formed here, not held in 32 registers
-                            *dst++ = pack_key(dist, jb + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
+                    for (int g = 0; g < 4; ++g) {
+                        // (the minima are from before the exclusions above: lower bounds, which is all this needs)
+                        if (__ballot(run_min[g] <= lim) == 0) continue;
+#pragma unroll
+                        for (int v = 0; v < 8; ++v) {
+                            const int e = 8 * g + v;
+                            const float dist = e < 16 ? acc0[e & 15] : acc1[e & 15];
+                            if (dist <= lim) {
+                                int jb = jbase;
+                                asm volatile("" : "+v"(jb));  // the index is formed here, not held in 32 registers
+                                *dst++ = pack_key(dist, jb + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
+                            }
                         }
                     }
                     my_n += (int)(dst - dst0);
