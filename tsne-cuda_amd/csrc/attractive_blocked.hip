@@ -10,13 +10,14 @@
 //   * columns into partitions of kPartPoints points,
 //   * inside a strip the entries are grouped by partition; an entry is 8 bytes:
 //     the probability and a packed (column within partition | row within strip),
-//   * a strip's work list names, in order, runs ("items") of at most
-//     kItemEntries entries that share a partition; partitions the strip never
-//     references do not appear in it.
+//   * a strip's work list cuts its entries into "items" of kItemEntries
+//     consecutive entries and marks, per item, where the run of the next
+//     partition starts inside it (at most one such start per item: an item
+//     ends early where a second one would fall into it).
 //
 // A workgroup keeps its strip's positions and force accumulators in LDS and
-// walks its work list; the partition an item refers to is staged in LDS, so
-// every neighbour gather is an LDS read and every accumulation an LDS atomic.
+// walks its work list; the partition the current entries refer to is staged in
+// LDS, so every neighbour gather is an LDS read and every accumulation an LDS atomic.
 // HBM sees the 8 bytes per entry once, coalesced, plus the positions of the
 // referenced partitions once per workgroup (mostly served by the L2).
 //
@@ -90,6 +91,7 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
                                                          int seg_stride, float *__restrict__ ent_p,
                                                          unsigned int *__restrict__ seg, float *__restrict__ p_max) {
     __shared__ unsigned int cursor[kMaxParts];
+    __shared__ unsigned int run_start[kMaxParts];  // first entry of the k-th referenced partition's run
     __shared__ unsigned int scan[kBlock];
     const int tid = threadIdx.x;
     const int strip = blockIdx.x;
@@ -107,36 +109,44 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
     scan_slots(mine, first, scan, tid);
 #pragma unroll
     for (int i = 0; i < kSlotsPerThread; ++i) cursor[tid * kSlotsPerThread + i] = first[i];
-    // Work list of the strip: every referenced partition contributes ceil(entries / kItemEntries) items
-    // (runs of at most kItemEntries entries that share the partition); a second scan, over the item counts.
-    unsigned int items[kSlotsPerThread], item_slot[kSlotsPerThread];
-#pragma unroll
-    for (int i = 0; i < kSlotsPerThread; ++i) items[i] = (mine[i] + kItemEntries - 1u) / kItemEntries;
-    const unsigned int n_items_total = scan_slots(items, item_slot, scan, tid);
     // Layout of a strip's list: {item count, fresh count, -, -}, then one record per item
-    // {first entry, end entry, partition, 1 if the item opens the partition}, kPadItems empty records,
-    // then the partitions in the order they are opened.
+    // {first entry, end entry, first entry of the partition the item opens, 1 if it opens one}, kPadItems
+    // empty records, then the partitions in the order they are opened.
     unsigned int *hdr = seg + (size_t)strip * seg_stride;
     uint4 *records = reinterpret_cast<uint4 *>(hdr + 4);
     unsigned int *fresh_parts = hdr + 4 + 4 * (max_items + kPadItems);
-#pragma unroll
-    for (int i = 0; i < kSlotsPerThread; ++i)
-        for (unsigned int it = 0; it < items[i]; ++it) {
-            const unsigned int b = first[i] + it * kItemEntries;
-            records[item_slot[i] + it] = make_uint4(b, min(first[i] + mine[i], b + kItemEntries),
-                                                    (unsigned int)(tid * kSlotsPerThread + i), it == 0 ? 1u : 0u);
-        }
-    if (tid < kPadItems) records[n_items_total + tid] = make_uint4(count, count, 0u, 0u);
-    if (tid == 0) hdr[0] = n_items_total;
-    // Third scan, over the "referenced at all" flags: the order in which partitions are opened.
+    // Second scan, over the "referenced at all" flags: the order in which partitions are opened.
     unsigned int flag[kSlotsPerThread], order[kSlotsPerThread];
 #pragma unroll
     for (int i = 0; i < kSlotsPerThread; ++i) flag[i] = mine[i] > 0u ? 1u : 0u;
     const unsigned int n_fresh = scan_slots(flag, order, scan, tid);
 #pragma unroll
     for (int i = 0; i < kSlotsPerThread; ++i)
-        if (flag[i]) fresh_parts[order[i]] = (unsigned int)(tid * kSlotsPerThread + i);
+        if (flag[i]) {
+            fresh_parts[order[i]] = (unsigned int)(tid * kSlotsPerThread + i);
+            run_start[order[i]] = first[i];
+        }
     if (tid == 0) hdr[1] = n_fresh;
+    __syncthreads();
+    // Work list of the strip: items of kItemEntries consecutive entries, whatever partitions they belong to.
+    // An item may contain the start of one partition's run (the force kernel switches partitions in the
+    // middle of it); where a second run would start inside an item, the item ends there instead.  Every
+    // strip therefore has about entries / kItemEntries items, however its entries spread over the partitions.
+    if (tid == 0) {
+        unsigned int x = 0u, next_run = 0u, n_items = 0u;
+        while (x < count) {
+            unsigned int limit = min(x + kItemEntries, count), opens = limit, has = 0u;
+            if (next_run < n_fresh && run_start[next_run] < limit) {
+                opens = run_start[next_run++];
+                has = 1u;
+                if (next_run < n_fresh && run_start[next_run] < limit) limit = run_start[next_run];
+            }
+            records[n_items++] = make_uint4(x, limit, opens, has);
+            x = limit;
+        }
+        for (int i = 0; i < kPadItems; ++i) records[n_items + i] = make_uint4(count, count, count, 0u);
+        hdr[0] = n_items;
+    }
     // Entries are visited neighbour slot by neighbour slot, so that neighbouring positions of a
     // partition's run belong to different rows: a wave of the force kernel then spreads its LDS
     // atomics over many accumulators even when most neighbours of a row share one partition.
@@ -170,10 +180,10 @@ __global__ void clear_pmax_kernel(float *p_max) {
 // (three rotating register sets, two items in flight, all loads unconditional so
 // that the outstanding-load counts the compiler works with are exact) and do the
 // LDS gathers and accumulations.  Waves 12-15 only stage partitions: they hold
-// the next partition in registers, and when the streaming waves reach an item
-// that opens it, everybody meets at a barrier, the staging waves write it to LDS,
+// the next two partitions in registers, and when the streaming waves reach the entry
+// that opens one, everybody meets at a barrier, the staging waves write it to LDS,
 // a second barrier releases the streaming waves, and the staging waves go and
-// fetch the partition after that.  A barrier does not wait for memory, so the
+// fetch the partition after the next.  A barrier does not wait for memory, so the
 // entry stream never drains at a partition switch.  Both roles execute two
 // barriers per opened partition and one at the end.
 // ---------------------------------------------------------------------------
@@ -235,20 +245,34 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         const Quad *yxy4 = reinterpret_cast<const Quad *>(yxy);
         Quad *part4 = reinterpret_cast<Quad *>(part);
         const int last_pair_all = (N - 1) / 2;  // yxy is padded, so a pair may run one point past N
-        Quad stage[kPartLoads];
-        auto fetch = [&](int k) {
-            const int p = (int)fresh_parts[k];
+        // Two partitions ahead, in two register sets: a strip that references many partitions opens one every
+        // microsecond or so, which is less than a fetch takes.  The fetches are unconditional (past the last
+        // partition they repeat it) so that the compiler's outstanding-load counts are exact and a write to LDS
+        // waits for its own set only.
+        Quad stage_a[kPartLoads], stage_b[kPartLoads];
+        auto fetch = [&](Quad (&stage)[kPartLoads], int k) {
+            const int p = (int)fresh_parts[min(k, n_fresh - 1)];
 #pragma unroll
             for (int u = 0; u < kPartLoads; ++u)
                 stage[u] = yxy4[min(p * (kPartPoints / 2) + lt + u * kLoadThreads, last_pair_all)];
         };
-        if (n_fresh > 0) fetch(0);
-        for (int k = 0; k < n_fresh; ++k) {
+        auto publish = [&](const Quad (&stage)[kPartLoads]) {
             __syncthreads();  // the streaming waves are done with the partition in LDS
 #pragma unroll
             for (int u = 0; u < kPartLoads; ++u) part4[lt + u * kLoadThreads] = stage[u];
-            __syncthreads();  // partition k is staged
-            if (k + 1 < n_fresh) fetch(k + 1);
+            __syncthreads();  // the partition is staged
+        };
+        if (n_fresh > 0) {
+            fetch(stage_a, 0);
+            fetch(stage_b, 1);
+            int k = 0;
+            for (; k + 1 < n_fresh; k += 2) {
+                publish(stage_a);
+                fetch(stage_a, k + 2);
+                publish(stage_b);
+                fetch(stage_b, k + 3);
+            }
+            if (k < n_fresh) publish(stage_a);
         }
     } else {
         // ---- streaming waves ----
@@ -256,7 +280,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         const Entry *ent = reinterpret_cast<const Entry *>(ent_p);
         struct PhaseRegs {
             Entry en[kPrefetch];
-            Record rec;  // {first entry, end entry, partition, opens a partition}
+            Record rec;  // {first entry, end entry, first entry of the partition it opens, opens a partition}
         };
         const size_t last_entry = (size_t)nrows * K - 1;
         auto issue = [&](PhaseRegs &R) {
@@ -266,21 +290,29 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
                 R.en[k] = ent[base + t];
             }
         };
+        auto entry_force = [&](const Entry &en) {
+            const unsigned int rl = en.y >> kColBits;
+            const float2 yj = part[en.y & ((1u << kColBits) - 1u)];
+            const float2 y0 = yi[rl];
+            const float dx = y0.x - yj.x, dy = y0.y - yj.y;
+            const float w = __uint_as_float(en.x) * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
+            add_force(acc, rl, w * dx, w * dy, scale);
+        };
+        // Entries [rec.x, rec.z) of an item belong to the partition in LDS; when the item opens a partition
+        // (rec.w), the rest, [rec.z, rec.y), belongs to that one (otherwise rec.z == rec.y).
         auto consume = [&](PhaseRegs &R) {
-            if (R.rec.w) {
-                __syncthreads();  // everyone is done with the previous partition
-                __syncthreads();  // the staging waves have written the new one
-            }
 #pragma unroll
             for (int k = 0; k < kPrefetch; ++k) {
                 const unsigned int t = R.rec.x + tid + k * kStreamThreads;
-                if (t < R.rec.y) {
-                    const unsigned int rl = R.en[k].y >> kColBits;
-                    const float2 yj = part[R.en[k].y & ((1u << kColBits) - 1u)];
-                    const float2 y0 = yi[rl];
-                    const float dx = y0.x - yj.x, dy = y0.y - yj.y;
-                    const float w = __uint_as_float(R.en[k].x) * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
-                    add_force(acc, rl, w * dx, w * dy, scale);
+                if (t < R.rec.z) entry_force(R.en[k]);
+            }
+            if (R.rec.w) {
+                __syncthreads();  // everyone is done with the previous partition
+                __syncthreads();  // the staging waves have written the new one
+#pragma unroll
+                for (int k = 0; k < kPrefetch; ++k) {
+                    const unsigned int t = R.rec.x + tid + k * kStreamThreads;
+                    if (t >= R.rec.z && t < R.rec.y) entry_force(R.en[k]);
                 }
             }
         };
@@ -356,7 +388,7 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     p->strip_rows = strip_rows;
     p->n_strips = div_up(N, strip_rows);
     p->n_parts = n_parts;
-    // A strip's work list: one item per referenced partition plus one per further kItemEntries entries.
+    // A strip's work list: one item per kItemEntries entries, plus at most one early end per referenced partition.
     p->max_items = n_parts + (int)(((int64_t)strip_rows * K) / kItemEntries) + 1;
     p->seg_stride = 4 + 4 * (p->max_items + kPadItems) + ((n_parts + 3) & ~3);
     const size_t nnz = (size_t)N * K;
