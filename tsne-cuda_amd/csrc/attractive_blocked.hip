@@ -10,13 +10,11 @@
 //   * columns into partitions of kPartPoints points,
 //   * inside a strip the entries are grouped by partition; an entry is 8 bytes:
 //     the probability and a packed (column within partition | row within strip),
-//   * a strip's work list cuts its entries into "items" of kItemEntries
-//     consecutive entries and marks, per item, where the run of the next
-//     partition starts inside it (at most one such start per item: an item
-//     ends early where a second one would fall into it).
+//   * a strip's list names the partitions it references, in order, and the
+//     entry at which each partition's run starts.
 //
 // A workgroup keeps its strip's positions and force accumulators in LDS and
-// walks its work list; the partition the current entries refer to is staged in
+// walks its entries; the partition the current entries refer to is staged in
 // LDS, so every neighbour gather is an LDS read and every accumulation an LDS atomic.
 // HBM sees the 8 bytes per entry once, coalesced, plus the positions of the
 // referenced partitions once per workgroup (mostly served by the L2).
@@ -36,19 +34,22 @@ namespace tsnehip {
 
 namespace {
 
-constexpr int kColBits = 12;
-constexpr int kPartPoints = 4096;   // == 1 << kColBits; 32 KB of (x, y) pairs
-constexpr int kStripMax = 3968;     // rows per strip: 31 KB of positions + 62 KB of accumulators; with the
-                                    // partition 125 KB, which leaves 35 KB of a CU's LDS to the kernels of the
+constexpr int kColBits = 11;
+constexpr int kPartPoints = 2048;   // == 1 << kColBits; 16 KB of (x, y) pairs, two of them in LDS
+constexpr int kStripMax = 3968;     // rows per strip: 31 KB of positions + 62 KB of accumulators; with the two
+                                    // partitions 125 KB, which leaves 35 KB of a CU's LDS to the kernels of the
                                     // repulsive chain that run beside this one
 constexpr double kRoundMagic = 6755399441055744.0;  // 1.5 * 2^52: adding it rounds a double to an integer
 constexpr int kBlock = 1024;
-constexpr int kMaxParts = 4096;     // column partitions: up to 16.7 M points
+constexpr int kMaxParts = 8192;     // column partitions: up to 16.7 M points
 constexpr int kPrefetch = 4;        // entries per thread in one work item
 constexpr int kStreamThreads = 768; // force kernel: waves 0-11 stream entries ...
+constexpr int kStreamWaves = kStreamThreads / kWave;
 constexpr int kLoadThreads = kBlock - kStreamThreads;  // ... waves 12-15 stage the partitions
+constexpr int kLoadWaves = kLoadThreads / kWave;
 constexpr unsigned int kItemEntries = kPrefetch * kStreamThreads;
-constexpr int kPadItems = 4;        // empty records after a strip's last item: the pipelined loop needs no guards
+constexpr int kSpinLimit = 1 << 18; // polls of an LDS counter before a wave gives up waiting (about ten milliseconds;
+                                    // a wait normally ends within a microsecond): every wave reaches the kernel's end
 
 // ---------------------------------------------------------------------------
 // Re-blocking: one workgroup per strip.  Histogram of the strip's entries over
@@ -87,11 +88,10 @@ __device__ __forceinline__ unsigned int scan_slots(const unsigned int (&value)[k
 }
 
 __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
-                                                         int N, int K, int strip_rows, int max_items,
+                                                         int N, int K, int strip_rows, int list_words,
                                                          int seg_stride, float *__restrict__ ent_p,
                                                          unsigned int *__restrict__ seg, float *__restrict__ p_max) {
     __shared__ unsigned int cursor[kMaxParts];
-    __shared__ unsigned int run_start[kMaxParts];  // first entry of the k-th referenced partition's run
     __shared__ unsigned int scan[kBlock];
     const int tid = threadIdx.x;
     const int strip = blockIdx.x;
@@ -109,12 +109,12 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
     scan_slots(mine, first, scan, tid);
 #pragma unroll
     for (int i = 0; i < kSlotsPerThread; ++i) cursor[tid * kSlotsPerThread + i] = first[i];
-    // Layout of a strip's list: {item count, fresh count, -, -}, then one record per item
-    // {first entry, end entry, first entry of the partition the item opens, 1 if it opens one}, kPadItems
-    // empty records, then the partitions in the order they are opened.
+    // Layout of a strip's list: {-, partitions referenced, -, -}, then for the k-th referenced partition the
+    // first entry of its run (n_parts + 4 words, unused ones hold ~0), then the partitions themselves in the
+    // same order (n_parts words).
     unsigned int *hdr = seg + (size_t)strip * seg_stride;
-    uint4 *records = reinterpret_cast<uint4 *>(hdr + 4);
-    unsigned int *fresh_parts = hdr + 4 + 4 * (max_items + kPadItems);
+    unsigned int *run_start = hdr + 4;
+    unsigned int *fresh_parts = run_start + list_words;
     // Second scan, over the "referenced at all" flags: the order in which partitions are opened.
     unsigned int flag[kSlotsPerThread], order[kSlotsPerThread];
 #pragma unroll
@@ -126,27 +126,8 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
             fresh_parts[order[i]] = (unsigned int)(tid * kSlotsPerThread + i);
             run_start[order[i]] = first[i];
         }
+    for (unsigned int b = n_fresh + tid; b < (unsigned int)list_words; b += kBlock) run_start[b] = ~0u;
     if (tid == 0) hdr[1] = n_fresh;
-    __syncthreads();
-    // Work list of the strip: items of kItemEntries consecutive entries, whatever partitions they belong to.
-    // An item may contain the start of one partition's run (the force kernel switches partitions in the
-    // middle of it); where a second run would start inside an item, the item ends there instead.  Every
-    // strip therefore has about entries / kItemEntries items, however its entries spread over the partitions.
-    if (tid == 0) {
-        unsigned int x = 0u, next_run = 0u, n_items = 0u;
-        while (x < count) {
-            unsigned int limit = min(x + kItemEntries, count), opens = limit, has = 0u;
-            if (next_run < n_fresh && run_start[next_run] < limit) {
-                opens = run_start[next_run++];
-                has = 1u;
-                if (next_run < n_fresh && run_start[next_run] < limit) limit = run_start[next_run];
-            }
-            records[n_items++] = make_uint4(x, limit, opens, has);
-            x = limit;
-        }
-        for (int i = 0; i < kPadItems; ++i) records[n_items + i] = make_uint4(count, count, count, 0u);
-        hdr[0] = n_items;
-    }
     // Entries are visited neighbour slot by neighbour slot, so that neighbouring positions of a
     // partition's run belong to different rows: a wave of the force kernel then spreads its LDS
     // atomics over many accumulators even when most neighbours of a row share one partition.
@@ -173,19 +154,32 @@ __global__ void clear_pmax_kernel(float *p_max) {
 }
 
 // ---------------------------------------------------------------------------
-// One workgroup per strip; dynamic LDS: part[kPartPoints] float2, then
+// One workgroup per strip; dynamic LDS: part[2][kPartPoints] float2, then
 // yi[kStripMax] float2, then acc_x[kStripMax] and acc_y[kStripMax], 64-bit fixed point.
 //
-// The waves have two roles.  Waves 0-11 stream the strip's entries item by item
-// (three rotating register sets, two items in flight, all loads unconditional so
-// that the outstanding-load counts the compiler works with are exact) and do the
-// LDS gathers and accumulations.  Waves 12-15 only stage partitions: they hold
-// the next two partitions in registers, and when the streaming waves reach the entry
-// that opens one, everybody meets at a barrier, the staging waves write it to LDS,
-// a second barrier releases the streaming waves, and the staging waves go and
-// fetch the partition after the next.  A barrier does not wait for memory, so the
-// entry stream never drains at a partition switch.  Both roles execute two
-// barriers per opened partition and one at the end.
+// The waves have two roles.  Waves 0-11 stream the strip's entries in items of
+// kItemEntries (three rotating register sets, two items in flight, all loads
+// unconditional so that the outstanding-load counts the compiler works with are
+// exact) and do the LDS gathers and accumulations.  Waves 12-15 only stage
+// partitions: the k-th partition the strip references goes into LDS buffer
+// k & 1, the two after the one being written wait in registers.
+//
+// No barrier separates the roles, only two counters per LDS buffer b:
+//   staged[b]   += 1 by every staging wave once its part of a partition is written
+//                  to b; a streaming wave enters run k when
+//                  staged[k & 1] >= kLoadWaves * (k / 2 + 1),
+//   released[b] += 1 by every streaming wave that leaves a run in b; a staging wave
+//                  overwrites buffer k & 1 with partition k once
+//                  released[k & 1] >= kStreamWaves * (k / 2), i.e. all streaming
+//                  waves have left partition k - 2.
+// Partition k + 2 is only written after every streaming wave has left partition k,
+// which they only entered after every staging wave had written it: a buffer's
+// counters never run ahead by a generation, so the thresholds are exact.
+// A streaming wave therefore never waits for another streaming wave, and waits for
+// the staging waves only when they are less than one partition ahead.  The LDS
+// executes one wave's operations in order, so a counter update that follows a
+// wave's reads or writes of a buffer is seen after them; the counters only grow.
+// Every wait is a bounded poll.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int rl, float vx, float vy,
                                           double scale) {
@@ -199,31 +193,50 @@ __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int 
     atomicAdd(&acc[kStripMax + rl], (unsigned long long)iy);
 }
 
+// Polls *counter until it reaches `need` (or kSpinLimit polls have passed).  The compiler barriers keep the
+// buffer accesses of the caller on their side of the wait.
+__device__ __forceinline__ void wait_for_count(const unsigned int *counter, unsigned int need) {
+    asm volatile("" ::: "memory");
+    for (int spin = 0; spin < kSpinLimit; ++spin) {
+        if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= need) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
+    asm volatile("" ::: "memory");
+}
+
+// One count from this wave, after everything it has issued to the LDS so far.
+__device__ __forceinline__ void count_wave(unsigned int *counter, int lane) {
+    asm volatile("" ::: "memory");
+    if (lane == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    asm volatile("" ::: "memory");
+}
+
 __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float *__restrict__ ent_p,
                                                                     const unsigned int *__restrict__ seg,
                                                                     const float2 *__restrict__ yxy,
                                                                     const float *__restrict__ p_max,
                                                                     float *__restrict__ attr, int N, int K,
-                                                                    int strip_rows, int max_items, int seg_stride) {
+                                                                    int strip_rows, int list_words, int seg_stride) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    float2 *part = reinterpret_cast<float2 *>(lds_raw);
-    float2 *yi = part + kPartPoints;
+    float2 *part = reinterpret_cast<float2 *>(lds_raw);  // two buffers of kPartPoints
+    float2 *yi = part + 2 * kPartPoints;
     unsigned long long *acc = reinterpret_cast<unsigned long long *>(yi + kStripMax);
+    __shared__ unsigned int staged[2], released[2];
 
     const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
     const int strip = blockIdx.x;
     const int row0 = strip * strip_rows;
     const int nrows = min(strip_rows, N - row0);
     const size_t base = (size_t)row0 * K;
-    // The work list is read through the constant address space: it is never written while this
+    // The list is read through the constant address space: it is never written while this
     // kernel runs, and constant-space loads at uniform addresses are scalar loads, which do not
     // queue behind the vector loads in flight.
     typedef const __attribute__((address_space(4))) unsigned int *ConstWords;
-    typedef unsigned int Record __attribute__((ext_vector_type(4)));
     ConstWords hdr = (ConstWords)(seg + (size_t)strip * seg_stride);
-    const int n_items = (int)hdr[0];
     const int n_fresh = (int)hdr[1];
-    ConstWords fresh_parts = hdr + 4 + 4 * (max_items + kPadItems);
+    ConstWords run_start = hdr + 4;  // ~0 after the last run
+    ConstWords fresh_parts = run_start + list_words;
     const float pm = *p_max;
     const double scale = pm > 0.0f ? 2251799813685248.0 / (double)pm : 1.0;  // 2^51 / p_max
 
@@ -232,7 +245,13 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         acc[r] = 0ull;
         acc[kStripMax + r] = 0ull;
     }
-    // (the first partition switch's barriers also publish yi / acc)
+    if (tid == 0) {
+        staged[0] = 0u;
+        staged[1] = 0u;
+        released[0] = 0u;
+        released[1] = 0u;
+    }
+    __syncthreads();
 
     if (tid >= kStreamThreads) {
         // ---- staging waves ----
@@ -245,10 +264,8 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         const Quad *yxy4 = reinterpret_cast<const Quad *>(yxy);
         Quad *part4 = reinterpret_cast<Quad *>(part);
         const int last_pair_all = (N - 1) / 2;  // yxy is padded, so a pair may run one point past N
-        // Two partitions ahead, in two register sets: a strip that references many partitions opens one every
-        // microsecond or so, which is less than a fetch takes.  The fetches are unconditional (past the last
-        // partition they repeat it) so that the compiler's outstanding-load counts are exact and a write to LDS
-        // waits for its own set only.
+        // The fetches are unconditional (past the last partition they repeat it) so that the compiler's
+        // outstanding-load counts are exact and a write to LDS waits for its own register set only.
         Quad stage_a[kPartLoads], stage_b[kPartLoads];
         auto fetch = [&](Quad (&stage)[kPartLoads], int k) {
             const int p = (int)fresh_parts[min(k, n_fresh - 1)];
@@ -256,91 +273,90 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
             for (int u = 0; u < kPartLoads; ++u)
                 stage[u] = yxy4[min(p * (kPartPoints / 2) + lt + u * kLoadThreads, last_pair_all)];
         };
-        auto publish = [&](const Quad (&stage)[kPartLoads]) {
-            __syncthreads();  // the streaming waves are done with the partition in LDS
+        auto publish = [&](const Quad (&stage)[kPartLoads], int k) {
+            wait_for_count(&released[k & 1], (unsigned int)(kStreamWaves * (k >> 1)));
+            Quad *dst = part4 + (k & 1) * (kPartPoints / 2);
 #pragma unroll
-            for (int u = 0; u < kPartLoads; ++u) part4[lt + u * kLoadThreads] = stage[u];
-            __syncthreads();  // the partition is staged
+            for (int u = 0; u < kPartLoads; ++u) dst[lt + u * kLoadThreads] = stage[u];
+            count_wave(&staged[k & 1], lane);
         };
         if (n_fresh > 0) {
             fetch(stage_a, 0);
             fetch(stage_b, 1);
             int k = 0;
             for (; k + 1 < n_fresh; k += 2) {
-                publish(stage_a);
+                publish(stage_a, k);
                 fetch(stage_a, k + 2);
-                publish(stage_b);
+                publish(stage_b, k + 1);
                 fetch(stage_b, k + 3);
             }
-            if (k < n_fresh) publish(stage_a);
+            if (k < n_fresh) publish(stage_a, k);
         }
     } else {
         // ---- streaming waves ----
         typedef unsigned int Entry __attribute__((ext_vector_type(2)));  // {probability bits, packed row / column}
         const Entry *ent = reinterpret_cast<const Entry *>(ent_p);
+        const unsigned int count = (unsigned int)nrows * (unsigned int)K;
+        const size_t last_entry = (size_t)count - 1;
+        const unsigned int n_items = (count + kItemEntries - 1u) / kItemEntries;
         struct PhaseRegs {
             Entry en[kPrefetch];
-            Record rec;  // {first entry, end entry, first entry of the partition it opens, opens a partition}
         };
-        const size_t last_entry = (size_t)nrows * K - 1;
-        auto issue = [&](PhaseRegs &R) {
+        auto issue = [&](PhaseRegs &R, unsigned int item) {
 #pragma unroll
             for (int k = 0; k < kPrefetch; ++k) {
-                const size_t t = min((size_t)R.rec.x + tid + k * kStreamThreads, last_entry);
+                const size_t t = min((size_t)item * kItemEntries + tid + k * kStreamThreads, last_entry);
                 R.en[k] = ent[base + t];
             }
         };
-        auto entry_force = [&](const Entry &en) {
-            const unsigned int rl = en.y >> kColBits;
-            const float2 yj = part[en.y & ((1u << kColBits) - 1u)];
-            const float2 y0 = yi[rl];
-            const float dx = y0.x - yj.x, dy = y0.y - yj.y;
-            const float w = __uint_as_float(en.x) * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
-            add_force(acc, rl, w * dx, w * dy, scale);
-        };
-        // Entries [rec.x, rec.z) of an item belong to the partition in LDS; when the item opens a partition
-        // (rec.w), the rest, [rec.z, rec.y), belongs to that one (otherwise rec.z == rec.y).
-        auto consume = [&](PhaseRegs &R) {
+        // The run this wave is in (-1: none yet), the buffer that holds its partition, and where the next
+        // two runs start (fetched a run ahead of their use; ~0 when there is none).
+        int run = -1;
+        const float2 *cur = part;
+        unsigned int next_start = run_start[0], after_next_start = run_start[1];
+        // Entries [from, to) of the item, all in the current run.
+        auto span = [&](PhaseRegs &R, unsigned int first, unsigned int from, unsigned int to) {
 #pragma unroll
             for (int k = 0; k < kPrefetch; ++k) {
-                const unsigned int t = R.rec.x + tid + k * kStreamThreads;
-                if (t < R.rec.z) entry_force(R.en[k]);
-            }
-            if (R.rec.w) {
-                __syncthreads();  // everyone is done with the previous partition
-                __syncthreads();  // the staging waves have written the new one
-#pragma unroll
-                for (int k = 0; k < kPrefetch; ++k) {
-                    const unsigned int t = R.rec.x + tid + k * kStreamThreads;
-                    if (t >= R.rec.z && t < R.rec.y) entry_force(R.en[k]);
+                const unsigned int t = first + tid + k * kStreamThreads;
+                if (t >= from && t < to) {
+                    const unsigned int rl = R.en[k].y >> kColBits;
+                    const float2 yj = cur[R.en[k].y & ((1u << kColBits) - 1u)];
+                    const float2 y0 = yi[rl];
+                    const float dx = y0.x - yj.x, dy = y0.y - yj.y;
+                    const float w = __uint_as_float(R.en[k].x) * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
+                    add_force(acc, rl, w * dx, w * dy, scale);
                 }
             }
         };
-        // Prefetch distance two: while item p is consumed, the loads of items p+1 and p+2 are in
-        // flight; the record of item p+3 is fetched (a scalar load) a whole item before it is needed.
-        // The list ends in kPadItems empty records, so nothing here is guarded.
-        typedef const __attribute__((address_space(4))) Record *ConstRecords;
-        ConstRecords records = (ConstRecords)(seg + (size_t)strip * seg_stride + 4);
+        auto consume = [&](PhaseRegs &R, unsigned int item) {
+            const unsigned int first = item * kItemEntries;
+            const unsigned int end = min(first + kItemEntries, count);  // (an item past the last one: end < first)
+            unsigned int from = first;
+            while (next_start < end) {  // a run starts inside this item
+                span(R, first, from, next_start);
+                if (run >= 0) count_wave(&released[run & 1], lane);
+                ++run;
+                wait_for_count(&staged[run & 1], (unsigned int)(kLoadWaves * ((run >> 1) + 1)));
+                cur = part + (run & 1) * kPartPoints;
+                from = next_start;
+                next_start = after_next_start;
+                after_next_start = run_start[run + 2];
+            }
+            span(R, first, from, end);
+        };
+        // Prefetch distance two: while item p is consumed, the loads of items p+1 and p+2 are in flight.
+        // Items past the last one load the last entry again and consume nothing.
         PhaseRegs R0, R1, R2;
-        Record next0, next1, next2;
-        R0.rec = records[0];
-        R1.rec = records[1];
-        R2.rec = records[2];
-        issue(R0);
-        issue(R1);
-        for (int p = 0; p < n_items; p += 3) {
-            next0 = records[p + 3];
-            issue(R2);
-            consume(R0);
-            R0.rec = next0;
-            next1 = records[p + 4];
-            issue(R0);
-            consume(R1);
-            R1.rec = next1;
-            next2 = records[p + 5];
-            issue(R1);
-            consume(R2);
-            R2.rec = next2;
+        issue(R0, 0u);
+        issue(R1, 1u);
+        for (unsigned int p = 0; p < n_items; p += 3) {
+            issue(R2, p + 2);
+            consume(R0, p);
+            issue(R0, p + 3);
+            consume(R1, p + 1);
+            issue(R1, p + 4);
+            consume(R2, p + 2);
         }
     }
     __syncthreads();
@@ -352,7 +368,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
 }
 
 constexpr size_t kBlockedLds =
-    sizeof(float2) * kPartPoints + sizeof(float2) * kStripMax + sizeof(unsigned long long) * 2 * kStripMax;
+    sizeof(float2) * 2 * kPartPoints + sizeof(float2) * kStripMax + sizeof(unsigned long long) * 2 * kStripMax;
 static_assert(kBlockedLds <= 160 * 1024, "one workgroup must fit the 160 KB of LDS");
 
 }  // namespace
@@ -388,9 +404,9 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     p->strip_rows = strip_rows;
     p->n_strips = div_up(N, strip_rows);
     p->n_parts = n_parts;
-    // A strip's work list: one item per kItemEntries entries, plus at most one early end per referenced partition.
-    p->max_items = n_parts + (int)(((int64_t)strip_rows * K) / kItemEntries) + 1;
-    p->seg_stride = 4 + 4 * (p->max_items + kPadItems) + ((n_parts + 3) & ~3);
+    // A strip's list: the run starts (padded: the force kernel reads two past the last run) and the partitions.
+    p->list_words = (n_parts + 4 + 3) & ~3;
+    p->seg_stride = 4 + p->list_words + ((n_parts + 3) & ~3);
     const size_t nnz = (size_t)N * K;
     bool ok = hipMalloc(&p->ent_p, 2 * sizeof(float) * nnz) == hipSuccess &&
               hipMalloc(&p->seg, sizeof(unsigned int) * (size_t)p->n_strips * p->seg_stride) == hipSuccess;
@@ -401,7 +417,7 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     }
     clear_pmax_kernel<<<1, 64, 0, s>>>(&p->scalars->vmax);
     TSNE_LAUNCHED(s);
-    reblock_kernel<<<p->n_strips, kBlock, 0, s>>>(pij, indices, N, K, strip_rows, p->max_items, p->seg_stride, p->ent_p,
+    reblock_kernel<<<p->n_strips, kBlock, 0, s>>>(pij, indices, N, K, strip_rows, p->list_words, p->seg_stride, p->ent_p,
                                                   p->seg,
                                                   &p->scalars->vmax);
     TSNE_LAUNCHED(s);
@@ -420,7 +436,7 @@ int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s) {
     if (profile_mark(p, kKernelAttractive, s)) return 1;
     attractive_blocked_kernel<<<p->n_strips, kBlock, kBlockedLds, s>>>(p->ent_p, p->seg, p->yxy,
                                                                        &p->scalars->vmax, attr, p->num_points,
-                                                                       p->num_neighbors, p->strip_rows, p->max_items,
+                                                                       p->num_neighbors, p->strip_rows, p->list_words,
                                                                        p->seg_stride);
     TSNE_LAUNCHED(s);
     return 0;

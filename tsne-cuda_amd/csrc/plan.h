@@ -73,8 +73,8 @@ struct tsne_hip_plan {
     // Re-blocked copy of the sparse pattern for the LDS-staged attractive kernel.
     float *ent_p = nullptr;         // nnz entries {probability, packed (column in partition | row in strip << 13)},
                                     // 8 bytes each, grouped by (row strip, column partition)
-    unsigned int *seg = nullptr;    // per strip seg_stride words: counts, item records, partitions in opening order
-    int strip_rows = 0, n_strips = 0, n_parts = 0, max_items = 0, seg_stride = 0;
+    unsigned int *seg = nullptr;    // per strip seg_stride words: counts, run starts, partitions in opening order
+    int strip_rows = 0, n_strips = 0, n_parts = 0, list_words = 0, seg_stride = 0;
     bool blocked_ready = false;
 
     // The repulsive chain and the attractive kernel of a step are independent: the fused loop runs
