@@ -87,6 +87,15 @@ __device__ __forceinline__ unsigned int scan_slots(const unsigned int (&value)[k
     return total;
 }
 
+// Where entry `pos` of a strip lives: the strips' items are interleaved (item 0 of every strip, then item 1 of
+// every strip, ...).  The workgroups of the force kernel advance through their strips at about the same pace, so
+// at any moment the chip reads one window of a few items' worth of consecutive addresses, like a plain
+// sequential read, instead of one stream per strip megabytes apart.  Every item starts on a 16-byte boundary.
+__device__ __forceinline__ size_t entry_slot(unsigned int pos, int strip, int n_strips) {
+    const unsigned int item = pos / kItemEntries;
+    return ((size_t)item * n_strips + strip) * kItemEntries + (pos - item * kItemEntries);
+}
+
 __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
                                                          int N, int K, int strip_rows, int list_words,
                                                          int seg_stride, float *__restrict__ ent_p,
@@ -141,7 +150,7 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
         const unsigned int pos = atomicAdd(&cursor[part], 1u);
         const float pv = pij[base + e];
         biggest = fmaxf(biggest, fabsf(pv));
-        reinterpret_cast<uint2 *>(ent_p)[base + pos] =
+        reinterpret_cast<uint2 *>(ent_p)[entry_slot(pos, strip, (int)gridDim.x)] =
             make_uint2(__float_as_uint(pv), (unsigned int)(col - part * kPartPoints) | (row_local << kColBits));
     }
     biggest = group_max<kWave>(biggest);
@@ -228,7 +237,6 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
     const int strip = blockIdx.x;
     const int row0 = strip * strip_rows;
     const int nrows = min(strip_rows, N - row0);
-    const size_t base = (size_t)row0 * K;
     // The list is read through the constant address space: it is never written while this
     // kernel runs, and constant-space loads at uniform addresses are scalar loads, which do not
     // queue behind the vector loads in flight.
@@ -297,16 +305,23 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         typedef unsigned int Entry __attribute__((ext_vector_type(2)));  // {probability bits, packed row / column}
         const Entry *ent = reinterpret_cast<const Entry *>(ent_p);
         const unsigned int count = (unsigned int)nrows * (unsigned int)K;
-        const size_t last_entry = (size_t)count - 1;
         const unsigned int n_items = (count + kItemEntries - 1u) / kItemEntries;
+        // A lane loads two neighbouring entries at a time (16 bytes); the entries are read once per launch and
+        // marked as such, so that they do not push the partitions' positions out of the caches.
+        typedef unsigned int EntryPair __attribute__((ext_vector_type(4)));
+        static_assert(kPrefetch % 2 == 0, "entries are loaded in pairs");
         struct PhaseRegs {
-            Entry en[kPrefetch];
+            Entry en[kPrefetch];  // en[2 j + h]: entry 2 (tid + j kStreamThreads) + h of the item
         };
+        const EntryPair *pairs = reinterpret_cast<const EntryPair *>(ent) + (size_t)strip * (kItemEntries / 2) + tid;
+        const size_t item_pitch = (size_t)gridDim.x * (kItemEntries / 2);  // pairs from one item of a strip to the next
         auto issue = [&](PhaseRegs &R, unsigned int item) {
+            const EntryPair *src = pairs + (size_t)min(item, n_items - 1u) * item_pitch;
 #pragma unroll
-            for (int k = 0; k < kPrefetch; ++k) {
-                const size_t t = min((size_t)item * kItemEntries + tid + k * kStreamThreads, last_entry);
-                R.en[k] = ent[base + t];
+            for (int j = 0; j < kPrefetch / 2; ++j) {
+                const EntryPair v = __builtin_nontemporal_load(src + j * kStreamThreads);
+                R.en[2 * j] = Entry{v.x, v.y};
+                R.en[2 * j + 1] = Entry{v.z, v.w};
             }
         };
         // The run this wave is in (-1: none yet), the buffer that holds its partition, and where the next
@@ -318,7 +333,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         auto span = [&](PhaseRegs &R, unsigned int first, unsigned int from, unsigned int to) {
 #pragma unroll
             for (int k = 0; k < kPrefetch; ++k) {
-                const unsigned int t = first + tid + k * kStreamThreads;
+                const unsigned int t = first + 2 * (tid + (k >> 1) * kStreamThreads) + (k & 1);
                 if (t >= from && t < to) {
                     const unsigned int rl = R.en[k].y >> kColBits;
                     const float2 yj = cur[R.en[k].y & ((1u << kColBits) - 1u)];
@@ -346,7 +361,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
             span(R, first, from, end);
         };
         // Prefetch distance two: while item p is consumed, the loads of items p+1 and p+2 are in flight.
-        // Items past the last one load the last entry again and consume nothing.
+        // Items past the last one load the last item again and consume nothing.
         PhaseRegs R0, R1, R2;
         issue(R0, 0u);
         issue(R1, 1u);
@@ -407,7 +422,9 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     // A strip's list: the run starts (padded: the force kernel reads two past the last run) and the partitions.
     p->list_words = (n_parts + 4 + 3) & ~3;
     p->seg_stride = 4 + p->list_words + ((n_parts + 3) & ~3);
-    const size_t nnz = (size_t)N * K;
+    // Entries: whole items for every strip (the last item of a strip is padded; the padding is never consumed).
+    const size_t items_per_strip = ((size_t)strip_rows * K + kItemEntries - 1) / kItemEntries;
+    const size_t nnz = items_per_strip * p->n_strips * kItemEntries;
     bool ok = hipMalloc(&p->ent_p, 2 * sizeof(float) * nnz) == hipSuccess &&
               hipMalloc(&p->seg, sizeof(unsigned int) * (size_t)p->n_strips * p->seg_stride) == hipSuccess;
     if (!ok) {
