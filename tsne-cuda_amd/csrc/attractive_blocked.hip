@@ -192,14 +192,15 @@ __global__ void clear_pmax_kernel(float *p_max) {
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int rl, float vx, float vy,
                                           double scale) {
+    // magic + v * scale is a double in [2^52, 2^53), where doubles are the integers: its bit pattern is the
+    // magic's plus round(v * scale).  The patterns themselves are summed; every row has exactly K entries, so
+    // its accumulators start at -K times the magic's pattern (mod 2^64) and end at the sum of the integers.
     const double tx = fma((double)vx, scale, kRoundMagic);
     const double ty = fma((double)vy, scale, kRoundMagic);
-    const long long ix = __double_as_longlong(tx) - __double_as_longlong(kRoundMagic);
-    const long long iy = __double_as_longlong(ty) - __double_as_longlong(kRoundMagic);
     // x sums and y sums live in separate arrays: consecutive rows then fall
     // into consecutive 8-byte slots and the atomics of a wave spread over all banks.
-    atomicAdd(&acc[rl], (unsigned long long)ix);
-    atomicAdd(&acc[kStripMax + rl], (unsigned long long)iy);
+    atomicAdd(&acc[rl], (unsigned long long)__double_as_longlong(tx));
+    atomicAdd(&acc[kStripMax + rl], (unsigned long long)__double_as_longlong(ty));
 }
 
 // Polls *counter until it reaches `need` (or kSpinLimit polls have passed).  The compiler barriers keep the
@@ -248,10 +249,12 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
     const float pm = *p_max;
     const double scale = pm > 0.0f ? 2251799813685248.0 / (double)pm : 1.0;  // 2^51 / p_max
 
+    const unsigned long long acc_start =
+        0ull - (unsigned long long)K * (unsigned long long)__double_as_longlong(kRoundMagic);
     for (int r = tid; r < nrows; r += kBlock) {
         yi[r] = yxy[row0 + r];
-        acc[r] = 0ull;
-        acc[kStripMax + r] = 0ull;
+        acc[r] = acc_start;
+        acc[kStripMax + r] = acc_start;
     }
     if (tid == 0) {
         staged[0] = 0u;
