@@ -91,10 +91,16 @@ __device__ __forceinline__ unsigned int scan_slots(const unsigned int (&value)[k
 // every strip, ...).  The workgroups of the force kernel advance through their strips at about the same pace, so
 // at any moment the chip reads one window of a few items' worth of consecutive addresses, like a plain
 // sequential read, instead of one stream per strip megabytes apart.  Every item starts on a 16-byte boundary.
+// Inside an item, every 128 entries are stored as 64 pairs (j, j + 64): a lane of the force kernel loads a pair
+// at a time, and the 64 lanes of a wave then hold 64 consecutive entries in each half of their registers
+// (consecutive entries belong to consecutive rows, whose accumulators lie in different LDS banks).
 __device__ __forceinline__ size_t entry_slot(unsigned int pos, int strip, int n_strips) {
     const unsigned int item = pos / kItemEntries;
-    return ((size_t)item * n_strips + strip) * kItemEntries + (pos - item * kItemEntries);
+    const unsigned int in_item = pos - item * kItemEntries;
+    const unsigned int j = in_item & 127u;
+    return ((size_t)item * n_strips + strip) * kItemEntries + (in_item - j) + 2u * (j & 63u) + (j >> 6);
 }
+static_assert(kItemEntries % 128 == 0, "items hold whole groups of 64 entry pairs");
 
 __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
                                                          int N, int K, int strip_rows, int list_words,
@@ -314,7 +320,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         typedef unsigned int EntryPair __attribute__((ext_vector_type(4)));
         static_assert(kPrefetch % 2 == 0, "entries are loaded in pairs");
         struct PhaseRegs {
-            Entry en[kPrefetch];  // en[2 j + h]: entry 2 (tid + j kStreamThreads) + h of the item
+            Entry en[kPrefetch];  // en[2 j + h]: entry 128 ((tid + j kStreamThreads) / 64) + 64 h + lane of the item
         };
         const EntryPair *pairs = reinterpret_cast<const EntryPair *>(ent) + (size_t)strip * (kItemEntries / 2) + tid;
         const size_t item_pitch = (size_t)gridDim.x * (kItemEntries / 2);  // pairs from one item of a strip to the next
@@ -336,7 +342,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         auto span = [&](PhaseRegs &R, unsigned int first, unsigned int from, unsigned int to) {
 #pragma unroll
             for (int k = 0; k < kPrefetch; ++k) {
-                const unsigned int t = first + 2 * (tid + (k >> 1) * kStreamThreads) + (k & 1);
+                const unsigned int t = first + 128 * ((tid + (k >> 1) * kStreamThreads) >> 6) + 64 * (k & 1) + lane;
                 if (t >= from && t < to) {
                     const unsigned int rl = R.en[k].y >> kColBits;
                     const float2 yj = cur[R.en[k].y & ((1u << kColBits) - 1u)];
