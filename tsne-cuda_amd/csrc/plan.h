@@ -71,8 +71,9 @@ struct tsne_hip_plan {
     float *rep = nullptr;   // 2N
 
     // Re-blocked copy of the sparse pattern for the LDS-staged attractive kernel.
-    float *ent_p = nullptr;         // nnz entries {probability, packed (column in partition | row in strip << 13)},
-                                    // 8 bytes each, grouped by (row strip, column partition)
+    float *ent_p = nullptr;         // entries {probability, packed (column in partition | row in strip << 11)},
+                                    // 8 bytes each, grouped by (row strip, column partition), in items of
+                                    // consecutive entries that are interleaved over the strips
     unsigned int *seg = nullptr;    // per strip seg_stride words: counts, run starts, partitions in opening order
     int strip_rows = 0, n_strips = 0, n_parts = 0, list_words = 0, seg_stride = 0;
     bool blocked_ready = false;
