@@ -286,13 +286,18 @@ def test_errors_are_reported(stages):
         stages.Plan(100, 5, n_boxes_per_dim=1000)
 
 
-@pytest.mark.parametrize("n,k", [(5000, 90), (20000, 30), (9000, 7), (300, 300)])
+@pytest.mark.parametrize("n,k", [(5000, 90), (20000, 30), (9000, 7), (300, 300), (150000, 12)])
 def test_attractive_blocked_pattern(stages, n, k):
     """The re-blocked (row strip x column partition) copy of the pattern gives
     the same forces as the oracle; 20000 and 9000 points span several column
-    partitions, 300 x 300 is a dense pattern in a single bucket."""
+    partitions, 300 x 300 is a dense pattern in a single bucket, 150000 x 12
+    gives every strip several work items with dozens of partition runs in
+    each (74 partitions, ~95 entries per run)."""
     rng = np.random.default_rng(n + k)
-    idx = np.stack([rng.permutation(n)[:k] for _ in range(n)]).astype(np.int32)
+    if n <= 20000:
+        idx = np.stack([rng.permutation(n)[:k] for _ in range(n)]).astype(np.int32)
+    else:  # (a row may name a column twice: the forces just add)
+        idx = rng.integers(0, n, (n, k)).astype(np.int32)
     idx[:, 0] = np.arange(n)
     P = (rng.random((n, k)) * 1e-5).astype(np.float32)
     P[:, 0] = 0.0
