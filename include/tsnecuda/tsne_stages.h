@@ -150,6 +150,15 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
                      float pre_exaggeration_momentum, float post_exaggeration_momentum,
                      float early_exaggeration, float *normalization, void *stream);
 
+/* Whether a kernel of this plan has reported trouble since the last call (no
+ * counterpart in the reference).  Call it after synchronising the streams the
+ * plan was used on.  The one condition reported today: waves of the re-blocked
+ * attractive kernel coordinate through bounded waits, and a workgroup whose
+ * wait ran out writes NaN forces and counts itself here.  Returns 0 when
+ * nothing was reported, 1 (with tsne_hip_last_error) otherwise; clears the
+ * report. */
+int tsne_hip_plan_check(tsne_hip_plan *plan);
+
 /* Squared L2 norm of n device floats into the device scalar *out
  * (tsnecuda::util::L2NormDeviceVector without the root, src/util/math_utils.cu:51-57). */
 int tsne_hip_sum_squares(tsne_hip_plan *plan, const float *values, int64_t n, float *out, void *stream);

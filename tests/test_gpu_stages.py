@@ -313,6 +313,34 @@ def test_attractive_blocked_pattern(stages, n, k):
     plan.close()
 
 
+def test_attractive_wait_that_runs_out_is_reported(stages, monkeypatch):
+    """The two roles of the re-blocked attractive kernel wait for each other with
+    bounded polls.  With the limit forced to zero from the host every wait runs
+    out at once: the kernel still ends normally, the forces are NaN and the plan
+    reports it once; a plan prepared without the override is unaffected."""
+    n, k = 20000, 30
+    rng = np.random.default_rng(77)
+    idx = rng.integers(0, n, (n, k)).astype(np.int32)
+    P = (rng.random((n, k)) * 1e-5).astype(np.float32)
+    y = (rng.standard_normal(2 * n) * 8.0).astype(np.float32)
+    monkeypatch.setenv("TSNE_ATTRACTIVE_SPIN_LIMIT", "0")
+    plan = stages.Plan(n, k)
+    plan.prepare_attractive(dev(P), dev(idx))
+    got = plan.attractive(None, None, dev(y)).cpu().numpy()
+    assert np.isnan(got).all()
+    with pytest.raises(RuntimeError, match="timed out"):
+        plan.check()
+    plan.check()  # the report was cleared
+    plan.close()
+    monkeypatch.delenv("TSNE_ATTRACTIVE_SPIN_LIMIT")
+    plan = stages.Plan(n, k)
+    plan.prepare_attractive(dev(P), dev(idx))
+    got = plan.attractive(None, None, dev(y)).cpu().numpy()
+    assert rel_l2(got, oracle.attractive(P, idx, y)) <= 1e-4
+    plan.check()
+    plan.close()
+
+
 def test_attractive_blocked_clustered_pattern(stages):
     """A pattern whose rows reference only a few column partitions (what the
     locality ordering produces): runs longer than one work item share a staged

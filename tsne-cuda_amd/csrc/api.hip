@@ -501,6 +501,12 @@ int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches) {
     return 0;
 }
 
+int tsne_hip_plan_check(tsne_hip_plan *plan) {
+    if (check_plan(plan, "plan_check")) return 1;
+    TSNE_TRY(hipSetDevice(plan->device));
+    return check_attractive_waits(plan);
+}
+
 int tsne_hip_sum_squares(tsne_hip_plan *plan, const float *values, int64_t n, float *out, void *stream) {
     if (check_plan(plan, "sum_squares")) return 1;
     TSNE_REQUIRE(values && out && n > 0, "sum_squares: need a non-empty array and an output");

@@ -28,6 +28,9 @@
 //
 // Semantics are those of src/kernels/attr_forces.cu:129-184 of the reference;
 // only the order of the additions inside a row differs.
+#include <algorithm>
+#include <cstdlib>
+
 #include "plan.h"
 
 namespace tsnehip {
@@ -49,7 +52,9 @@ constexpr int kLoadThreads = kBlock - kStreamThreads;  // ... waves 12-15 stage 
 constexpr int kLoadWaves = kLoadThreads / kWave;
 constexpr unsigned int kItemEntries = kPrefetch * kStreamThreads;
 constexpr int kSpinLimit = 1 << 18; // polls of an LDS counter before a wave gives up waiting (about ten milliseconds;
-                                    // a wait normally ends within a microsecond): every wave reaches the kernel's end
+                                    // a wait normally ends within a microsecond): every wave reaches the kernel's end.
+                                    // TSNE_ATTRACTIVE_SPIN_LIMIT (read when the pattern is prepared) overrides it, so
+                                    // that a test can make the waits fail (0: every wait) without any kernel hanging.
 
 // ---------------------------------------------------------------------------
 // Re-blocking: one workgroup per strip.  Histogram of the strip's entries over
@@ -209,11 +214,17 @@ __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int 
     atomicAdd(&acc[kStripMax + rl], (unsigned long long)__double_as_longlong(ty));
 }
 
-// Polls *counter until it reaches `need` (or kSpinLimit polls have passed).  The compiler barriers keep the
-// buffer accesses of the caller on their side of the wait.
-__device__ __forceinline__ void wait_for_count(const unsigned int *counter, unsigned int need) {
+// Polls *counter until it reaches `need`; after kSpinLimit polls the wave sets *gave_up and goes on (the
+// workgroup then reports it and writes NaN forces).  The compiler barriers keep the buffer accesses of the
+// caller on their side of the wait.
+__device__ __forceinline__ void wait_for_count(const unsigned int *counter, unsigned int need, int spin_limit,
+                                               unsigned int *gave_up) {
     asm volatile("" ::: "memory");
-    for (int spin = 0; spin < kSpinLimit; ++spin) {
+    for (int spin = 0;; ++spin) {
+        if (spin >= spin_limit) {  // (a limit of 0 gives up without looking)
+            *gave_up = 1u;
+            break;
+        }
         if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= need) break;
         __builtin_amdgcn_s_sleep(1);
     }
@@ -227,17 +238,22 @@ __device__ __forceinline__ void count_wave(unsigned int *counter, int lane) {
     asm volatile("" ::: "memory");
 }
 
+// RUNTIME_LIMIT: the poll limit is the argument (the override for tests); otherwise it is the constant, with
+// which the compiler lays the wait loops out better (197 against 203 us per launch at a million points).
+template <bool RUNTIME_LIMIT>
 __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float *__restrict__ ent_p,
                                                                     const unsigned int *__restrict__ seg,
                                                                     const float2 *__restrict__ yxy,
-                                                                    const float *__restrict__ p_max,
+                                                                    LoopScalars *__restrict__ scalars,
                                                                     float *__restrict__ attr, int N, int K,
-                                                                    int strip_rows, int list_words, int seg_stride) {
+                                                                    int strip_rows, int list_words, int seg_stride,
+                                                                    int spin_limit_arg) {
+    const int spin_limit = RUNTIME_LIMIT ? spin_limit_arg : kSpinLimit;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     float2 *part = reinterpret_cast<float2 *>(lds_raw);  // two buffers of kPartPoints
     float2 *yi = part + 2 * kPartPoints;
     unsigned long long *acc = reinterpret_cast<unsigned long long *>(yi + kStripMax);
-    __shared__ unsigned int staged[2], released[2];
+    __shared__ unsigned int staged[2], released[2], gave_up;
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -252,7 +268,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
     const int n_fresh = (int)hdr[1];
     ConstWords run_start = hdr + 4;  // ~0 after the last run
     ConstWords fresh_parts = run_start + list_words;
-    const float pm = *p_max;
+    const float pm = scalars->vmax;
     const double scale = pm > 0.0f ? 2251799813685248.0 / (double)pm : 1.0;  // 2^51 / p_max
 
     const unsigned long long acc_start =
@@ -267,6 +283,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         staged[1] = 0u;
         released[0] = 0u;
         released[1] = 0u;
+        gave_up = 0u;
     }
     __syncthreads();
 
@@ -291,7 +308,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
                 stage[u] = yxy4[min(p * (kPartPoints / 2) + lt + u * kLoadThreads, last_pair_all)];
         };
         auto publish = [&](const Quad (&stage)[kPartLoads], int k) {
-            wait_for_count(&released[k & 1], (unsigned int)(kStreamWaves * (k >> 1)));
+            wait_for_count(&released[k & 1], (unsigned int)(kStreamWaves * (k >> 1)), spin_limit, &gave_up);
             Quad *dst = part4 + (k & 1) * (kPartPoints / 2);
 #pragma unroll
             for (int u = 0; u < kPartLoads; ++u) dst[lt + u * kLoadThreads] = stage[u];
@@ -361,7 +378,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
                 span(R, first, from, next_start);
                 if (run >= 0) count_wave(&released[run & 1], lane);
                 ++run;
-                wait_for_count(&staged[run & 1], (unsigned int)(kLoadWaves * ((run >> 1) + 1)));
+                wait_for_count(&staged[run & 1], (unsigned int)(kLoadWaves * ((run >> 1) + 1)), spin_limit, &gave_up);
                 cur = part + (run & 1) * kPartPoints;
                 from = next_start;
                 next_start = after_next_start;
@@ -384,11 +401,12 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
         }
     }
     __syncthreads();
-    const double inv_scale = 1.0 / scale;
+    const double inv_scale = gave_up ? (double)NAN : 1.0 / scale;
     for (int r = tid; r < nrows; r += kBlock) {
         attr[row0 + r] = (float)((double)(long long)acc[r] * inv_scale);
         attr[N + row0 + r] = (float)((double)(long long)acc[kStripMax + r] * inv_scale);
     }
+    if (gave_up && tid == 0) atomicAdd(&scalars->wait_timeouts, 1u);
 }
 
 constexpr size_t kBlockedLds =
@@ -447,8 +465,12 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
                                                   p->seg,
                                                   &p->scalars->vmax);
     TSNE_LAUNCHED(s);
-    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attractive_blocked_kernel),
+    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attractive_blocked_kernel<false>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBlockedLds));
+    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attractive_blocked_kernel<true>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBlockedLds));
+    p->spin_limit = kSpinLimit;
+    if (const char *v = std::getenv("TSNE_ATTRACTIVE_SPIN_LIMIT")) p->spin_limit = std::max(0, std::atoi(v));
     p->blocked_ready = true;
     return 0;
 }
@@ -460,12 +482,23 @@ int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s) {
         return 1;
     }
     if (profile_mark(p, kKernelAttractive, s)) return 1;
-    attractive_blocked_kernel<<<p->n_strips, kBlock, kBlockedLds, s>>>(p->ent_p, p->seg, p->yxy,
-                                                                       &p->scalars->vmax, attr, p->num_points,
-                                                                       p->num_neighbors, p->strip_rows, p->list_words,
-                                                                       p->seg_stride);
+    const auto kernel = p->spin_limit == kSpinLimit ? attractive_blocked_kernel<false> : attractive_blocked_kernel<true>;
+    kernel<<<p->n_strips, kBlock, kBlockedLds, s>>>(p->ent_p, p->seg, p->yxy, p->scalars, attr, p->num_points,
+                                                    p->num_neighbors, p->strip_rows, p->list_words, p->seg_stride,
+                                                    p->spin_limit);
     TSNE_LAUNCHED(s);
     return 0;
+}
+
+// After the stream has been synchronised: whether any attractive launch since the last check lost step
+// between its waves (see LoopScalars::wait_timeouts).  Clears the count.
+int check_attractive_waits(tsne_hip_plan *p) {
+    unsigned int n = 0;
+    TSNE_TRY(hipMemcpy(&n, &p->scalars->wait_timeouts, sizeof(n), hipMemcpyDeviceToHost));
+    if (n == 0) return 0;
+    TSNE_TRY(hipMemset(&p->scalars->wait_timeouts, 0, sizeof(n)));
+    set_error("attractive: %u workgroup(s) timed out waiting for a staged partition; their forces are NaN", n);
+    return 1;
 }
 
 }  // namespace tsnehip

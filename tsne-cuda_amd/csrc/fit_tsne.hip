@@ -365,6 +365,7 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         }
     }
     hip_or_die(hipStreamSynchronize(stream), "gradient loop");
+    if (blocked) TSNE_OR_DIE(tsnehip::check_attractive_waits(plan), "gradient loop");
     if (opt.iterations > 0)
         hip_or_die(hipMemcpy(&normalization, d_norm.ptr, sizeof(float), hipMemcpyDeviceToHost), "normalisation");
 

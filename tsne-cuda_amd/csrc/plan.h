@@ -76,6 +76,7 @@ struct tsne_hip_plan {
                                     // consecutive entries that are interleaved over the strips
     unsigned int *seg = nullptr;    // per strip seg_stride words: counts, run starts, partitions in opening order
     int strip_rows = 0, n_strips = 0, n_parts = 0, list_words = 0, seg_stride = 0;
+    int spin_limit = 0;             // polls before a wave of the attractive kernel gives up a wait
     bool blocked_ready = false;
 
     // The repulsive chain and the attractive kernel of a step are independent: the fused loop runs
@@ -144,6 +145,7 @@ int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, fl
 int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s);
 void release_blocked(tsne_hip_plan *p);
 int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s);
+int check_attractive_waits(tsne_hip_plan *p);
 int launch_sum_squares(const float *values, int64_t n, float *out, hipStream_t s);
 int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, float *gains, float *old_forces,
                   float eta, const float *normalization, float momentum, float exaggeration, int next_slot,

@@ -32,6 +32,7 @@ def lib():
         L.tsne_hip_perplexity.argtypes = [_vp, c_int, c_int, c_float, c_float, _vp, _vp, _vp]
         L.tsne_hip_symmetrize.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
         L.tsne_hip_plan_create.argtypes = [ctypes.POINTER(_vp), c_int, c_int, c_int, c_int]
+        L.tsne_hip_plan_check.argtypes = [_vp]
         L.tsne_hip_plan_destroy.argtypes = [_vp]
         L.tsne_hip_plan_destroy.restype = None
         L.tsne_hip_attractive.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp]
@@ -157,6 +158,12 @@ class Plan(object):
             self.close()
         except Exception:
             pass
+
+    def check(self):
+        """Raises if a kernel of this plan reported trouble since the last call
+        (synchronises the device first)."""
+        torch.cuda.synchronize(self.device)
+        _check(lib().tsne_hip_plan_check(self._h))
 
     def prepare_attractive(self, pij, idx):
         """Re-blocks (pij, idx) into the plan; afterwards attractive() and
