@@ -505,6 +505,26 @@ def test_knn_matrix_sweep_verification_falls_back(stages):
     assert np.array_equal(d2.cpu().numpy(), d2_o)
 
 
+def test_knn_few_failed_queries_are_redone_by_candidate_range(stages):
+    """A clump of 400 nearly identical points: for some of its members the 300th
+    neighbour and the sweep's threshold lie closer together than the matrix sweep
+    can tell apart, so they fail its verification (95 of them on this seed) while
+    the other points pass.  The vector sweep takes just those queries, cut over the chip by candidate range and merged
+    (K - 1 = 299 keys per range)."""
+    rng = np.random.default_rng(11)
+    n, d, k = 20000, 16, 300
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    clump = rng.choice(n, 400, replace=False)
+    X[clump] = (rng.standard_normal((1, d)) + rng.standard_normal((400, d)) * 1e-5).astype(np.float32)
+    idx, d2, stats = stages.knn_select(dev(X), k, 2)
+    assert stats[0] == 1 and 0 < stats[1] <= 400
+    rows = np.concatenate([clump[:80], rng.choice(n, 24, replace=False)])
+    for q in rows:
+        idx_o, d2_o = oracle.knn(X, k, rows=(int(q), int(q) + 1))
+        assert np.array_equal(idx[q].cpu().numpy(), idx_o[0])
+        assert np.array_equal(d2[q].cpu().numpy(), d2_o[0])
+
+
 def test_iterate_graph_replay_matches_eager(stages, c0_problem, monkeypatch):
     """Small problems replay a captured graph of two steps.  Replays, with eager
     work and synchronisations between them, give what the eager loop gives (to

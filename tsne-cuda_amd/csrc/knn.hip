@@ -398,13 +398,19 @@ __device__ __forceinline__ bool tile_may_matter_wide(const float *qcenter, float
 // only the tiles whose ball may hold a point below the largest k-th distance found so far.  The
 // distances here are the canonical ones, so a skipped tile is strictly farther than every threshold.
 // Dynamic LDS: cap keys, then D floats (the query tile's ball centre), then the visit bitmap.
+//
+// slices > 1 (listed queries only): a handful of queries would occupy a handful of workgroups for a sweep over
+// all points, so the candidate tiles are cut into `slices` ranges and a (query tile, range) pair is one unit of
+// work; each unit leaves its K-1 best keys in slice_keys[(slot * slices + range) * (K-1) ...] (padded with ~0)
+// and knn_merge_slices_kernel forms the rows.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict__ Xt, int N, int Npad, int D, int K,
                                                         int cap, u64 *__restrict__ lists, int num_qtiles,
                                                         const int *__restrict__ qlist, int nq,
                                                         int *__restrict__ out_idx, float *__restrict__ out_d,
                                                         const float *__restrict__ centers_t,
-                                                        const float *__restrict__ radius, int bitmap_words) {
+                                                        const float *__restrict__ radius, int bitmap_words,
+                                                        int slices, u64 *__restrict__ slice_keys) {
     __shared__ __attribute__((aligned(16))) float xq[kDC][kQT];
     __shared__ __attribute__((aligned(16))) float xc[kDC][kCT];
     __shared__ u64 thr[kQT];
@@ -421,7 +427,8 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
     const int T = (N + kCT - 1) / kCT;
     u64 *list = lists + (size_t)blockIdx.x * kQT * cap;
 
-    for (int qt = blockIdx.x; qt < num_qtiles; qt += gridDim.x) {
+    for (int unit = blockIdx.x; unit < num_qtiles * slices; unit += gridDim.x) {
+        const int qt = unit / slices, slice = unit - qt * slices;
         if (tid < kQT) {
             const int slot = qt * kQT + tid;
             thr[tid] = ~0ull;
@@ -489,7 +496,11 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
         };
         const bool prune = bitmap_words > 0 && qlist == nullptr;
         const int bt = (qt * kQT) / kCT;  // the ball tile this query tile lies in
-        const int h0 = prune ? max(bt - kHomeTiles, 0) : 0, h1 = prune ? min(bt + kHomeTiles, T - 1) : T - 1;
+        int h0 = prune ? max(bt - kHomeTiles, 0) : 0, h1 = prune ? min(bt + kHomeTiles, T - 1) : T - 1;
+        if (slices > 1) {  // this unit's range of the candidate tiles
+            h0 = (int)(((long long)T * slice) / slices);
+            h1 = (int)(((long long)T * (slice + 1)) / slices) - 1;
+        }
         for (int ct = h0; ct <= h1; ++ct) process(ct * kCT);
         if (prune && (h0 > 0 || h1 < T - 1)) {
             // Thresholds from what the neighbourhood held, then the tiles that may still matter.
@@ -530,6 +541,13 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
             const int q = qid[ql];
             if (q < 0) break;
             compact_query(list, cap, want, cnt, thr, ql, sortbuf, tid);
+            if (slices > 1) {
+                // (compact_query leaves the sorted keys in sortbuf, ~0 beyond the entries there were)
+                u64 *dst = slice_keys + ((size_t)(qt * kQT + ql) * slices + slice) * want;
+                for (int e = tid; e < want; e += 256) dst[e] = sortbuf[e];
+                __syncthreads();
+                continue;
+            }
             for (int e = tid; e < K; e += 256) {
                 int j = q;
                 float d = 0.0f;
@@ -543,6 +561,31 @@ __global__ __launch_bounds__(256) void knn_sweep_kernel(const float *__restrict_
             }
             __syncthreads();
         }
+    }
+}
+
+// Rows of the listed queries from the keys their `slices` units left: one workgroup per query sorts the
+// slices * (K-1) keys (sort_n: that count rounded up to a power of two; dynamic LDS: sort_n keys).
+__global__ __launch_bounds__(256) void knn_merge_slices_kernel(const u64 *__restrict__ slice_keys, int slices, int K,
+                                                               int sort_n, const int *__restrict__ qlist,
+                                                               int *__restrict__ out_idx, float *__restrict__ out_d) {
+    extern __shared__ u64 merge_sortbuf[];
+    const int tid = threadIdx.x, slot = blockIdx.x, want = K - 1;
+    const int q = qlist[slot];
+    const int total = slices * want;
+    for (int e = tid; e < sort_n; e += 256) merge_sortbuf[e] = e < total ? slice_keys[(size_t)slot * total + e] : ~0ull;
+    __syncthreads();
+    bitonic_sort(merge_sortbuf, sort_n, tid);
+    for (int e = tid; e < K; e += 256) {
+        int j = q;
+        float d = 0.0f;
+        if (e > 0) {
+            const u64 key = merge_sortbuf[e - 1];
+            j = key_index(key);
+            d = key_distance(key);
+        }
+        out_idx[(size_t)q * K + e] = j;
+        out_d[(size_t)q * K + e] = d;
     }
 }
 
@@ -1389,14 +1432,23 @@ int run_valu_sweep(const float *points, const float *Xt, int N, int Npad, int D,
                    int cus, int *indices, float *sq_dist, hipStream_t s) {
     const int cap = valu_cap(K);
     const int num_qtiles = div_up(nq, kQT);
-    const int grid = std::min(num_qtiles, cus * 3);
+    // A few listed queries: cut the candidates into ranges so that the whole chip works on them (as many
+    // ranges as keep about four workgroups per CU busy, the merge's sort within 8192 keys, and at least one
+    // candidate tile per range).
+    int slices = 1;
+    if (qlist != nullptr && K > 1)
+        while (slices < 64 && num_qtiles * slices * 2 <= 4 * cus && slices * 2 * (K - 1) <= 8192 &&
+               slices * 2 <= div_up(N, kCT))
+            slices *= 2;
+    const int grid = std::min(num_qtiles * slices, cus * 3);
     // Tile balls for skipping far-away candidate tiles: only when all queries are swept and the
     // neighbourhood that is always swept does not cover everything anyway.
     const int T = div_up(N, kCT);
     const bool prune = qlist == nullptr && T > 2 * kHomeTiles + 1;
     const int bitmap_words = prune ? div_up(T, 32) : 0;
-    DeviceMem lists, centers, radius;
+    DeviceMem lists, centers, radius, slice_keys;
     if (!lists.alloc(sizeof(u64) * (size_t)grid * kQT * cap) ||
+        (slices > 1 && !slice_keys.alloc(sizeof(u64) * (size_t)num_qtiles * kQT * slices * (K - 1))) ||
         (prune && (!centers.alloc(sizeof(float) * (size_t)D * T) || !radius.alloc(sizeof(float) * T)))) {
         set_error("knn: out of device memory for the candidate lists");
         return 1;
@@ -1407,8 +1459,16 @@ int run_valu_sweep(const float *points, const float *Xt, int N, int Npad, int D,
     }
     const size_t lds = sizeof(u64) * cap + (prune ? sizeof(float) * D + sizeof(unsigned int) * bitmap_words : 0);
     knn_sweep_kernel<<<grid, 256, lds, s>>>(Xt, N, Npad, D, K, cap, lists.as<u64>(), num_qtiles, qlist, nq, indices,
-                                            sq_dist, centers.as<float>(), radius.as<float>(), bitmap_words);
+                                            sq_dist, centers.as<float>(), radius.as<float>(), bitmap_words, slices,
+                                            slice_keys.as<u64>());
     TSNE_TRY(hipGetLastError());
+    if (slices > 1) {
+        int sort_n = 256;
+        while (sort_n < slices * (K - 1)) sort_n <<= 1;
+        knn_merge_slices_kernel<<<nq, 256, sizeof(u64) * sort_n, s>>>(slice_keys.as<u64>(), slices, K, sort_n, qlist,
+                                                                     indices, sq_dist);
+        TSNE_TRY(hipGetLastError());
+    }
     TSNE_TRY(hipStreamSynchronize(s));
     return 0;
 }
@@ -1632,11 +1692,12 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         stats[1] = failed;
         stats[2] = (int)((1000.0 * (double)swept) / ((double)num_tiles * (double)num_tiles) + 0.5);
     }
-    // The chunked sweep takes the tiles of the few queries that failed once more with twice the margin
-    // (a vector sweep of one query tile over all points in hundreds of dimensions takes as long as the
-    // whole matrix sweep); what fails again, and every failure of the register-resident sweep, goes to
-    // the vector sweep.
-    if (failed > 0 && chunked && failed * 10 <= N) {
+    // Up to a few query tiles' worth of failures go straight to the vector sweep, which spreads a short list of
+    // queries over the chip by candidate range.  Beyond that the chunked sweep takes the tiles of the queries
+    // that failed once more with twice the margin (a vector sweep of many query tiles over all points in hundreds
+    // of dimensions takes as long as the whole matrix sweep); what fails again, and every failure of the
+    // register-resident sweep, goes to the vector sweep.
+    if (failed > 4 * kQT && chunked && failed * 10 <= N) {
         const int wider = std::min(N - 1, 2 * want);
         if (wider != want && sweep_fits(wider)) {
             std::vector<int> queries(failed), tiles;
