@@ -107,12 +107,27 @@ __device__ __forceinline__ size_t entry_slot(unsigned int pos, int strip, int n_
 }
 static_assert(kItemEntries % 128 == 0, "items hold whole groups of 64 entry pairs");
 
+// Order of the entries inside a partition's run.  The force kernel's wave handles 64 consecutive entries at a
+// time and touches, per entry, the position and the two accumulators of the entry's row: 8-byte slots, 32 of
+// which span the LDS banks.  A run is therefore dealt out by row residue: its entries are bucketed by
+// (row mod 32) and emitted round robin, one from every bucket that still has one, so that any 64 consecutive
+// entries hit every bank pair twice (until the fuller buckets are all that is left, at the end of the run).
+// That needs two counters per (referenced partition, residue) in LDS; a strip that references more than
+// kBalancedParts partitions keeps the order of arrival instead (neighbour slot by neighbour slot).
+constexpr int kBalancedParts = 320;
+constexpr int kResidues = 32;
+constexpr int kResidueStride = kResidues + 1;  // odd: the 32 counters of different partitions spread over the banks
+constexpr size_t kReblockLds = sizeof(unsigned int) * 2 * kBalancedParts * kResidueStride;
+
 __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
                                                          int N, int K, int strip_rows, int list_words,
                                                          int seg_stride, float *__restrict__ ent_p,
                                                          unsigned int *__restrict__ seg, float *__restrict__ p_max) {
     __shared__ unsigned int cursor[kMaxParts];
+    __shared__ unsigned short fresh_of[kMaxParts];  // partition -> its place among the partitions the strip references
     __shared__ unsigned int scan[kBlock];
+    extern __shared__ unsigned int residue_count[];                             // [place][kResidueStride]
+    unsigned int *residue_cursor = residue_count + kBalancedParts * kResidueStride;  // same shape
     const int tid = threadIdx.x;
     const int strip = blockIdx.x;
     const int row0 = strip * strip_rows;
@@ -145,12 +160,23 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
         if (flag[i]) {
             fresh_parts[order[i]] = (unsigned int)(tid * kSlotsPerThread + i);
             run_start[order[i]] = first[i];
+            fresh_of[tid * kSlotsPerThread + i] = (unsigned short)order[i];
         }
     for (unsigned int b = n_fresh + tid; b < (unsigned int)list_words; b += kBlock) run_start[b] = ~0u;
     if (tid == 0) hdr[1] = n_fresh;
-    // Entries are visited neighbour slot by neighbour slot, so that neighbouring positions of a
-    // partition's run belong to different rows: a wave of the force kernel then spreads its LDS
-    // atomics over many accumulators even when most neighbours of a row share one partition.
+    const bool balanced = n_fresh <= (unsigned int)kBalancedParts;
+    if (balanced) {
+        for (unsigned int b = tid; b < 2u * kBalancedParts * kResidueStride; b += kBlock) residue_count[b] = 0u;
+        __syncthreads();
+        for (unsigned int e = tid; e < count; e += kBlock) {
+            const unsigned int row_local = e / (unsigned int)K;
+            const unsigned int place = fresh_of[idx[base + e] / kPartPoints];
+            atomicAdd(&residue_count[place * kResidueStride + (row_local & (kResidues - 1))], 1u);
+        }
+    }
+    __syncthreads();
+    // Entries are visited neighbour slot by neighbour slot, so that the entries of one row lie far apart
+    // in a partition's run (also within a residue's bucket): a wave of the force kernel never meets a row twice.
     float biggest = 0.0f;
     for (unsigned int v = tid; v < count; v += kBlock) {
         const unsigned int slot = v / (unsigned int)nrows;
@@ -158,7 +184,21 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
         const unsigned int e = row_local * (unsigned int)K + slot;
         const int col = idx[base + e];
         const int part = col / kPartPoints;
-        const unsigned int pos = atomicAdd(&cursor[part], 1u);
+        unsigned int pos;
+        if (balanced) {
+            const unsigned int q = row_local & (kResidues - 1);
+            const unsigned int *counts = residue_count + fresh_of[part] * kResidueStride;
+            const unsigned int j = atomicAdd(&residue_cursor[fresh_of[part] * kResidueStride + q], 1u);
+            // Round j of the dealing: everything of the rounds before it, then the buckets before q that reach round j.
+            pos = cursor[part];
+#pragma unroll 8
+            for (unsigned int other = 0; other < (unsigned int)kResidues; ++other) {
+                const unsigned int c = counts[other];
+                pos += min(c, j) + ((other < q && c > j) ? 1u : 0u);
+            }
+        } else {
+            pos = atomicAdd(&cursor[part], 1u);
+        }
         const float pv = pij[base + e];
         biggest = fmaxf(biggest, fabsf(pv));
         reinterpret_cast<uint2 *>(ent_p)[entry_slot(pos, strip, (int)gridDim.x)] =
@@ -461,7 +501,9 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     }
     clear_pmax_kernel<<<1, 64, 0, s>>>(&p->scalars->vmax);
     TSNE_LAUNCHED(s);
-    reblock_kernel<<<p->n_strips, kBlock, 0, s>>>(pij, indices, N, K, strip_rows, p->list_words, p->seg_stride, p->ent_p,
+    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(reblock_kernel),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kReblockLds));
+    reblock_kernel<<<p->n_strips, kBlock, kReblockLds, s>>>(pij, indices, N, K, strip_rows, p->list_words, p->seg_stride, p->ent_p,
                                                   p->seg,
                                                   &p->scalars->vmax);
     TSNE_LAUNCHED(s);
