@@ -191,9 +191,9 @@ def main():
             oracle_kl = json.load(f).get("kl_exact_z")
 
     # HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes whose
-    # summary sits in profiles/bench_c3_1M_hbm_counters.txt (396057 x 2 KiB fetched + 7826 x 1 KiB written);
+    # summary sits in profiles/bench_c3_1M_hbm_counters.txt (395672 x 2 KiB fetched + 7826 x 1 KiB written);
     # the counters belong to that exact workload, so other sizes report null.
-    traffic = 819.1e6 if (args.workload == "c3" and n == 1000000 and k == 90) else None
+    traffic = 818.4e6 if (args.workload == "c3" and n == 1000000 and k == 90) else None
     out = {
         "metric": "gradient_iters_per_sec",
         "value": iters_per_s,
