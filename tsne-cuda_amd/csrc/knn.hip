@@ -746,10 +746,9 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
             // ~0 is "no threshold yet": its distance field does not decode to a number.
             const float limit_d = limit == ~0ull ? INFINITY : key_distance(limit);
             // Two candidate blocks at a time: two independent accumulator chains keep the matrix pipe busy.
-#pragma unroll
-            for (int cb = 0; cb < 4; cb += 2) {
-                v16f acc0 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                v16f acc1 = acc0;
+            auto multiply = [&](int cb, v16f &acc0, v16f &acc1) {
+                acc0 = v16f{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                acc1 = acc0;
                 const float4 *a0 = a_lds + (size_t)(buf * 4 + cb) * S4 * 64 + lane;
                 const float4 *a1 = a0 + S4 * 64;
 #pragma unroll
@@ -770,6 +769,8 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                         acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.w, bq[4 * s4 + 3], acc1, 0, 0, 0);
                     }
                 }
+            };
+            auto filter = [&](int cb, v16f &acc0, v16f &acc1) {
                 // Register v of lane l holds candidate row 8*(v/4) + 4*(l/32) + v%4 of the block, query column l%32.
                 // Smallest of the lane's 32 values, three operands per instruction (the accumulators are
                 // never signalling NaNs, so the library fminf's quieting moves are left out).
@@ -823,7 +824,21 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                     }
                     my_n += (int)(dst - dst0);
                 }
+            };
+            // The filter's stores to the lists count among the outstanding memory operations that the wait for
+            // the next tile's registers has to see through, so the second block pair is filtered only after the
+            // next tile has gone to LDS: what that wait then meets are the first pair's stores, a whole pair of
+            // matrix products old.
+            v16f acc0, acc1;
+            multiply(0, acc0, acc1);
+            filter(0, acc0, acc1);
+            multiply(2, acc0, acc1);
+            __syncthreads();  // all waves are done with tile `buf`
+            if (next_ct >= 0) {
+                stash(buf);
+                __syncthreads();
             }
+            filter(2, acc0, acc1);
             // Lists that a further tile could overflow are compacted by their own wave, right away.
             {
                 // (a region takes at most 64 entries per tile)
@@ -839,11 +854,6 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                     }
                     my_n = fill[tid];
                 }
-            }
-            __syncthreads();  // all waves are done with tile `buf`
-            if (next_ct >= 0) {
-                stash(buf);
-                __syncthreads();
             }
         };
 
