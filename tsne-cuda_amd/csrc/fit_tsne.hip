@@ -299,7 +299,6 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
                         "gradient step");
         } else {
             // Sampled steps run the phases one after the other so that the phase timers mean something.
-            TSNE_OR_DIE(tsnehip::launch_join(plan, stream), "stream join");
             hip_or_die(hipEventRecord(ev[0], stream), "event");
             TSNE_OR_DIE(tsnehip::launch_repulsive(plan, d_emb.as<float>(), slot, plan->rep, nullptr, nullptr, stream),
                         "repulsive forces");
@@ -317,11 +316,6 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         }
         slot ^= 1;
         if (timing) hip_or_die(hipEventRecord(ev[3], stream), "event");
-        // The host looks at this step's results: bring the side stream's work into `stream` first.
-        if (want_stop || printing || (want_dump && step % dump_interval == 0) ||
-            (want_snap && step % snap_interval == 0) || step + 1 == iterations)
-            TSNE_OR_DIE(tsnehip::launch_join(plan, stream), "stream join");
-
         // Norm of the step just taken (the reference prints it as "Avg. Gradient Norm").
         float grad_norm = 0.0f;
         if (want_stop || printing) {

@@ -82,8 +82,7 @@ struct tsne_hip_plan {
     // The repulsive chain and the attractive kernel of a step are independent: the fused loop runs
     // the chain on this side stream (default priority) and joins before the update.
     hipStream_t side_stream = nullptr;
-    hipEvent_t fork_event = nullptr, join_event = nullptr, update_event = nullptr;
-    bool side_open = false;  // the side stream holds steps the caller's stream has not joined yet
+    hipEvent_t fork_event = nullptr, join_event = nullptr;
     // The fused loop runs on this stream of the plan's own (default priority), tied to the caller's stream
     // by an event at either end: stream capture needs a stream that is not the legacy default one.
     hipStream_t loop_stream = nullptr;
@@ -127,8 +126,8 @@ int launch_pack_xy(tsne_hip_plan *p, const float *embedding, hipStream_t s);
 int launch_kl_terms(const float *pij, const int *indices, const float *embedding, int N, int K, double *out,
                     hipStream_t s);
 // One gradient step: repulsive chain, attractive forces (prepared pattern when pij is null), optional
-// normalisation output, update.  Unless profiling is on or TSNE_OVERLAP=0 is set, chain and update go to the
-// plan's side stream and overlap the attractive kernel on s; call launch_join before reading results.
+// normalisation output, update.  Unless profiling is on or TSNE_OVERLAP=0 is set, the chain goes to the plan's
+// side stream and overlaps the attractive kernel on s; the update on s waits for it, so s alone orders the results.
 int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
                 float *old_forces, float eta, float momentum, float exaggeration, int slot, float *normalization,
                 hipStream_t s);
@@ -140,7 +139,6 @@ int launch_steps(tsne_hip_plan *p, const float *pij, const int *indices, float *
                  hipStream_t s);
 // Makes stream s wait for the steps launch_step left on the side stream (no-op when there are none);
 // needed before anything else reads the loop's arrays.
-int launch_join(tsne_hip_plan *p, hipStream_t s);
 int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, float *attr, hipStream_t s);
 int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s);
 void release_blocked(tsne_hip_plan *p);
