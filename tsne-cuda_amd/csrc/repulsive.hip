@@ -30,6 +30,7 @@ namespace tsnehip {
 namespace {
 
 constexpr int kLog2Fft = 10;
+constexpr int kBothPairsMaxPoints = 262144;  // up to here the column pass transforms both plane pairs together
 
 __device__ __forceinline__ int rev4(int x) {
     // Reverse the five base-4 digits of a 10-bit index.
@@ -614,13 +615,18 @@ __global__ __launch_bounds__(256) void conv_rows_forward_kernel(float4 *__restri
 // spectrum column of each position is produced here from kernel_rows (one more
 // packed transform) so it never travels through memory.
 // ---------------------------------------------------------------------------
+// BOTH_PAIRS: the two plane pairs go through the transforms together (40 KB of LDS, half as many
+// stages one after the other) instead of one after the other (24 KB: what fits beside the attractive
+// kernel's workgroup on a CU; chosen for problem sizes where that kernel fills the chip).
+template <bool BOTH_PAIRS>
 __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restrict__ row_spectra, int G,
                                                            const float *__restrict__ kernel_rows,
                                                            const float2 *__restrict__ twiddles,
                                                            float2 *__restrict__ col_results) {
-    // 24 KB of LDS: the two plane pairs go through one after the other (the kernel columns are
-    // transformed with the first), twiddles come straight from memory.
-    __shared__ float2 s[3][kFft];  // [col], then the kernel columns
+    // Twiddles come straight from memory.  Layout: [pair in flight][col], then the kernel columns.
+    constexpr int kPairsInFlight = BOTH_PAIRS ? 2 : 1;
+    constexpr int kData = 2 * kPairsInFlight;  // transforms of data per round
+    __shared__ float2 s[kData + 1][kFft];
     const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int c0 = blockIdx.x * 2;
@@ -635,32 +641,33 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
                 v.x = kernel_rows[(size_t)v0 * kNodePad + a];
                 v.y = kernel_rows[(size_t)v1 * kNodePad + a];
             }
-            s[2][m] = v;
+            s[kData][m] = v;
         }
     }
-    for (int pair = 0; pair < 2; ++pair) {
-        for (int e = tid; e < 2 * kFft; e += 512) {
-            const int col = e >> kLog2Fft, m = e & (kFft - 1);
+    for (int pair0 = 0; pair0 < 2; pair0 += kPairsInFlight) {
+        for (int e = tid; e < kData * kFft; e += 512) {
+            const int t = e >> kLog2Fft, m = e & (kFft - 1);  // t = pair in flight * 2 + col
             float2 v = make_float2(0.f, 0.f);
-            if (m < G) v = row_spectra[((size_t)pair * kFft + c0 + col) * kNodePad + m];
-            s[col][m] = v;
+            if (m < G) v = row_spectra[((size_t)(pair0 + (t >> 1)) * kFft + c0 + (t & 1)) * kNodePad + m];
+            s[t][m] = v;
         }
         __syncthreads();
-        fft_forward(&s[0][0], pair == 0 ? 3 : 2, tw, tid, 512);
-        for (int e = tid; e < 2 * kFft; e += 512) {
-            const int col = e >> kLog2Fft, m = e & (kFft - 1);
-            const float2 kk = s[2][m];
-            const float kv = col ? kk.y : kk.x;
-            float2 v = s[col][m];
+        // (the kernel columns are transformed with the first round)
+        fft_forward(&s[0][0], pair0 == 0 ? kData + 1 : kData, tw, tid, 512);
+        for (int e = tid; e < kData * kFft; e += 512) {
+            const int t = e >> kLog2Fft, m = e & (kFft - 1);
+            const float2 kk = s[kData][m];
+            const float kv = (t & 1) ? kk.y : kk.x;
+            float2 v = s[t][m];
             v.x *= kv;
             v.y *= kv;
-            s[col][m] = v;
+            s[t][m] = v;
         }
         __syncthreads();
-        fft_inverse(&s[0][0], 2, tw, tid, 512);
-        for (int e = tid; e < 2 * kFft; e += 512) {
-            const int col = e >> kLog2Fft, m = e & (kFft - 1);
-            if (m < G) col_results[((size_t)pair * kFft + c0 + col) * kNodePad + m] = s[col][m];
+        fft_inverse(&s[0][0], kData, tw, tid, 512);
+        for (int e = tid; e < kData * kFft; e += 512) {
+            const int t = e >> kLog2Fft, m = e & (kFft - 1);
+            if (m < G) col_results[((size_t)(pair0 + (t >> 1)) * kFft + c0 + (t & 1)) * kNodePad + m] = s[t][m];
         }
         __syncthreads();
     }
@@ -817,7 +824,13 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
                                                                          p->twiddles, p->row_spectra, p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
-    conv_columns_kernel<<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
+    // Both plane pairs at once where the attractive kernel leaves the CUs mostly free anyway.
+    if (N <= kBothPairsMaxPoints)
+        conv_columns_kernel<true><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
+                                                           p->col_results);
+    else
+        conv_columns_kernel<false><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
+                                                            p->col_results);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvRowsInverse, s)) return 1;
     conv_rows_inverse_kernel<<<div_up(G, 2), 256, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
