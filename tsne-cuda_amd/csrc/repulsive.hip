@@ -30,6 +30,7 @@ namespace tsnehip {
 namespace {
 
 constexpr int kLog2Fft = 10;
+constexpr int kRowThreads = 512;  // threads of a row-pass workgroup (four transforms of 1024 points)
 constexpr int kBothPairsMaxPoints = 262144;  // up to here the column pass transforms both plane pairs together
 
 __device__ __forceinline__ int rev4(int x) {
@@ -539,7 +540,7 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
     const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
     const int a0 = block * 4;
-    for (int e = tid; e < 2 * kFft; e += 256) {
+    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
         const int f = e >> kLog2Fft, m = e & (kFft - 1);
         const int b = m < kFft / 2 ? m : kFft - m;
         const int ra = a0 + 2 * f;
@@ -551,8 +552,8 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
         s[f][m] = v;
     }
     __syncthreads();
-    fft_forward(&s[0][0], 2, tw, tid, 256);
-    for (int e = tid; e < 2 * kFft; e += 256) {
+    fft_forward(&s[0][0], 2, tw, tid, kRowThreads);
+    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
         const int f = e >> kLog2Fft, pos = e & (kFft - 1);
         const int v = rev4(pos);
         if (v <= kFft / 2) {
@@ -569,7 +570,7 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
 // starts from zero without a memset.  Output is transposed:
 // row_spectra[pair][pos][m], pos = digit-reversed frequency position.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void conv_rows_forward_kernel(float4 *__restrict__ w, int G, int n_boxes,
+__global__ __launch_bounds__(kRowThreads) void conv_rows_forward_kernel(float4 *__restrict__ w, int G, int n_boxes,
                                                                 const LoopScalars *sc, int slot,
                                                                 const float2 *__restrict__ twiddles,
                                                                 float2 *__restrict__ row_spectra,
@@ -588,7 +589,7 @@ __global__ __launch_bounds__(256) void conv_rows_forward_kernel(float4 *__restri
     }
     const int m0 = blockIdx.x * 2;
     const float s3 = r2_plane_scale(sc, slot);
-    for (int e = tid; e < 2 * kFft; e += 256) {
+    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
         const int r = e >> kLog2Fft, n = e & (kFft - 1);
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (n < G && m0 + r < G) {
@@ -600,8 +601,8 @@ __global__ __launch_bounds__(256) void conv_rows_forward_kernel(float4 *__restri
         s[r * 2 + 1][n] = make_float2(v.y, v.z);       // planes x and y
     }
     __syncthreads();
-    fft_forward(&s[0][0], 4, tw, tid, 256);
-    for (int e = tid; e < 2 * kFft; e += 256) {
+    fft_forward(&s[0][0], 4, tw, tid, kRowThreads);
+    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
         const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
         const float2 r0 = s[0 + pair][pos], r1 = s[2 + pair][pos];
         float4 *dst = reinterpret_cast<float4 *>(row_spectra + ((size_t)pair * kFft + pos) * kNodePad + m0);
@@ -677,7 +678,7 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
 // Inverse row pass for x nodes m0, m0+1: consumes digit-reversed positions,
 // produces node potentials in natural order, scaled by 1/1024^2.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void conv_rows_inverse_kernel(const float2 *__restrict__ col_results, int G,
+__global__ __launch_bounds__(kRowThreads) void conv_rows_inverse_kernel(const float2 *__restrict__ col_results, int G,
                                                                 const LoopScalars *sc, int slot,
                                                                 const float2 *__restrict__ twiddles,
                                                                 float4 *__restrict__ node_potentials) {
@@ -685,7 +686,7 @@ __global__ __launch_bounds__(256) void conv_rows_inverse_kernel(const float2 *__
     const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int m0 = blockIdx.x * 2;
-    for (int e = tid; e < 2 * kFft; e += 256) {
+    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
         const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
         const float4 v =
             *reinterpret_cast<const float4 *>(col_results + ((size_t)pair * kFft + pos) * kNodePad + m0);
@@ -693,10 +694,10 @@ __global__ __launch_bounds__(256) void conv_rows_inverse_kernel(const float2 *__
         s[2 + pair][pos] = make_float2(v.z, v.w);
     }
     __syncthreads();
-    fft_inverse(&s[0][0], 4, tw, tid, 256);
+    fft_inverse(&s[0][0], 4, tw, tid, kRowThreads);
     const float scale = 1.0f / ((float)kFft * (float)kFft);
     const float scale3 = scale / r2_plane_scale(sc, slot);
-    for (int e = tid; e < 2 * kFft; e += 256) {
+    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
         const int r = e >> kLog2Fft, n = e & (kFft - 1);
         if (n < G && m0 + r < G) {
             const float2 p0 = s[r * 2 + 0][n], p1 = s[r * 2 + 1][n];
@@ -820,7 +821,7 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
         TSNE_TRY(hipMemcpyAsync(charges_out, p->node_charges, sizeof(float4) * (size_t)G * G,
                                 hipMemcpyDeviceToDevice, s));
     if (profile_mark(p, kKernelConvRowsForward, s)) return 1;
-    conv_rows_forward_kernel<<<div_up(G, 2) + div_up(G, 4), 256, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
+    conv_rows_forward_kernel<<<div_up(G, 2) + div_up(G, 4), kRowThreads, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
                                                                          p->twiddles, p->row_spectra, p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
@@ -833,7 +834,7 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
                                                             p->col_results);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvRowsInverse, s)) return 1;
-    conv_rows_inverse_kernel<<<div_up(G, 2), 256, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
+    conv_rows_inverse_kernel<<<div_up(G, 2), kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
                                                           p->node_potentials);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelGather, s)) return 1;
