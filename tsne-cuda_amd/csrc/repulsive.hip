@@ -31,7 +31,9 @@ namespace {
 
 constexpr int kLog2Fft = 10;
 constexpr int kRowThreads = 512;  // threads of a row-pass workgroup (four transforms of 1024 points)
-constexpr int kBothPairsMaxPoints = 262144;  // up to here the column pass transforms both plane pairs together
+// Up to this many points the chain of repulsive kernels is what a step waits for (the attractive kernel beside it
+// is short): the column pass then transforms both plane pairs together and the tile sort gives every thread one point.
+constexpr int kSmallProblemPoints = 262144;
 
 __device__ __forceinline__ int rev4(int x) {
     // Reverse the five base-4 digits of a 10-bit index.
@@ -800,7 +802,8 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     const int tiles_per_dim = (nb + kTileBoxes - 1) / kTileBoxes;
     // Few, large workgroups: every workgroup ends with one global atomic per tile counter, and
     // same-address atomics serialise (about a thousand per counter cost ~20 us).
-    const int sort_blocks = std::min(div_up(N, 1024 * 4), kSortBlocks);
+    // (a small problem has workgroups to spare: one point per thread shortens the kernel by three rounds)
+    const int sort_blocks = std::min(div_up(N, N <= kSmallProblemPoints ? 1024 : 1024 * 4), kSortBlocks);
     if (profile_mark(p, kKernelTileCount, s)) return 1;
     tile_count_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, slot ^ 1, nb, p->tile_count,
                                                    p->tile_cursor, p->chunks, p->num_chunks, p->num_chunks + 1,
@@ -826,7 +829,7 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
     // Both plane pairs at once where the attractive kernel leaves the CUs mostly free anyway.
-    if (N <= kBothPairsMaxPoints)
+    if (N <= kSmallProblemPoints)
         conv_columns_kernel<true><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
                                                            p->col_results);
     else
