@@ -31,9 +31,6 @@ namespace {
 
 constexpr int kLog2Fft = 10;
 constexpr int kRowThreads = 512;  // threads of a row-pass workgroup (four transforms of 1024 points)
-// Up to this many points the chain of repulsive kernels is what a step waits for (the attractive kernel beside it
-// is short): the column pass then transforms both plane pairs together and the tile sort gives every thread one point.
-constexpr int kSmallProblemPoints = 262144;
 
 __device__ __forceinline__ int rev4(int x) {
     // Reverse the five base-4 digits of a 10-bit index.
@@ -618,16 +615,15 @@ __global__ __launch_bounds__(kRowThreads) void conv_rows_forward_kernel(float4 *
 // spectrum column of each position is produced here from kernel_rows (one more
 // packed transform) so it never travels through memory.
 // ---------------------------------------------------------------------------
-// BOTH_PAIRS: the two plane pairs go through the transforms together (40 KB of LDS, half as many
-// stages one after the other) instead of one after the other (24 KB: what fits beside the attractive
-// kernel's workgroup on a CU; chosen for problem sizes where that kernel fills the chip).
-template <bool BOTH_PAIRS>
+// The two plane pairs go through the transforms together (40 KB of LDS): half as many stages one after
+// the other as with one pair at a time (24 KB, which would also fit beside the attractive kernel's
+// workgroup on a CU: no faster at a million points, 3-4 % slower per step from 5000 to 800000).
 __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restrict__ row_spectra, int G,
                                                            const float *__restrict__ kernel_rows,
                                                            const float2 *__restrict__ twiddles,
                                                            float2 *__restrict__ col_results) {
     // Twiddles come straight from memory.  Layout: [pair in flight][col], then the kernel columns.
-    constexpr int kPairsInFlight = BOTH_PAIRS ? 2 : 1;
+    constexpr int kPairsInFlight = 2;
     constexpr int kData = 2 * kPairsInFlight;  // transforms of data per round
     __shared__ float2 s[kData + 1][kFft];
     const float2 *tw = twiddles;
@@ -802,8 +798,8 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     const int tiles_per_dim = (nb + kTileBoxes - 1) / kTileBoxes;
     // Few, large workgroups: every workgroup ends with one global atomic per tile counter, and
     // same-address atomics serialise (about a thousand per counter cost ~20 us).
-    // (a small problem has workgroups to spare: one point per thread shortens the kernel by three rounds)
-    const int sort_blocks = std::min(div_up(N, N <= kSmallProblemPoints ? 1024 : 1024 * 4), kSortBlocks);
+    // (one point per thread until that many workgroups are in use)
+    const int sort_blocks = std::min(div_up(N, 1024), kSortBlocks);
     if (profile_mark(p, kKernelTileCount, s)) return 1;
     tile_count_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, slot ^ 1, nb, p->tile_count,
                                                    p->tile_cursor, p->chunks, p->num_chunks, p->num_chunks + 1,
@@ -828,13 +824,7 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
                                                                          p->twiddles, p->row_spectra, p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
-    // Both plane pairs at once where the attractive kernel leaves the CUs mostly free anyway.
-    if (N <= kSmallProblemPoints)
-        conv_columns_kernel<true><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
-                                                           p->col_results);
-    else
-        conv_columns_kernel<false><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
-                                                            p->col_results);
+    conv_columns_kernel<<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvRowsInverse, s)) return 1;
     conv_rows_inverse_kernel<<<div_up(G, 2), kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
