@@ -137,8 +137,8 @@ static bool graphs_enabled(const tsne_hip_plan *p) {
     const int mode = v ? (v[0] == '0' ? 0 : 1) : -1;
     if (p->profiling || sync_kernels_enabled() || mode == 0) return false;
     // Measured gain per step: 15 % at 5000-60000 points, 2-3.5 % at 400000-800000, 0.3 % at a million; setting a
-    // graph up costs 5-35 ms (growing with the point count), so it is the default where a few hundred steps repay it.
-    return mode == 1 || p->num_points <= 262144;
+    // graph up costs about 4 ms whatever the size.
+    return mode == 1 || p->num_points <= 1048576;
 }
 
 int launch_steps(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,

@@ -290,22 +290,26 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         const bool timing = printing;  // phase timers sample the steps that already synchronise
 
         const bool want_norm = step + 1 == iterations || want_stop;
-        if (!verbose && !want_stop && !want_dump && !want_snap && N <= 65536 && iterations >= 500) {
+        if (!verbose && !want_stop && !want_dump && !want_snap) {
             // Nothing looks at the steps in between: everything up to the schedule switch, or up to the last
-            // step (launched singly below: it delivers the normalisation), goes out as one batch, which
-            // replays a captured graph of two steps.  Setting the two graphs up costs 10 ms at 5000 points and
-            // more with every point (70 ms at a million), replaying saves ~15 us per step: over a fit's 1000
-            // steps that pays up to about 60000 points.
+            // step (launched singly below: it delivers the normalisation), goes out as one batch on the plan's
+            // own stream (tied to `stream` by an event at either end), where problems of up to 262144 points
+            // replay a captured graph of two steps: ~4 ms to set up per schedule, 10-15 us saved per step.
             size_t run_end = iterations - 1;
             if (!late && opt.force_magnify_iters >= 0)
                 run_end = std::min(run_end, (size_t)opt.force_magnify_iters);
             if (run_end > step + 1) {
                 const size_t count = std::min<size_t>(run_end - step, 1u << 30);
+                hipStream_t batch_stream = plan->loop_stream;
+                hip_or_die(hipEventRecord(plan->enter_event, stream), "event");
+                hip_or_die(hipStreamWaitEvent(batch_stream, plan->enter_event, 0), "event");
                 TSNE_OR_DIE(tsnehip::launch_steps(plan, blocked ? nullptr : d_pij.as<float>(),
                                                   blocked ? nullptr : d_idx.as<int>(), d_emb.as<float>(),
                                                   d_gains.as<float>(), d_old.as<float>(), opt.learning_rate,
-                                                  momentum, exaggeration, (int)count, slot, stream),
+                                                  momentum, exaggeration, (int)count, slot, batch_stream),
                             "gradient steps");
+                hip_or_die(hipEventRecord(plan->leave_event, batch_stream), "event");
+                hip_or_die(hipStreamWaitEvent(stream, plan->leave_event, 0), "event");
                 step += count - 1;
                 continue;
             }
