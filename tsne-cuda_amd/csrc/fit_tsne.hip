@@ -293,7 +293,7 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         if (!verbose && !want_stop && !want_dump && !want_snap) {
             // Nothing looks at the steps in between: everything up to the schedule switch, or up to the last
             // step (launched singly below: it delivers the normalisation), goes out as one batch on the plan's
-            // own stream (tied to `stream` by an event at either end), where problems of up to 262144 points
+            // own stream (tied to `stream` by an event at either end), where problems of up to about a million points
             // replay a captured graph of two steps: ~4 ms to set up per schedule, 10-15 us saved per step.
             size_t run_end = iterations - 1;
             if (!late && opt.force_magnify_iters >= 0)
