@@ -341,6 +341,35 @@ def test_attractive_wait_that_runs_out_is_reported(stages, monkeypatch):
     plan.close()
 
 
+def test_iterate_after_preparing_a_second_pattern(stages, c0_problem):
+    """Steps replay captured graphs, which hold the addresses of the re-blocked
+    pattern: preparing another pattern in the same plan must drop them.  The
+    second run has to follow the second pattern, like a fresh plan does."""
+    c = c0_problem
+    n, k = c["P"].shape
+    dP, di = dev(c["P"]), dev(c["idx"])
+    rng = np.random.default_rng(9)
+    P2 = (c["P"] * rng.uniform(0.5, 1.5, c["P"].shape)).astype(np.float32)
+
+    def run(plan, first):
+        if first:
+            plan.prepare_attractive(dP, di)
+            y = dev(c["y0"]).clone()
+            plan.iterate_(None, None, y, torch.ones_like(y), torch.zeros_like(y), 0, 6, eta=200.0)
+        plan.prepare_attractive(dev(P2), di)
+        y = dev(c["y0"]).clone()
+        gains, old = torch.ones_like(y), torch.zeros_like(y)
+        plan.iterate_(None, None, y, gains, old, 0, 6, eta=200.0)
+        torch.cuda.synchronize()
+        return y.cpu().numpy()
+
+    plan_a, plan_b = stages.Plan(n, k), stages.Plan(n, k)
+    twice, once = run(plan_a, True), run(plan_b, False)
+    plan_a.close()
+    plan_b.close()
+    assert rel_l2(twice, once) <= 1e-5
+
+
 def test_attractive_blocked_clustered_pattern(stages):
     """A pattern whose rows reference only a few column partitions (what the
     locality ordering produces): runs longer than one work item share a staged

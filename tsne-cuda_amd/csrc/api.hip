@@ -260,6 +260,7 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     if (p->fork_event) (void)hipEventDestroy(p->fork_event);
     if (p->join_event) (void)hipEventDestroy(p->join_event);
     for (auto &g : p->step_graphs) (void)hipGraphExecDestroy(g.exec);
+    p->step_graphs.clear();
     if (p->enter_event) (void)hipEventDestroy(p->enter_event);
     if (p->leave_event) (void)hipEventDestroy(p->leave_event);
     if (p->loop_stream) (void)hipStreamDestroy(p->loop_stream);

@@ -461,6 +461,9 @@ void release_blocked(tsne_hip_plan *p) {
     p->ent_p = nullptr;
     p->seg = nullptr;
     p->blocked_ready = false;
+    // Captured steps hold the addresses just freed (hipFree has waited for the device, so none is running).
+    for (auto &g : p->step_graphs) (void)hipGraphExecDestroy(g.exec);
+    p->step_graphs.clear();
 }
 
 int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s) {
