@@ -370,6 +370,57 @@ def test_iterate_after_preparing_a_second_pattern(stages, c0_problem):
     assert rel_l2(twice, once) <= 1e-5
 
 
+def test_plan_closed_or_reprepared_while_steps_are_in_flight(stages, c0_problem):
+    """iterate_ returns while its steps (a replaying graph here) still run.  Closing the
+    plan, or preparing another pattern in it, right away - no synchronisation in
+    between - must wait for them: the embedding ends where a synchronised run ends."""
+    c = c0_problem
+    n, k = c["P"].shape
+    dP, di = dev(c["P"]), dev(c["idx"])
+
+    def run(after):
+        plan = stages.Plan(n, k)
+        plan.prepare_attractive(dP, di)
+        y = dev(c["y0"]).clone()
+        gains, old = torch.ones_like(y), torch.zeros_like(y)
+        plan.iterate_(None, None, y, gains, old, 0, 40)
+        after(plan)
+        torch.cuda.synchronize()
+        return y.cpu().numpy()
+
+    def sync_then_close(plan):
+        torch.cuda.synchronize()
+        plan.close()
+
+    def reprepare(plan):
+        plan.prepare_attractive(dP, di)
+        plan.close()
+
+    want = run(sync_then_close)
+    assert np.isfinite(want).all()
+    assert rel_l2(run(lambda plan: plan.close()), want) <= 1e-5
+    assert rel_l2(run(reprepare), want) <= 1e-5
+
+
+def test_prepare_reports_unsupported_shapes_apart_from_failures(stages):
+    """A pattern the blocked format cannot hold (num_neighbors >= 4096) is status 2, which
+    callers may answer by keeping the row-ordered kernel; the plan goes on working with an
+    explicit pattern."""
+    n, k = 4200, 4100
+    rng = np.random.default_rng(3)
+    idx = rng.integers(0, n, (n, k)).astype(np.int32)
+    P = (rng.random((n, k)) * 1e-6).astype(np.float32)
+    y = (rng.standard_normal(2 * n) * 3.0).astype(np.float32)
+    plan = stages.Plan(n, k)
+    dP, di = dev(P), dev(idx)
+    rc = stages.lib().tsne_hip_attractive_prepare(plan._h, dP.data_ptr(), di.data_ptr(), None)
+    assert rc == 2
+    assert b"too large for the blocked format" in stages.lib().tsne_hip_last_error()
+    got = plan.attractive(dP, di, dev(y)).cpu().numpy()
+    assert rel_l2(got, oracle.attractive(P, idx, y)) <= 1e-4
+    plan.close()
+
+
 def test_attractive_blocked_clustered_pattern(stages):
     """A pattern whose rows reference only a few column partitions (what the
     locality ordering produces): runs longer than one work item share a staged

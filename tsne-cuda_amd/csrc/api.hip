@@ -256,6 +256,14 @@ int tsne_hip_symmetrize(const float *pij_non_symmetric, const int *indices, int 
 
 void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     if (!p) return;
+    // tsne_hip_iterate returns while its steps (or a replaying graph) are still running: nothing of the plan
+    // may go before its streams and its device are idle.
+    int current = -1;
+    const bool switched = hipGetDevice(&current) == hipSuccess && current != p->device &&
+                          hipSetDevice(p->device) == hipSuccess;
+    if (p->loop_stream) (void)hipStreamSynchronize(p->loop_stream);
+    if (p->side_stream) (void)hipStreamSynchronize(p->side_stream);
+    (void)hipDeviceSynchronize();
     for (hipEvent_t e : p->events) (void)hipEventDestroy(e);
     if (p->fork_event) (void)hipEventDestroy(p->fork_event);
     if (p->join_event) (void)hipEventDestroy(p->join_event);
@@ -284,6 +292,7 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     (void)hipFree(p->attr);
     (void)hipFree(p->rep);
     delete p;
+    if (switched) (void)hipSetDevice(current);
 }
 
 int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors, int n_boxes_per_dim,

@@ -456,14 +456,18 @@ static_assert(kBlockedLds <= 160 * 1024, "one workgroup must fit the 160 KB of L
 }  // namespace
 
 void release_blocked(tsne_hip_plan *p) {
+    // Steps may still be running (tsne_hip_iterate is asynchronous) and captured steps hold the addresses
+    // about to be freed: wait for the plan's own streams and the device before anything is destroyed.
+    if (p->loop_stream) (void)hipStreamSynchronize(p->loop_stream);
+    if (p->side_stream) (void)hipStreamSynchronize(p->side_stream);
+    (void)hipDeviceSynchronize();
+    for (auto &g : p->step_graphs) (void)hipGraphExecDestroy(g.exec);
+    p->step_graphs.clear();
     (void)hipFree(p->ent_p);
     (void)hipFree(p->seg);
     p->ent_p = nullptr;
     p->seg = nullptr;
     p->blocked_ready = false;
-    // Captured steps hold the addresses just freed (hipFree has waited for the device, so none is running).
-    for (auto &g : p->step_graphs) (void)hipGraphExecDestroy(g.exec);
-    p->step_graphs.clear();
 }
 
 int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s) {
@@ -473,7 +477,7 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     if (n_parts > kMaxParts) {
         set_error("attractive_prepare: %d points need %d column partitions, more than the %d supported", N, n_parts,
                   kMaxParts);
-        return 1;
+        return kShapeNotSupported;
     }
     int cus = 256;
     TSNE_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, p->device));
@@ -484,7 +488,7 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     // Segment offsets are 32-bit and a row sum of K fixed-point terms must stay below 2^62.
     if ((int64_t)strip_rows * K >= (int64_t)1 << 31 || K >= 4096) {
         set_error("attractive_prepare: num_neighbors = %d is too large for the blocked format", K);
-        return 1;
+        return kShapeNotSupported;
     }
     p->strip_rows = strip_rows;
     p->n_strips = div_up(N, strip_rows);

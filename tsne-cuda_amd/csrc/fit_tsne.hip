@@ -248,7 +248,11 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     // Re-block the sparse pattern for the LDS-staged attractive kernel; shapes it
     // cannot hold (very large K or N) keep the row-ordered kernel.
     // (The row-ordered pattern stays: the objective of the final embedding is evaluated on it.)
-    const bool blocked = tsnehip::prepare_blocked(plan, d_pij.as<float>(), d_idx.as<int>(), stream) == 0;
+    const int prepared = tsnehip::prepare_blocked(plan, d_pij.as<float>(), d_idx.as<int>(), stream);
+    if (prepared != 0 && prepared != tsnehip::kShapeNotSupported) die("re-blocking of the sparse pattern");
+    const bool blocked = prepared == 0;
+    if (!blocked && verbose)
+        std::cout << "(" << tsnehip::last_error() << "; using the row-ordered attractive kernel) " << std::flush;
 
     std::ofstream dump_file;
     if (opt.get_dump_points()) {

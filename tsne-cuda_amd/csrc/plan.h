@@ -140,6 +140,10 @@ int launch_steps(tsne_hip_plan *p, const float *pij, const int *indices, float *
 // Makes stream s wait for the steps launch_step left on the side stream (no-op when there are none);
 // needed before anything else reads the loop's arrays.
 int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, float *attr, hipStream_t s);
+// Returns 0, kShapeNotSupported when the blocked format cannot hold the problem (more than 8192 column
+// partitions, num_neighbors >= 4096, or a strip of more than 2^31 entries; the row-ordered kernel then
+// serves), or 1 for any other failure (allocation, launch).
+constexpr int kShapeNotSupported = 2;
 int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s);
 void release_blocked(tsne_hip_plan *p);
 int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s);
