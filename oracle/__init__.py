@@ -37,6 +37,7 @@ def lib():
         L.oracle_iterate.restype = ctypes.c_float
         L.oracle_fit.restype = ctypes.c_float
         L.oracle_kl.restype = ctypes.c_double
+        L.oracle_row_sum.restype = ctypes.c_float
         _lib = L
     return _lib
 
@@ -76,6 +77,28 @@ def perplexity(d2, perplexity, eps, return_search=False):
     lib().oracle_perplexity(_opt(d2), N, K, ctypes.c_float(perplexity), ctypes.c_float(eps), _opt(p), _opt(beta),
                             _opt(iters))
     return (p, beta, iters) if return_search else p
+
+
+def expf(x):
+    """The search's exp (a fixed sequence of fp32 operations), element-wise."""
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty_like(x)
+    lib().oracle_expf_array(_opt(x), ctypes.c_int64(x.size), _opt(out))
+    return out
+
+
+def logf(v):
+    """The search's log, element-wise."""
+    v = np.ascontiguousarray(v, np.float32)
+    out = np.empty_like(v)
+    lib().oracle_logf_array(_opt(v), ctypes.c_int64(v.size), _opt(out))
+    return out
+
+
+def row_sum(v):
+    """Sum of a row in the search's stated order (64 interleaved partial sums, then a balanced tree)."""
+    v = np.ascontiguousarray(v, np.float32).ravel()
+    return float(lib().oracle_row_sum(_opt(v), int(v.size)))
 
 
 def symmetrize(p, idx):

@@ -22,7 +22,9 @@
 // Pinning status (what fixes each function independently of this file):
 //   knn         brute force over numpy float32 arithmetic + sklearn brute kNN
 //   max_norm    closed form
-//   perplexity  row sums, entropy target, uniform closed form, sklearn bisection
+//   perplexity  row sums, entropy target, uniform closed form, sklearn bisection;
+//               its exp / log against double-precision exp / log (<= 2 units in the last place),
+//               its row-sum order against an exact (fsum) sum
 //   symmetrize  dense (A + A^T)/2N masked to the pattern
 //   attractive  dense O(N^2) sum
 //   repulsive   direct node-to-node convolution on reduced grids, numpy FFT at
@@ -267,6 +269,103 @@ float oracle_max_normalize(float *d2, int64_t n) {
     return m;
 }
 
+// exp and log as fixed sequences of correctly rounded single-precision operations (any machine that
+// follows the sequence gets the same bits), accurate to about one unit in the last place.  The perplexity
+// search stops on |H - ln perplexity| < eps, so the last bit of an exponential can move a row's stopping
+// point by a whole bisection step; the reference's __expf / __logf (perplexity_search.cu:32,
+// thrust_transform_functions.h:34) cannot be reproduced bit for bit anywhere but on its own GPU, and any
+// exp/log this accurate is as good a restatement.  These two are pinned against double-precision
+// exp / log in tests/test_oracle.py.
+static inline float bits_to_float(uint32_t u) {
+    float f;
+    std::memcpy(&f, &u, sizeof(f));
+    return f;
+}
+static inline uint32_t float_to_bits(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, sizeof(u));
+    return u;
+}
+
+// e^x: n = round(x log2 e) by the 1.5 * 2^23 trick, r = x - n ln2 with a split ln2, degree-7 Taylor
+// polynomial (Horner, fused multiply-adds), scaling by 2^n in two exact power-of-two factors.
+float oracle_expf(float x) {
+    if (x != x) return x;
+    if (!(x > -104.0f)) return 0.0f;
+    if (x > 88.72f) return bits_to_float(0x7f800000u);
+    const float t = std::fmaf(x, 1.44269504f, 12582912.0f);
+    const float n = t - 12582912.0f;
+    float r = std::fmaf(n, -0.693145752f, x);
+    r = std::fmaf(n, -1.42860677e-6f, r);
+    float p = 1.0f / 5040.0f;
+    p = std::fmaf(p, r, 1.0f / 720.0f);
+    p = std::fmaf(p, r, 1.0f / 120.0f);
+    p = std::fmaf(p, r, 1.0f / 24.0f);
+    p = std::fmaf(p, r, 1.0f / 6.0f);
+    p = std::fmaf(p, r, 0.5f);
+    p = std::fmaf(p, r, 1.0f);
+    p = std::fmaf(p, r, 1.0f);
+    const int ni = (int)n;
+    const int half = ni / 2;
+    const float a = bits_to_float((uint32_t)(half + 127) << 23);
+    const float b = bits_to_float((uint32_t)(ni - half + 127) << 23);
+    return (p * a) * b;
+}
+
+// ln v: v = m 2^e, m in [sqrt(1/2), sqrt(2)); f = m - 1, s = f / (2 + f), z = s^2,
+// ln m = f - s (f - R), R = z (2/3 + z (2/5 + z (2/7 + z (2/9 + z 2/11)))); ln v = e ln2_hi + (ln m + e ln2_lo).
+float oracle_logf(float v) {
+    if (v != v) return v;
+    if (v < 0.0f) return bits_to_float(0x7fc00000u);
+    if (v == 0.0f) return bits_to_float(0xff800000u);
+    uint32_t bits = float_to_bits(v);
+    if (bits == 0x7f800000u) return v;
+    int e = 0;
+    if (bits < 0x00800000u) {  // subnormal
+        v = v * 33554432.0f;
+        bits = float_to_bits(v);
+        e = -25;
+    }
+    bits += 0x3f800000u - 0x3f3504f3u;
+    e += (int)(bits >> 23) - 127;
+    bits = (bits & 0x007fffffu) + 0x3f3504f3u;
+    const float f = bits_to_float(bits) - 1.0f;
+    const float s = f / (2.0f + f);
+    const float z = s * s;
+    float R = 2.0f / 11.0f;
+    R = std::fmaf(R, z, 2.0f / 9.0f);
+    R = std::fmaf(R, z, 2.0f / 7.0f);
+    R = std::fmaf(R, z, 2.0f / 5.0f);
+    R = std::fmaf(R, z, 2.0f / 3.0f);
+    R = R * z;
+    const float ef = (float)e;
+    float res = std::fmaf(ef, 1.42860677e-6f, -(s * (f - R)));
+    res = res + f;
+    return std::fmaf(ef, 0.693145752f, res);
+}
+
+// Row sum in the stated order of the search: 64 interleaved partial sums (partial c takes slots c, c + 64,
+// c + 128, ... in ascending order, starting from +0), then a balanced tree, partial[c] + partial[c ^ m] for
+// m = 32, 16, 8, 4, 2, 1.  (The reference sums a row with cublasSgemv, reduce_utils.cu:24-27, whose order is
+// not documented; a pairwise order is what a GPU reduction does and it is one a GPU kernel can follow.)
+static inline float ordered_row_sum(const float *v, int K) {
+    float part[64];
+    for (int c = 0; c < 64; ++c) part[c] = 0.0f;
+    for (int s = 0; s < K; ++s) part[s & 63] += v[s];
+    for (int m = 32; m > 0; m >>= 1)
+        for (int c = 0; c < m; ++c) part[c] = part[c] + part[c + m];
+    return part[0];
+}
+
+// Array forms of the three helpers above, for the tests that pin them.
+void oracle_expf_array(const float *x, int64_t n, float *out) {
+    for (int64_t t = 0; t < n; ++t) out[t] = oracle_expf(x[t]);
+}
+void oracle_logf_array(const float *v, int64_t n, float *out) {
+    for (int64_t t = 0; t < n; ++t) out[t] = oracle_logf(v[t]);
+}
+float oracle_row_sum(const float *v, int K) { return ordered_row_sum(v, K); }
+
 // src/kernels/perplexity_search.cu:81-141.  Rows are independent: the
 // reference iterates all rows in lock-step and freezes converged rows, which is
 // the same as running each row until it converges or 200 evaluations are done.
@@ -275,10 +374,10 @@ float oracle_max_normalize(float *d2, int64_t n) {
 // evaluations.
 void oracle_perplexity(const float *d2, int N, int K, float perplexity, float eps, float *p, float *beta_out,
                        int *iters_out) {
-    const float log_target = std::log(perplexity);
+    const float log_target = oracle_logf(perplexity);
 #pragma omp parallel
     {
-        std::vector<float> row(K);
+        std::vector<float> row(K), ent_terms(K);
 #pragma omp for schedule(static)
         for (int i = 0; i < N; ++i) {
             const float *d = d2 + (size_t)i * K;
@@ -286,22 +385,21 @@ void oracle_perplexity(const float *d2, int N, int K, float perplexity, float ep
             float used_beta = beta, sum = 0.0f;
             int it = 0;
             for (;;) {
-                sum = 0.0f;
-                float ent = 0.0f;
                 for (int s = 0; s < K; ++s) {
                     // perplexity_search.cu:32
-                    const float v = (s == 0 && d[s] == 0.0f) ? 0.0f : std::exp(-beta * d[s]);
+                    const float v = (s == 0 && d[s] == 0.0f) ? 0.0f : oracle_expf(-beta * d[s]);
                     row[s] = v;
-                    sum += v;
                     // thrust_transform_functions.h:32-37
-                    float e = v * std::log(v);
+                    float e = v * oracle_logf(v);
                     if (e != e || std::isinf(e)) e = 0.0f;
-                    ent += e;
+                    ent_terms[s] = e;
                 }
+                sum = ordered_row_sum(row.data(), K);
+                const float ent = ordered_row_sum(ent_terms.data(), K);
                 used_beta = beta;
                 ++it;
                 const float neg_ent = -ent;
-                const float H = (neg_ent / sum) + std::log(sum);
+                const float H = (neg_ent / sum) + oracle_logf(sum);
                 const float diff = H - log_target;
                 const bool found = (diff < eps && -diff < eps);
                 if (found || it >= 200) break;

@@ -153,6 +153,75 @@ def test_perplexity_against_sklearn(small):
     np.testing.assert_allclose(ours, ref, rtol=2e-3, atol=1e-7)
 
 
+def _ulp_error(got, exact):
+    """|got - exact| in units of the last place of the fp32 result nearest to `exact`."""
+    exact = np.asarray(exact, np.float64)
+    ref = exact.astype(np.float32)
+    spacing = np.spacing(np.abs(ref)).astype(np.float64)
+    spacing = np.maximum(spacing, 2.0 ** -149)
+    return np.abs(got.astype(np.float64) - exact) / spacing
+
+
+def test_search_exp_against_double_precision():
+    # The search's exp is a hand-written operation sequence; what pins it is the double-precision
+    # exponential (numpy / libm), over its whole range including results that are subnormal.
+    rng = np.random.default_rng(0)
+    x = np.concatenate([np.linspace(-103.9, 0.0, 200001), -np.abs(rng.standard_cauchy(100000)),
+                        np.linspace(0.0, 88.7, 20001), -rng.random(50000) * 1e-3]).astype(np.float32)
+    x = x[x > -104.0]
+    got = oracle.expf(x)
+    err = _ulp_error(got, np.exp(x.astype(np.float64)))
+    assert err.max() <= 2.0, err.max()
+    assert np.mean(err <= 1.0) > 0.99
+    assert np.all(np.diff(oracle.expf(np.sort(x))) >= 0)  # monotone
+    edge = oracle.expf(np.array([0.0, -np.inf, -200.0, np.inf, 100.0], np.float32))
+    assert edge[0] == 1.0 and edge[1] == 0.0 and edge[2] == 0.0 and np.isinf(edge[3]) and np.isinf(edge[4])
+    assert np.isnan(oracle.expf(np.array([np.nan], np.float32))[0])
+
+
+def test_search_log_against_double_precision():
+    rng = np.random.default_rng(1)
+    v = np.concatenate([np.exp(rng.uniform(-103.0, 88.0, 300000)), np.linspace(0.5, 2.0, 100001),
+                        1.0 + rng.standard_normal(50000) * 1e-4, rng.uniform(0.0, 100.0, 50000)]).astype(np.float32)
+    v = v[v > 0]
+    got = oracle.logf(v)
+    exact = np.log(v.astype(np.float64))
+    err = _ulp_error(got, exact)
+    # Next to 1 the result is tiny and its last place with it: bound the absolute error there.
+    near_one = np.abs(v - 1.0) < 0.05
+    assert err[~near_one].max() <= 2.0, err[~near_one].max()
+    assert np.abs(got[near_one] - exact[near_one]).max() <= 2.0 ** -25
+    edge = oracle.logf(np.array([1.0, 0.0, np.inf, -1.0, 1e-45], np.float32))
+    assert edge[0] == 0.0 and edge[1] == -np.inf and edge[2] == np.inf and np.isnan(edge[3])
+    assert abs(edge[4] - np.log(float(np.float32(1e-45)))) < 1e-4
+
+
+def test_search_row_sum_order():
+    import math
+    rng = np.random.default_rng(2)
+    for k in (1, 3, 63, 64, 65, 90, 128, 129, 1100):
+        v = rng.random(k).astype(np.float32)
+        exact = math.fsum(float(t) for t in v)
+        assert abs(oracle.row_sum(v) - exact) <= 8 * np.spacing(np.float32(exact))
+    # Integer-valued floats: every order gives the exact sum.
+    v = rng.integers(0, 1000, 500).astype(np.float32)
+    assert oracle.row_sum(v) == float(v.astype(np.float64).sum())
+    # The order itself, followed by hand on a case where it shows: slots 0 and 64 share partial 0 and cancel
+    # there before anything else is added; a sequential sum would have absorbed the 1 at slot 1 into 2^30.
+    v = np.zeros(70, np.float32)
+    v[0], v[64], v[1] = 2.0 ** 30, -2.0 ** 30, 1.0
+    assert oracle.row_sum(v) == 1.0
+    assert float(np.add.accumulate(np.array([2.0 ** 30, 1.0, -2.0 ** 30], np.float32))[-1]) == 0.0
+    # ... and slots 0 and 32 only meet at the top of the tree (m = 32), after slot 1 met slot 33:
+    v = np.zeros(70, np.float32)
+    v[0], v[32], v[1], v[33] = 2.0 ** 30, -2.0 ** 30, 1.0, 1.0
+    assert oracle.row_sum(v) == 2.0
+    # ... whereas slots 0 and 1 meet last (m = 1), so a unit at slot 2 is absorbed by slot 0 first (m = 2):
+    v = np.zeros(70, np.float32)
+    v[0], v[1], v[2] = 2.0 ** 30, -2.0 ** 30, 1.0
+    assert oracle.row_sum(v) == 0.0
+
+
 # ---------------------------------------------------------- symmetrize ------
 def test_symmetrize_dense(small):
     n, k, idx, p, P = small["n"], small["k"], small["idx"], small["p"], small["P"]

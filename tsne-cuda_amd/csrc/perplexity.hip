@@ -8,6 +8,19 @@
 // lanes owns a row, keeps its distances in registers and runs the whole
 // bisection privately: the distances are read once and the probabilities
 // written once.
+//
+// Reproducible arithmetic.  Whether a row stops at one bisection step or the
+// next hangs on the last bits of its entropy, so every operation of the search
+// is pinned down: exp and log are the fixed operation sequences of det_math.h,
+// nothing is contracted, and the two row sums (of p and of p ln p) are formed in
+// one stated order whatever the kernel variant:
+//   * 64 interleaved partial sums, partial c taking the values of the slots
+//     s = c, c + 64, c + 128, ... in ascending order, starting from +0;
+//   * then a balanced tree: partial[c] + partial[c ^ m] for m = 32, 16, 8, 4, 2, 1.
+// A CPU restatement that follows the same order gets the same probabilities bit
+// for bit.  (The reference's sums are cuBLAS sgemv calls whose order is not
+// documented, and its exp/log are the fast intrinsics.)
+#include "det_math.h"
 #include "plan.h"
 
 #include <algorithm>
@@ -38,8 +51,29 @@ __global__ void zero_scalar_kernel(float *p) {
 
 // thrust_transform_functions.h:32-37: x*log(x) with NaN/Inf mapped to 0.
 __device__ __forceinline__ float entropy_term(float v) {
-    const float e = v * logf(v);
+#pragma clang fp contract(off)
+    const float e = v * det_logf(v);
     return (e != e || isinf(e)) ? 0.0f : e;
+}
+
+// The stated summation order for a group of LANES lanes whose lane l holds the slots l + v * LANES: a lane
+// owns 64 / LANES of the 64 partial sums (classes l + LANES * (v mod (64 / LANES))); it forms them one after
+// the other, combines them by the upper levels of the tree, and the lower levels run across the lanes.
+template <int LANES, int VPL>
+__device__ __forceinline__ float ordered_row_sum(const float (&val)[VPL]) {
+#pragma clang fp contract(off)
+    constexpr int kClasses = kWave / LANES;
+    float q[kClasses];
+#pragma unroll
+    for (int c = 0; c < kClasses; ++c) q[c] = 0.0f;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) q[v % kClasses] += val[v];
+    // Class index c * LANES + lane: the tree's level m = 32 pairs classes c and c ^ (32 / LANES), and so on down.
+#pragma unroll
+    for (int m = kClasses / 2; m > 0; m >>= 1)
+#pragma unroll
+        for (int c = 0; c < m; ++c) q[c] += q[c + m];
+    return group_sum<LANES>(q[0]);
 }
 
 // One row per LANES-lane group, VPL values per lane held in registers.
@@ -70,19 +104,18 @@ __global__ __launch_bounds__(256) void perplexity_kernel(const float *__restrict
     bool done = !live;
     for (int it = 0; it < 200; ++it) {
         if (!done) {
-            float ls = 0.0f, le = 0.0f;
+            float et[VPL];
 #pragma unroll
             for (int v = 0; v < VPL; ++v) {
                 const int s = lane + v * LANES;
                 float pv = 0.0f;
-                if (s < K && !self[v]) pv = expf(-beta * d[v]);
+                if (s < K && !self[v]) pv = det_expf(-beta * d[v]);
                 p[v] = pv;
-                ls += pv;
-                if (s < K) le += entropy_term(pv);
+                et[v] = s < K ? entropy_term(pv) : 0.0f;
             }
-            sum = group_sum<LANES>(ls);
-            const float ent = group_sum<LANES>(le);
-            const float H = (-ent / sum) + logf(sum);
+            sum = ordered_row_sum<LANES, VPL>(p);
+            const float ent = ordered_row_sum<LANES, VPL>(et);
+            const float H = (-ent / sum) + det_logf(sum);
             const float diff = H - log_target;
             const bool found = (diff < eps && -diff < eps);
             if (found || it == 199) {
@@ -122,13 +155,13 @@ __global__ __launch_bounds__(256) void perplexity_generic_kernel(const float *__
         float ls = 0.0f, le = 0.0f;
         for (int s = lane; s < K; s += kWave) {
             const float dv = sq_dist[base + s];
-            const float pv = (s == 0 && dv == 0.0f) ? 0.0f : expf(-beta * dv);
+            const float pv = (s == 0 && dv == 0.0f) ? 0.0f : det_expf(-beta * dv);
             ls += pv;
             le += entropy_term(pv);
         }
         sum = group_sum<kWave>(ls);
         const float ent = group_sum<kWave>(le);
-        const float H = (-ent / sum) + logf(sum);
+        const float H = (-ent / sum) + det_logf(sum);
         const float diff = H - log_target;
         const bool found = (diff < eps && -diff < eps);
         if (found || it == 199) break;
@@ -142,7 +175,7 @@ __global__ __launch_bounds__(256) void perplexity_generic_kernel(const float *__
     }
     for (int s = lane; s < K; s += kWave) {
         const float dv = sq_dist[base + s];
-        const float pv = (s == 0 && dv == 0.0f) ? 0.0f : expf(-beta * dv);
+        const float pv = (s == 0 && dv == 0.0f) ? 0.0f : det_expf(-beta * dv);
         pij[base + s] = pv / sum;
     }
     if (betas && lane == 0) betas[row] = beta;
@@ -164,7 +197,7 @@ int launch_max_normalize(float *values, int64_t n, float *scratch, hipStream_t s
 
 int launch_perplexity(const float *sq_dist, int N, int K, float perplexity, float eps, float *pij, float *betas,
                       hipStream_t s) {
-    const float log_target = logf(perplexity);
+    const float log_target = det_logf(perplexity);
 #define TSNE_PERP(LANES, VPL)                                                                                  \
     perplexity_kernel<LANES, VPL><<<div_up(N, 256 / LANES), 256, 0, s>>>(sq_dist, N, K, log_target, eps, pij, \
                                                                          betas)
