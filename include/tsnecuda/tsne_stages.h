@@ -85,6 +85,18 @@ double tsne_hip_last_kl_divergence(void);
  * Replaces tsnecuda::util::MaxNormalizeDeviceVector (src/util/math_utils.cu:66-74). */
 int tsne_hip_max_normalize(float *values, int64_t n, void *stream);
 
+/* tsne_hip_max_normalize for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  The reduction scalar lives in a 256-byte
+ * array that is part of the library's device image (one copy per GPU, held until
+ * the process ends) instead of a per-call allocation: the call allocates and
+ * frees nothing, is asynchronous on `stream` (it does not synchronise), and
+ * records kernels only.  n may be at most 2^32 values; larger inputs are
+ * rejected with an error.  All calls on one GPU share that GPU's array: calls
+ * that overlap on one GPU (different streams or host threads) race and must be
+ * serialised by the caller.  The result is bit-identical to tsne_hip_max_normalize. */
+int tsne_hip_max_normalize_noalloc(float *values, int64_t n, void *stream);
+
 /* Per-row search for the Gaussian precision that gives the requested
  * perplexity; writes row-normalised conditional probabilities.
  * Replaces tsnecuda::SearchPerplexity (src/kernels/perplexity_search.cu:81-141,
@@ -113,7 +125,10 @@ void tsne_hip_plan_destroy(tsne_hip_plan *plan);
  * memory; pij and indices are not referenced after the call has completed on
  * the stream.  Afterwards tsne_hip_attractive and tsne_hip_iterate accept
  * pij = indices = NULL and use the re-blocked copy.  Has no counterpart in the
- * reference (its P matrix stays in N x K order, src/fit_tsne.cu:153). */
+ * reference (its P matrix stays in N x K order, src/fit_tsne.cu:153).
+ * Returns 2 (with tsne_hip_last_error) when the blocked format cannot hold the
+ * problem - more than 16,777,216 points or num_neighbors >= 4096 - in which case
+ * the plan keeps working with an explicit (pij, indices); 1 for any other failure. */
 int tsne_hip_attractive_prepare(tsne_hip_plan *plan, const float *pij, const int *indices, void *stream);
 
 /* attr_i = sum_s P[i,s] (y_i - y_j) / (1 + |y_i - y_j|^2), j = idx[i,s].

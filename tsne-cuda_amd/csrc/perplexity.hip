@@ -25,6 +25,14 @@
 
 #include <algorithm>
 #include <cfloat>
+#include <mutex>
+
+#include "../../include/tsnecuda/tsne_stages.h"
+
+// Scratch of tsne_hip_max_normalize_noalloc: the device scalar that receives the largest absolute value.
+// Every GPU holds its own copy of this array at its own address until the process ends; in host code the
+// name is only a handle for hipGetSymbolAddress, never a device address.
+static __device__ __align__(256) float scratch[64];
 
 namespace tsnehip {
 
@@ -195,6 +203,35 @@ int launch_max_normalize(float *values, int64_t n, float *scratch, hipStream_t s
     return 0;
 }
 
+namespace {
+constexpr int kMaxDevices = 64;
+constexpr int64_t kNoAllocMaxValues = (int64_t)1 << 32;
+std::mutex g_scratch_mutex;
+float *g_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+// The address of `scratch` on the current device, looked up once per device.
+int noalloc_scratch(float **out) {
+    int dev = -1;
+    TSNE_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) {
+        set_error("max_normalize_noalloc: device %d is outside the supported range [0, %d)", dev, kMaxDevices);
+        return 1;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        float *ptr = nullptr;
+        TSNE_TRY(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) {
+            set_error("max_normalize_noalloc: hipGetSymbolAddress returned a null address");
+            return 1;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
 int launch_perplexity(const float *sq_dist, int N, int K, float perplexity, float eps, float *pij, float *betas,
                       hipStream_t s) {
     const float log_target = det_logf(perplexity);
@@ -224,3 +261,20 @@ int launch_perplexity(const float *sq_dist, int N, int K, float perplexity, floa
 }
 
 }  // namespace tsnehip
+
+extern "C" int tsne_hip_max_normalize_noalloc(float *values, int64_t n, void *stream) {
+    using namespace tsnehip;
+    if (!values || n <= 0) {
+        set_error("max_normalize_noalloc: need a non-empty array");
+        return 1;
+    }
+    if (n > kNoAllocMaxValues) {
+        set_error("max_normalize_noalloc: %lld values exceed the supported maximum of %lld", (long long)n,
+                  (long long)kNoAllocMaxValues);
+        return 1;
+    }
+    float *ptr = nullptr;
+    if (noalloc_scratch(&ptr)) return 1;
+    // launch_max_normalize clears the scalar with a kernel (no memset node, so the call may be captured).
+    return launch_max_normalize(values, n, ptr, (hipStream_t)stream);
+}

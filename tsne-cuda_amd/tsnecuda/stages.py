@@ -29,6 +29,8 @@ def lib():
         L.tsne_hip_locality_order.argtypes = [_vp, c_int, c_int, _vp, _vp]
         L.tsne_hip_gather_rows.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
         L.tsne_hip_max_normalize.argtypes = [_vp, c_i64, _vp]
+        L.tsne_hip_max_normalize_noalloc.argtypes = [_vp, c_i64, _vp]
+        L.tsne_hip_max_normalize_noalloc.restype = c_int
         L.tsne_hip_perplexity.argtypes = [_vp, c_int, c_int, c_float, c_float, _vp, _vp, _vp]
         L.tsne_hip_symmetrize.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
         L.tsne_hip_plan_create.argtypes = [ctypes.POINTER(_vp), c_int, c_int, c_int, c_int]
@@ -117,6 +119,13 @@ def gather_rows(rows, order):
 
 def max_normalize_(values):
     _check(lib().tsne_hip_max_normalize(_ptr(_f32(values)), values.numel(), _stream()))
+    return values
+
+
+def max_normalize_noalloc_(values, n=None):
+    """max_normalize_ through the entry point that allocates nothing (asynchronous;
+    calls on one GPU must not overlap).  n: number of leading values (default all)."""
+    _check(lib().tsne_hip_max_normalize_noalloc(_ptr(_f32(values)), values.numel() if n is None else n, _stream()))
     return values
 
 
