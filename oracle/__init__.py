@@ -51,10 +51,17 @@ def num_threads():
 
 
 def knn(X, K, rows=None):
-    """Exact kNN (self first).  rows=(begin, end) restricts the query rows."""
+    """Exact kNN (self first).  rows=(begin, end) restricts the query rows to a range;
+    rows=<int array> to the listed rows (outputs in that order)."""
     X = np.ascontiguousarray(X, np.float32)
     N, D = X.shape
     K = min(K, N)
+    if rows is not None and not isinstance(rows, tuple):
+        rows = np.ascontiguousarray(rows, np.int32)
+        idx = np.empty((rows.size, K), np.int32)
+        d2 = np.empty((rows.size, K), np.float32)
+        lib().oracle_knn_row_list(_opt(X), N, D, K, _opt(rows), int(rows.size), _opt(idx), _opt(d2))
+        return idx, d2
     b, e = (0, N) if rows is None else rows
     idx = np.empty((e - b, K), np.int32)
     d2 = np.empty((e - b, K), np.float32)
@@ -99,6 +106,14 @@ def row_sum(v):
     """Sum of a row in the search's stated order (64 interleaved partial sums, then a balanced tree)."""
     v = np.ascontiguousarray(v, np.float32).ravel()
     return float(lib().oracle_row_sum(_opt(v), int(v.size)))
+
+
+def init(n, kind, seed, std=False):
+    """Initial embedding (flat 2N) of the reference's random initialisations: kind 0 = UNIFORM(-5, 5),
+    1 = GAUSSIAN (1e-4 N(0,1) after 2N discarded draws).  std=True: through the std:: classes themselves."""
+    Y = np.empty(2 * n, np.float32)
+    (lib().oracle_init_std if std else lib().oracle_init)(int(n), int(kind), int(seed), _opt(Y))
+    return Y
 
 
 def symmetrize(p, idx):

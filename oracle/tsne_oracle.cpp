@@ -16,6 +16,7 @@
 //   oracle_repulsive      src/kernels/rep_forces.cu:3-92, src/kernels/nbodyfft.cu:3-442,
 //                         src/fit_tsne.cu:246-323,430-467
 //   oracle_update         src/kernels/apply_forces.cu:11-57
+//   oracle_init           src/fit_tsne.cu:184-204 (random initial embeddings)
 //   oracle_fit            src/fit_tsne.cu:84-624 (schedule, state, outputs)
 //   oracle_kl             build-defined evaluator (the reference never computes KL)
 //
@@ -30,6 +31,7 @@
 //   repulsive   direct node-to-node convolution on reduced grids, numpy FFT at
 //               full size, exact O(N^2) sums to interpolation accuracy
 //   update      hand-computed single-coordinate cases
+//   init        the std:: engine and distributions themselves (oracle_init_std), moments of the draws
 //   The reference's own tests hold no golden vectors for this path and its kNN
 //   lives in un-vendored FAISS (v1.9.0, approximate IVF): kNN parity against the
 //   reference's *values* is unpinned; it is pinned against the exact definition.
@@ -66,7 +68,8 @@ struct Cand {
 };
 inline bool cand_less(const Cand &a, const Cand &b) { return a.d < b.d || (a.d == b.d && a.j < b.j); }
 
-void knn_rows(const float *X, const float *Xt, int N, int D, int K, int row_begin, int row_end, int *idx,
+// Query rows rows[0 .. n_rows); output row r belongs to query rows[r].
+void knn_rows(const float *X, const float *Xt, int N, int D, int K, const int *rows, int n_rows, int *idx,
               float *d2) {
     const int JB = 2048;
 #pragma omp parallel
@@ -75,7 +78,8 @@ void knn_rows(const float *X, const float *Xt, int N, int D, int K, int row_begi
         std::vector<Cand> heap;
         heap.reserve(K);
 #pragma omp for schedule(dynamic, 4)
-        for (int i = row_begin; i < row_end; ++i) {
+        for (int r = 0; r < n_rows; ++r) {
+            const int i = rows[r];
             heap.clear();
             const int want = K - 1;
             const float *xi = X + (size_t)i * D;
@@ -106,8 +110,8 @@ void knn_rows(const float *X, const float *Xt, int N, int D, int K, int row_begi
                 }
             }
             std::sort(heap.begin(), heap.end(), cand_less);
-            int *oi = idx + (size_t)(i - row_begin) * K;
-            float *od = d2 + (size_t)(i - row_begin) * K;
+            int *oi = idx + (size_t)r * K;
+            float *od = d2 + (size_t)r * K;
             oi[0] = i;
             od[0] = 0.0f;
             for (int s = 1; s < K; ++s) {
@@ -249,11 +253,18 @@ int oracle_num_threads() {
 
 // Rows [row_begin, row_end) of the exact kNN of X (N x D row-major); outputs are
 // (row_end-row_begin) x K, row-major, int32 indices and fp32 squared distances.
-void oracle_knn_rows(const float *X, int N, int D, int K, int row_begin, int row_end, int *idx, float *d2) {
+void oracle_knn_row_list(const float *X, int N, int D, int K, const int *rows, int n_rows, int *idx, float *d2) {
     std::vector<float> Xt((size_t)N * D);
-    for (int i = 0; i < N; ++i)
-        for (int d = 0; d < D; ++d) Xt[(size_t)d * N + i] = X[(size_t)i * D + d];
-    knn_rows(X, Xt.data(), N, D, K, row_begin, row_end, idx, d2);
+#pragma omp parallel for schedule(static)
+    for (int d = 0; d < D; ++d)
+        for (int i = 0; i < N; ++i) Xt[(size_t)d * N + i] = X[(size_t)i * D + d];
+    knn_rows(X, Xt.data(), N, D, K, rows, n_rows, idx, d2);
+}
+
+void oracle_knn_rows(const float *X, int N, int D, int K, int row_begin, int row_end, int *idx, float *d2) {
+    std::vector<int> rows(row_end - row_begin);
+    for (int i = row_begin; i < row_end; ++i) rows[i - row_begin] = i;
+    oracle_knn_row_list(X, N, D, K, rows.data(), (int)rows.size(), idx, d2);
 }
 
 void oracle_knn(const float *X, int N, int D, int K, int *idx, float *d2) {
@@ -415,6 +426,96 @@ void oracle_perplexity(const float *d2, int N, int K, float perplexity, float ep
             if (beta_out) beta_out[i] = used_beta;
             if (iters_out) iters_out[i] = it;
         }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Initial embedding, src/fit_tsne.cu:184-204 (and src/util/random_utils.cu:17-35 for UNIFORM).
+// The reference draws from std::default_random_engine(opt.random_seed) with
+// std::normal_distribution<float>(0, 1): first 2N values that only feed an unused noise vector
+// (x 0.001), then, for GAUSSIAN, the next 2N values x 0.0001 (a double product stored as float), or,
+// for UNIFORM, 2N values of std::uniform_real_distribution<float>(-5, 5) from the same engine.
+//
+// oracle_init spells those std:: components out (libstdc++'s algorithms):
+//   engine        minstd_rand0, x <- 16807 x mod (2^31 - 1), seeded with (seed as uint64) mod (2^31 - 1) (1 if that is 0)
+//   canonical     one engine call per float: float(x - 1) / 2147483646.0f, clamped below 1
+//   normal        Marsaglia's polar method: u, v = 2 c - 1 (double subtraction, stored as float), retried
+//                 until 0 < r2 = u u + v v <= 1; m = sqrt(-2 ln r2 / r2); returns v m now and u m at the
+//                 next call
+//   uniform(a,b)  c (b - a) + a in float
+// oracle_init_std calls the std:: classes themselves; tests/test_oracle.py holds the two against each other.
+// kind: 0 = UNIFORM, 1 = GAUSSIAN (the TSNE_INIT encodings of src/include/options.h:37-42).
+// ---------------------------------------------------------------------------
+namespace {
+struct MinStd {
+    uint32_t x;
+    // The engine's seed type is a 64-bit unsigned integer here: an int seed is sign-extended on the way in.
+    explicit MinStd(int seed) {
+        x = (uint32_t)((uint64_t)(int64_t)seed % 2147483647u);
+        if (x == 0) x = 1;
+    }
+    uint32_t next() {
+        x = (uint32_t)(((uint64_t)x * 16807u) % 2147483647u);
+        return x;
+    }
+    float canonical() {
+        const float sum = (float)(next() - 1u) * 1.0f;
+        const float tmp = 1.0f * 2147483646.0f;  // engine range as a float (rounds to 2^31)
+        float ret = sum / tmp;
+        if (ret >= 1.0f) ret = std::nextafter(1.0f, 0.0f);
+        return ret;
+    }
+};
+struct PolarNormal {
+    bool saved_available = false;
+    float saved = 0.0f;
+    float draw(MinStd &g) {
+        float ret;
+        if (saved_available) {
+            saved_available = false;
+            ret = saved;
+        } else {
+            float u, v, r2;
+            do {
+                u = (float)(2.0f * g.canonical() - 1.0);
+                v = (float)(2.0f * g.canonical() - 1.0);
+                r2 = u * u + v * v;
+            } while (r2 > 1.0 || r2 == 0.0);
+            const float mult = std::sqrt(-2 * std::log(r2) / r2);
+            saved = u * mult;
+            saved_available = true;
+            ret = v * mult;
+        }
+        return ret * 1.0f + 0.0f;
+    }
+};
+}  // namespace
+
+void oracle_init(int N, int kind, int seed, float *Y) {
+    MinStd g(seed);
+    PolarNormal normal;
+    const size_t n2 = (size_t)2 * N;
+    for (size_t i = 0; i < n2; ++i) Y[i] = (float)(0.001 * normal.draw(g));  // the unused noise vector
+    if (kind == 0) {
+        for (size_t i = 0; i < n2; ++i) Y[i] = g.canonical() * (5.0f - (-5.0f)) + (-5.0f);
+    } else {
+        for (size_t i = 0; i < n2; ++i) Y[i] = (float)(0.0001 * normal.draw(g));
+    }
+}
+
+}  // extern "C"
+#include <random>
+extern "C" {
+void oracle_init_std(int N, int kind, int seed, float *Y) {
+    std::default_random_engine generator(seed);
+    std::normal_distribution<float> distribution1(0.0, 1.0);
+    const size_t n2 = (size_t)2 * N;
+    for (size_t i = 0; i < n2; ++i) Y[i] = 0.001 * distribution1(generator);
+    if (kind == 0) {
+        std::uniform_real_distribution<float> distribution(-5, 5);
+        for (size_t i = 0; i < n2; ++i) Y[i] = distribution(generator);
+    } else {
+        for (size_t i = 0; i < n2; ++i) Y[i] = 0.0001 * distribution1(generator);
     }
 }
 

@@ -106,6 +106,82 @@ def test_gaussian_init_and_snapshots(c0_problem):
     assert not np.array_equal(snaps[1], snaps[2])
 
 
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+@pytest.mark.parametrize("n,seed", [(300, 7), (20000, 1700000000)])
+def test_random_initialisations_follow_the_reference_draw_order(tmp_path, kind, n, seed):
+    """RunTsne with zero iterations returns its initial embedding.  With Options::random_seed
+    fixed (only the C++ surface can: tests/harness/options_harness.cpp) it must be, bit for bit,
+    what src/fit_tsne.cu:184-204 draws: 2N normals discarded, then 2N x 1e-4 (GAUSSIAN) or 2N
+    uniform values in [-5, 5) (UNIFORM) - also through the locality renumbering (20000 points)."""
+    import subprocess
+    exe = os.path.join(REPO, "tests", "harness", "options_harness")
+    assert os.path.exists(exe), "build the harness with `make -C tsne-cuda_amd`"
+    out = tmp_path / "init.bin"
+    run = subprocess.run([exe, str(n), "4", str(kind), str(seed), "0", str(out)], capture_output=True, text=True,
+                         timeout=120)
+    assert run.returncode == 0, run.stdout + run.stderr
+    got = np.fromfile(out, np.float32)
+    want = oracle.init(n, kind, seed)
+    assert got.shape == want.shape
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+_EXIT_SNIPPET = """
+import ctypes, sys
+import numpy as np
+lib = ctypes.CDLL(sys.argv[1])
+c_float, c_int, c_bool, vp = ctypes.c_float, ctypes.c_int, ctypes.c_bool, ctypes.c_void_p
+lib.pymodule_tsne.restype = None
+lib.pymodule_tsne.argtypes = [vp, vp, vp] + [c_float] * 4 + [c_int] * 4 + [c_float] * 6 + [c_int, vp, c_bool, vp,
+    c_int, c_bool, vp, c_int, c_int, c_int, c_int, c_int, c_int, c_int]
+init, preinit_null, style = int(sys.argv[2]), int(sys.argv[3]), int(sys.argv[4])
+X = np.random.default_rng(0).random((200, 5)).astype(np.float32)
+res = np.zeros((200, 2), np.float32, order="F")
+pre = np.zeros((200, 2), np.float32, order="F")
+dims = (ctypes.c_ssize_t * 2)(200, 5)
+empty = ctypes.create_string_buffer(b"")
+lib.pymodule_tsne(res.ctypes.data, X.ctypes.data, ctypes.cast(dims, vp), 10.0, 200.0, 12.0, 5.0, 30, 5, 1000, 250,
+                  1e-3, 0.5, 0.8, 0.5, 0.0025, 0.0, init, None if preinit_null else pre.ctypes.data, False,
+                  ctypes.cast(empty, vp), 1, False, ctypes.cast(empty, vp), 1000, 0, 10, 0, style, 2, 1)
+print("returned")
+"""
+
+
+@pytest.mark.parametrize("init,preinit_null,style,message", [
+    (2, 0, 0, "E: RESUME initialization not yet supported fully..."),  # src/ext/pymodule_ext.cu:78-81
+    (7, 0, 0, "E: Invalid initialization supplied"),                   # :86-88
+    (3, 1, 0, "E: Invalid initialization. Initialization points are null."),  # src/fit_tsne.cu:218-222
+    (1, 0, 5, "E: Invalid return style supplied"),                     # src/ext/pymodule_ext.cu:114-115
+])
+def test_pymodule_exits_with_the_reference_messages(tmp_path, init, preinit_null, style, message):
+    """The shim has no status to return: invalid encodings print the reference's message and
+    exit(1), which only a child process can observe."""
+    import subprocess
+    import sys
+    script = tmp_path / "call.py"
+    script.write_text(_EXIT_SNIPPET)
+    lib = os.path.join(REPO, "tsne-cuda_amd", "tsnecuda", "libtsnecuda.so")
+    run = subprocess.run([sys.executable, str(script), lib, str(init), str(preinit_null), str(style)],
+                         capture_output=True, text=True, timeout=120)
+    assert run.returncode == 1, (run.returncode, run.stdout, run.stderr)
+    assert message in run.stderr
+    assert "returned" not in run.stdout
+
+
+def test_pymodule_child_process_runs_a_valid_call(tmp_path):
+    """The same child-process call with valid encodings returns (so the exits above are the shim's)."""
+    import subprocess
+    import sys
+    script = tmp_path / "call.py"
+    script.write_text(_EXIT_SNIPPET)
+    lib = os.path.join(REPO, "tsne-cuda_amd", "tsnecuda", "libtsnecuda.so")
+    run = subprocess.run([sys.executable, str(script), lib, "1", "0", "0"], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0 and "returned" in run.stdout, run.stderr
+
+
 def test_dump_file_format(tmp_path, c0_problem):
     """Text dump: header "N 2" then N lines "x y" per dumped step
     (src/fit_tsne.cu:347-352,563-570)."""
