@@ -24,6 +24,32 @@ for _p in (ROOT, os.path.join(ROOT, "tsne-cuda_amd")):
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 
+def traffic_from_profile(path):
+    """HBM bytes per launch of the attractive kernel from the committed rocprofv3 summary: the per-kernel
+    averages of its FETCH_SIZE and WRITE_SIZE passes, each scaled by what the same counter read for the plain
+    256 MiB device copy of the same run (262144 KiB read and written per launch)."""
+    if not os.path.exists(path):
+        return None, None
+    avg, copy_max = {}, {}
+    for line in open(path):
+        f = line.split()
+        if len(f) < 5 or f[-4] not in ("FETCH_SIZE", "WRITE_SIZE"):
+            continue
+        try:
+            a, m = float(f[-2]), float(f[-1])
+        except ValueError:
+            continue
+        if f[0].startswith("attractive_blocked_kernel"):
+            avg[f[-4]] = a
+        elif f[0] == "__amd_rocclr_copyBuffer":
+            copy_max[f[-4]] = m
+    if set(avg) != {"FETCH_SIZE", "WRITE_SIZE"} or set(copy_max) != {"FETCH_SIZE", "WRITE_SIZE"}:
+        return None, None
+    kib = 262144.0  # one calibration copy
+    total = sum(avg[c] * (kib / copy_max[c]) * 1024.0 for c in avg)
+    return total, "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes over this command, profiles/" + os.path.basename(path)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -36,7 +62,12 @@ def main():
     ap.add_argument("--no-overlap", action="store_true",
                     help="run the repulsive chain and the attractive kernel one after the other (TSNE_OVERLAP=0): "
                          "per-kernel durations in a trace then are those of kernels running alone")
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="times the stretch of --steps steps is timed (each bracketed by a device synchronisation "
+                         "on both sides); the median is reported")
     ap.add_argument("--fit-repeats", type=int, default=3, help="end-to-end fits timed (the median is reported)")
+    ap.add_argument("--no-small", action="store_true",
+                    help="skip the end-to-end fits of the smaller configurations (c0, c1, c2) and the CPU fit of c0")
     ap.add_argument("--cpu-steps", type=int, default=150, help="gradient steps of the CPU baseline sample")
     ap.add_argument("--cpu-knn-rows", type=int, default=4096, help="query rows of the CPU baseline's kNN sample")
     ap.add_argument("--calibrate", action="store_true",
@@ -95,7 +126,13 @@ def main():
     gains, old = torch.ones_like(y), torch.zeros_like(y)
     eta = fit["learning_rate"]
     _, warm_s = timed(lambda: plan.iterate_(None, None, y, gains, old, 0, args.warmup, eta=eta))
-    z, loop_s = timed(lambda: plan.iterate_(None, None, y, gains, old, args.warmup, args.warmup + args.steps, eta=eta))
+    # EXACTLY --steps steps per timed stretch, consecutive stretches of the same fit; the median stretch is reported.
+    loop_runs, done = [], args.warmup
+    for _ in range(max(1, args.repeats)):
+        z, run_s = timed(lambda: plan.iterate_(None, None, y, gains, old, done, done + args.steps, eta=eta))
+        loop_runs.append(run_s)
+        done += args.steps
+    loop_s = sorted(loop_runs)[len(loop_runs) // 2]
     ms_per_step = loop_s * 1e3 / args.steps
     iters_per_s = args.steps / loop_s
 
@@ -103,8 +140,7 @@ def main():
     # the library around every kernel of a further stretch of the same loop ----
     prof_steps = min(args.steps, 200)
     plan.profile_begin()
-    plan.iterate_(None, None, y, gains, old, args.warmup + args.steps, args.warmup + args.steps + prof_steps,
-                  eta=eta)
+    plan.iterate_(None, None, y, gains, old, done, done + prof_steps, eta=eta)
     prof = plan.profile_end()
     kernels_us = {name: 1e3 * ms / max(cnt, 1) for name, (ms, cnt) in prof.items()}
     attr_ms = kernels_us["attractive_kernel"] * 1e-3  # profiling slot of whichever attractive kernel ran
@@ -190,10 +226,39 @@ def main():
         with open(gold_path) as f:
             oracle_kl = json.load(f).get("kl_exact_z")
 
-    # HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes whose
-    # summary sits in profiles/bench_c3_1M_hbm_counters.txt (395672 x 2 KiB fetched + 7826 x 1 KiB written);
-    # the counters belong to that exact workload, so other sizes report null.
-    traffic = 818.4e6 if (args.workload == "c3" and n == 1000000 and k == 90) else None
+    # HBM bytes per launch of the dominant kernel: not measurable from inside this process (it takes two
+    # rocprofv3 counter passes), so it is read from the committed summary of those passes over this same
+    # command; the counters belong to that exact workload, so other sizes - or a missing summary - report null.
+    traffic, traffic_source = None, None
+    if args.workload == "c3" and n == 1000000 and k == 90:
+        traffic, traffic_source = traffic_from_profile(os.path.join(ROOT, "profiles", "bench_c3_1M_hbm_counters.txt"))
+
+    # ---- the smaller configurations end to end, and c0 in full on the CPU ----
+    small = None
+    if not args.no_small and args.points is None:
+        small = {}
+        for name in ("c0", "c1", "c2"):
+            Xc, fc = synthetic.make_config(name)
+            Yc = synthetic.initial_embedding(Xc.shape[0])
+            mc = TSNE(perplexity=fc["perplexity"], num_neighbors=fc["num_neighbors"], learning_rate=fc["learning_rate"],
+                      n_iter=1000, perplexity_epsilon=1e-4)
+            runs = []
+            for _ in range(3):
+                a = time.perf_counter()
+                mc.fit_transform(Xc, y=Yc)
+                runs.append(time.perf_counter() - a)
+            small[name] = {"shape": "%d x %d" % Xc.shape, "gpu_fit_seconds": sorted(runs)[1],
+                           "kl_divergence": mc.kl_divergence_}
+            if name == "c0" and not args.no_cpu:
+                # The configuration the reference's CPU path is quoted on, run in full on the host cores.
+                import oracle
+                yc = np.concatenate([Yc[:, 0], Yc[:, 1]])
+                a = time.perf_counter()
+                _, _, idx_c, P_c = oracle.fit(Xc, yc, fc["num_neighbors"], fc["perplexity"], eps=1e-4, iterations=1000,
+                                              eta=fc["learning_rate"])
+                small[name]["cpu_fit_seconds"] = time.perf_counter() - a
+                small[name]["cpu_cores"] = oracle.num_threads()
+            del Xc
     out = {
         "metric": "gradient_iters_per_sec",
         "value": iters_per_s,
@@ -209,8 +274,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": "%s: %d x %d fp32, perplexity %g, K=%d, lr %g; step = one gradient iteration"
                                % (args.workload, n, d, fit["perplexity"], k, eta)},
+        "loop_seconds_runs": loop_runs,
         "fit_seconds": fit_s,
         "fit_seconds_runs": fit_runs,
+        "smaller_configs": small,
         "fit_kl_divergence": kl_final,
         "fit_kl_divergence_oracle": oracle_kl,
         "phases_s": {"locality_order": order_s + gather_s, "knn": knn_s, "max_normalize": norm_s, "perplexity": perp_s, "symmetrize": sym_s,
@@ -218,7 +285,7 @@ def main():
                      "gradient_loop_%d_steps" % args.steps: loop_s, "data_generation_host": gen_s},
         "roofline": {"bound": "hbm", "kernel": "attractive_blocked_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "bytes_per_launch": attr_bytes, "ms_per_launch": attr_ms},
+                     "traffic_source": traffic_source, "bytes_per_launch": attr_bytes, "ms_per_launch": attr_ms},
         "kernels_us": kernels_us,
         "phase_rooflines": phase_rooflines,
         "cpu_baseline": cpu,
