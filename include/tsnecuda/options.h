@@ -91,6 +91,10 @@ class Options {
 
     int random_seed = 0;
 
+    // Not in the reference: subtract the embedding's centre in every update (its loop never re-centres,
+    // src/kernels/apply_forces.cu:11-57).  Off by default; TSNE_RECENTER=1 in the environment also enables it.
+    bool recenter_embedding = false;
+
     Options() {}
 
     Options(float *return_data, float *points, int num_points, int num_dims)

@@ -165,6 +165,14 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
                      float pre_exaggeration_momentum, float post_exaggeration_momentum,
                      float early_exaggeration, float *normalization, void *stream);
 
+/* Optional re-centring of the embedding inside tsne_hip_iterate (off by default; the
+ * reference's loop never re-centres, src/kernels/apply_forces.cu:11-57, its CPU
+ * ancestor FIt-SNE does after every step).  When enabled, every update subtracts
+ * the centre (mean x, mean y) the embedding had before the step, fused into the
+ * update kernel: the forces are translation invariant, so this is re-centring after
+ * every step, applied one step late and without a pass of its own. */
+int tsne_hip_plan_set_recenter(tsne_hip_plan *plan, int enable);
+
 /* Whether a kernel of this plan has reported trouble since the last call (no
  * counterpart in the reference).  Call it after synchronising the streams the
  * plan was used on.  The one condition reported today: waves of the re-blocked
@@ -173,6 +181,32 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
  * nothing was reported, 1 (with tsne_hip_last_error) otherwise; clears the
  * report. */
 int tsne_hip_plan_check(tsne_hip_plan *plan);
+
+/* How far the interpolated repulsive forces of `embedding` (device, 2N floats) are from
+ * exact sums over all points, on sample_count pseudo-randomly chosen points (all of them if
+ * sample_count >= num_points).  result (host, three doubles): [0] relative L2 error of
+ * the sampled forces F_i = sum_j (y_i - y_j) / (1 + |y_i - y_j|^2)^2, [1] relative error
+ * of the sampled part of the normalisation sum_i sum_{j != i} 1 / (1 + |y_i - y_j|^2),
+ * [2] the number of points sampled.  The scheme's own error (three nodes per box, 130
+ * boxes: src/fit_tsne.cu:246-272) is what shows, typically 1e-3 to 1e-2.  No counterpart
+ * in the reference.  Allocates its work buffers and synchronises the stream.  RunTsne
+ * prints the same measure on its progress steps when TSNE_REPULSION_MONITOR=<points> is
+ * set in the environment. */
+int tsne_hip_repulsive_error(tsne_hip_plan *plan, const float *embedding, int sample_count, double *result,
+                             void *stream);
+
+/* Trustworthiness (Venna & Kaski) of an embedding: how far the n_neighbors nearest
+ * points of every point in the embedding are from being its nearest points in the input
+ * space; 1 is best.  HOST pointers: points num_points x num_dims row-major, embedding
+ * 2 * num_points floats (xs then ys, i.e. a Fortran-ordered (num_points, 2) array).
+ * Evaluated on the points themselves up to max_sample (<= 8192) of them, beyond that on a
+ * fixed pseudo-random sample of max_sample points (neighbourhoods and ranks taken inside
+ * the sample - the definition applied to the sampled points and their embedding);
+ * sample_out (may be NULL, room for max_sample ints) receives the sampled indices,
+ * ascending.  Squared L2 distances in both spaces, ties broken by lower index.  No
+ * counterpart in the reference, which reports no quality measure.  Synchronous. */
+int tsnecuda_trustworthiness(const float *points, const float *embedding, int num_points, int num_dims,
+                             int n_neighbors, int max_sample, int device, double *trustworthiness, int *sample_out);
 
 /* Squared L2 norm of n device floats into the device scalar *out
  * (tsnecuda::util::L2NormDeviceVector without the root, src/util/math_utils.cu:51-57). */

@@ -167,9 +167,10 @@ def update(Y, attr, rep, gains, old_forces, eta, normalization, momentum, exagge
 
 
 def iterate(P, idx, Y, steps, step_begin=0, force_magnify_iters=250, eta=200.0, pre_momentum=0.5,
-            post_momentum=0.8, early_exaggeration=12.0, gains=None, old_forces=None, nb=130, p=3):
+            post_momentum=0.8, early_exaggeration=12.0, gains=None, old_forces=None, nb=130, p=3, recenter=False):
     """Runs gradient steps [step_begin, step_begin+steps).  Returns (Y, Z) and
-    updates gains / old_forces in place when given."""
+    updates gains / old_forces in place when given.  recenter: the library's optional
+    re-centring (every step subtracts the centre the embedding had before the step)."""
     P = np.ascontiguousarray(P, np.float32)
     idx = np.ascontiguousarray(idx, np.int32)
     Y = np.array(Y, np.float32, copy=True).ravel()
@@ -177,7 +178,7 @@ def iterate(P, idx, Y, steps, step_begin=0, force_magnify_iters=250, eta=200.0, 
     Z = lib().oracle_iterate(_opt(P), _opt(idx), _opt(Y), _opt(gains), _opt(old_forces), N, K, step_begin,
                              step_begin + steps, force_magnify_iters, ctypes.c_float(eta),
                              ctypes.c_float(pre_momentum), ctypes.c_float(post_momentum),
-                             ctypes.c_float(early_exaggeration), nb, p)
+                             ctypes.c_float(early_exaggeration), nb, p, 1 if recenter else 0)
     return Y, float(Z)
 
 

@@ -694,9 +694,11 @@ void oracle_update(float *Y, float *attr, float *rep, float *gains, float *old_f
 // Gradient loop of src/fit_tsne.cu:402-580 on a fixed (P, idx) and a given
 // initial embedding (VECTOR init).  Y is updated in place.  Returns the last Z.
 // gains and old_forces may be null (fresh state: gains 1, momentum buffer 0).
+// recenter (not in the reference, whose loop never re-centres; the library's option): every step subtracts
+// from the new positions the centre (mean x, mean y) the embedding had before the step.
 float oracle_iterate(const float *P, const int *idx, float *Y, float *gains, float *old_forces, int N, int K,
                      int step_begin, int step_end, int force_magnify_iters, float eta, float pre_momentum,
-                     float post_momentum, float early_exaggeration, int nb, int p) {
+                     float post_momentum, float early_exaggeration, int nb, int p, int recenter) {
     std::vector<float> attr((size_t)2 * N, 0.0f), rep((size_t)2 * N, 0.0f);
     std::vector<float> g_local, u_local;
     if (!gains) {
@@ -712,9 +714,23 @@ float oracle_iterate(const float *P, const int *idx, float *Y, float *gains, flo
         const bool late = step >= force_magnify_iters;
         const float momentum = late ? post_momentum : pre_momentum;
         const float exag = late ? 1.0f : early_exaggeration;
+        double cx = 0.0, cy = 0.0;
+        if (recenter) {
+            for (int i = 0; i < N; ++i) {
+                cx += Y[i];
+                cy += Y[N + i];
+            }
+        }
         oracle_repulsive(Y, N, nb, p, rep.data(), &Z, nullptr, nullptr, nullptr, 0);
         oracle_attractive(P, idx, Y, N, K, attr.data());
         oracle_update(Y, attr.data(), rep.data(), gains, old_forces, N, eta, Z, momentum, exag);
+        if (recenter) {
+            const float mx = (float)(cx / N), my = (float)(cy / N);
+            for (int i = 0; i < N; ++i) {
+                Y[i] = Y[i] - mx;
+                Y[N + i] = Y[N + i] - my;
+            }
+        }
     }
     return Z;
 }
@@ -734,7 +750,7 @@ float oracle_fit(const float *X, int N, int D, int num_neighbors, float perplexi
     if (idx_out) std::memcpy(idx_out, idx.data(), idx.size() * sizeof(int));
     if (P_out) std::memcpy(P_out, P.data(), P.size() * sizeof(float));
     return oracle_iterate(P.data(), idx.data(), Y, nullptr, nullptr, N, K, 0, iterations, force_magnify_iters, eta,
-                          pre_momentum, post_momentum, early_exaggeration, 130, 3);
+                          pre_momentum, post_momentum, early_exaggeration, 130, 3, 0);
 }
 
 // KL-style objective on the stored pattern:

@@ -182,6 +182,46 @@ def test_pymodule_child_process_runs_a_valid_call(tmp_path):
     assert run.returncode == 0 and "returned" in run.stdout, run.stderr
 
 
+def test_trustworthiness_output_against_sklearn(c0_problem):
+    """TSNE.trustworthiness() after a fit: the library's own evaluation against scikit-learn's
+    (an independent implementation) - on all points where they fit the sample, and on the
+    sample the library reports otherwise."""
+    from sklearn.manifold import trustworthiness
+    from tsnecuda import TSNE
+    X = c0_problem["X"][:3000]
+    model = TSNE(perplexity=20.0, num_neighbors=60, n_iter=300, perplexity_epsilon=1e-4)
+    emb = model.fit_transform(X)
+    for k in (5, 12, 30):
+        got = model.trustworthiness(n_neighbors=k)
+        assert got == model.trustworthiness_
+        assert abs(got - trustworthiness(X, emb, n_neighbors=k)) <= 1e-6
+    assert np.array_equal(model.trust_sample_, np.arange(3000))
+    # a sample of 1000 of the 3000 points: the definition applied to those points and their embedding
+    got = model.trustworthiness(n_neighbors=12, max_sample=1000)
+    sub = model.trust_sample_
+    assert sub.shape == (1000,) and np.all(np.diff(sub) > 0) and sub.max() < 3000
+    assert abs(got - trustworthiness(X[sub], emb[sub], n_neighbors=12)) <= 1e-6
+    # a shuffled embedding is not trustworthy
+    model.embedding = np.asfortranarray(emb[np.random.default_rng(0).permutation(3000)])
+    assert model.trustworthiness(n_neighbors=12) < got - 0.2
+    with pytest.raises(RuntimeError, match="n_neighbors must be"):
+        model.trustworthiness(n_neighbors=600, max_sample=1000)
+    with pytest.raises(RuntimeError, match="needs a fit"):
+        TSNE().trustworthiness()
+
+
+def test_repulsion_monitor_lines(c0_problem, capfd, monkeypatch):
+    from tsnecuda import TSNE
+    monkeypatch.setenv("TSNE_REPULSION_MONITOR", "300")
+    TSNE(perplexity=10.0, num_neighbors=30, n_iter=40, verbose=1, print_interval=20,
+         perplexity_epsilon=1e-4).fit_transform(c0_problem["X"][:1500])
+    out = capfd.readouterr().out
+    lines = [l for l in out.split("\n") if "Repulsion interpolation error" in l]
+    assert len(lines) == 2 and lines[0].startswith("[Step 0]") and "(300 points)" in lines[0]
+    err = float(lines[1].split("forces ")[1].split(",")[0])
+    assert 0.0 < err < 0.1
+
+
 def test_dump_file_format(tmp_path, c0_problem):
     """Text dump: header "N 2" then N lines "x y" per dumped step
     (src/fit_tsne.cu:347-352,563-570)."""

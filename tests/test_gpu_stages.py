@@ -166,6 +166,42 @@ def test_iterate_short(stages, c0_problem, start, steps):
     plan.close()
 
 
+@pytest.mark.parametrize("prepared", [False, True])
+def test_iterate_with_recentring(stages, c0_problem, prepared):
+    """The optional re-centring (not in the reference): every update subtracts the centre the
+    embedding had before the step.  Against the oracle's loop with the same rule, from a start
+    that sits far off the origin; the centre then stays at the size of one step's mean movement,
+    and without the option the offset start just stays where it is."""
+    c = c0_problem
+    n = c["X"].shape[0]
+    y0 = c["y0"].copy()
+    y0[:n] += np.float32(3e-3)
+    y0[n:] -= np.float32(2e-3)
+    y_o, z_o = oracle.iterate(c["P"], c["idx"], y0, 6, recenter=True)
+    plan = stages.Plan(n, c["K"])
+    plan.set_recenter(True)
+    dP, di = dev(c["P"]), dev(c["idx"])
+    if prepared:
+        plan.prepare_attractive(dP, di)
+    dy = dev(y0)
+    gains, old = torch.ones_like(dy), torch.zeros_like(dy)
+    z = plan.iterate_(None if prepared else dP, None if prepared else di, dy, gains, old, 0, 6)
+    y = dy.cpu().numpy()
+    assert rel_l2(y, y_o) <= 1e-4
+    assert abs(float(z.item()) - z_o) <= 1e-4 * abs(z_o)
+    extent = float(y.max() - y.min())
+    assert abs(y[:n].mean()) <= 1e-2 * extent and abs(y[n:].mean()) <= 1e-2 * extent
+    # the same start without the option keeps its offset (and follows the oracle's plain loop)
+    plan.set_recenter(False)
+    dy = dev(y0)
+    gains, old = torch.ones_like(dy), torch.zeros_like(dy)
+    plan.iterate_(None if prepared else dP, None if prepared else di, dy, gains, old, 0, 6)
+    y_plain, _ = oracle.iterate(c["P"], c["idx"], y0, 6)
+    assert rel_l2(dy.cpu().numpy(), y_plain) <= 1e-4
+    assert abs(float(dy[:n].mean()) - 3e-3) <= 3e-4
+    plan.close()
+
+
 @pytest.mark.parametrize("n,d,k,perp", [
     (2, 2, 2, 1.5),         # smallest problem: self plus one neighbour
     (50, 3, 50, 10.0),      # K == N, fewer points than one candidate tile
@@ -222,6 +258,32 @@ def test_knn_duplicates_and_ties(stages):
     idx, d2 = stages.knn(dev(X), 120)
     assert np.array_equal(idx.cpu().numpy(), idx_o)
     assert np.array_equal(d2.cpu().numpy(), d2_o)
+
+
+def test_repulsive_error_monitor(stages):
+    """tsne_hip_repulsive_error: the interpolated forces against exact O(N m) sums on sampled
+    points.  With every point sampled, its two figures must be what numpy finds for the forces
+    and potentials the stage itself returns; a sample gives a similar figure."""
+    rng = np.random.default_rng(21)
+    n = 2500
+    y = np.concatenate([rng.standard_normal(n) * 6.0, rng.standard_normal(n) * 4.0 + 1.0]).astype(np.float32)
+    plan = stages.Plan(n, 8)
+    rep, z, w, yt, phi = plan.repulsive(dev(y), details=True)
+    rep, phi = rep.cpu().numpy().astype(np.float64), phi.cpu().numpy().astype(np.float64)
+    x64, y64 = y[:n].astype(np.float64), y[n:].astype(np.float64)
+    dx, dy = x64[:, None] - x64[None, :], y64[:, None] - y64[None, :]
+    q = 1.0 / (1.0 + dx * dx + dy * dy)
+    exact = np.concatenate([(dx * q * q).sum(1), (dy * q * q).sum(1)])
+    z_exact = (q.sum(1) - 1.0).sum()
+    z_interp = ((1 + x64 ** 2 + y64 ** 2) * phi[:, 0] - 2 * (x64 * phi[:, 1] + y64 * phi[:, 2]) + phi[:, 3] - 1.0).sum()
+    f_err, z_err, m = plan.repulsive_error(dev(y), n)
+    assert m == n
+    assert abs(f_err - np.linalg.norm(rep - exact) / np.linalg.norm(exact)) <= 1e-6
+    assert abs(z_err - abs(z_interp - z_exact) / z_exact) <= 1e-6
+    assert 1e-6 < f_err < 5e-2 and z_err < 1e-2  # the scheme's own error: three nodes per box
+    f_s, z_s, m_s = plan.repulsive_error(dev(y), 400)
+    assert m_s == 400 and 0.2 * f_err < f_s < 5 * f_err
+    plan.close()
 
 
 @pytest.mark.parametrize("nb", [4, 7, 33])

@@ -433,6 +433,7 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
     // the update kernel keeps both current.
     int slot = 0;
     if (launch_bounds(plan, embedding, slot, s)) return 1;
+    if (plan->recenter && launch_centre_sums(plan, embedding, slot, s)) return 1;
     if (launch_pack_xy(plan, embedding, s)) return 1;
     // Schedule of src/fit_tsne.cu:416-420: two stretches of constant parameters; the step that reports the
     // normalisation runs by itself.
@@ -489,6 +490,18 @@ int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches) {
         launches[id] += 1;
     }
     plan->events_used = 0;
+    return 0;
+}
+
+int tsne_hip_plan_set_recenter(tsne_hip_plan *plan, int enable) {
+    if (check_plan(plan, "plan_set_recenter")) return 1;
+    // Captured steps carry the option as a kernel argument.
+    if ((enable != 0) != plan->recenter) {
+        TSNE_TRY(hipDeviceSynchronize());
+        for (auto &g : plan->step_graphs) (void)hipGraphExecDestroy(g.exec);
+        plan->step_graphs.clear();
+    }
+    plan->recenter = enable != 0;
     return 0;
 }
 

@@ -83,6 +83,9 @@ struct LoopScalars {
     // Workgroups of the re-blocked attractive kernel in which a wave gave up waiting for an LDS counter (their
     // rows come out as NaN).  Never non-zero unless the kernel's roles lose step; the host checks it after a loop.
     unsigned int wait_timeouts;
+    // Optional re-centring (off unless the plan asks for it): per bounds slot, the sums of the x and of the y
+    // coordinates of the embedding that slot's bounds describe.
+    double center_sum[2][2];
 };
 constexpr int kZParts = 16;
 

@@ -245,6 +245,8 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     const int n_boxes_per_dim = 130;  // 125 rounded up in the reference's allowed list
     tsne_hip_plan *plan = nullptr;
     TSNE_OR_DIE(tsne_hip_plan_create(&plan, N, K, n_boxes_per_dim, gpu_opt.device), "plan creation");
+    // Re-centring is this library's option (Options::recenter_embedding or TSNE_RECENTER=1); off, as in the reference.
+    plan->recenter = opt.recenter_embedding || env_int("TSNE_RECENTER", 0) != 0;
     // Re-block the sparse pattern for the LDS-staged attractive kernel; shapes it
     // cannot hold (very large K or N) keep the row-ordered kernel.
     // (The row-ordered pattern stays: the objective of the final embedding is evaluated on it.)
@@ -274,6 +276,7 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     const int print_interval = opt.print_interval > 0 ? opt.print_interval : 1;
     const bool want_snap = opt.return_style == RETURN_STYLE::SNAPSHOT && opt.return_data != nullptr;
     const bool want_stop = opt.min_gradient_norm > 0.0f;
+    const int monitor_points = verbose ? env_int("TSNE_REPULSION_MONITOR", 0) : 0;
     hipEvent_t ev[4];
     if (verbose)
         for (auto &e : ev) hip_or_die(hipEventCreate(&e), "event creation");
@@ -283,6 +286,7 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     int slot = 0;
     clock.start();
     TSNE_OR_DIE(tsnehip::launch_bounds(plan, d_emb.as<float>(), slot, stream), "bounds");
+    if (plan->recenter) TSNE_OR_DIE(tsnehip::launch_centre_sums(plan, d_emb.as<float>(), slot, stream), "centre");
     TSNE_OR_DIE(tsnehip::launch_pack_xy(plan, d_emb.as<float>(), stream), "pack");
     t_other += clock.stop();
     const size_t iterations = (size_t)opt.iterations;
@@ -370,6 +374,16 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
             break;
         }
         if (printing) std::cout << "[Step " << step << "] Avg. Gradient Norm: " << grad_norm << std::endl;
+        // TSNE_REPULSION_MONITOR=<points>: on the printed steps, the error of the interpolated repulsive forces
+        // of the embedding just produced against exact sums over all points, on that many sampled points.
+        if (printing && monitor_points > 0) {
+            double err[3] = {0.0, 0.0, 0.0};
+            TSNE_OR_DIE(tsnehip::repulsive_error(plan, d_emb.as<float>(), slot, monitor_points, 12345u + (unsigned)step,
+                                                 err, stream),
+                        "repulsion monitor");
+            std::cout << "[Step " << step << "] Repulsion interpolation error: forces " << err[0]
+                      << ", normalization " << err[1] << " (" << (int)err[2] << " points)" << std::endl;
+        }
 
         if (want_dump && step % dump_interval == 0) {
             hip_or_die(hipMemcpy(h_emb.data(), d_emb.ptr, sizeof(float) * h_emb.size(), hipMemcpyDeviceToHost),

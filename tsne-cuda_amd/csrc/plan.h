@@ -78,6 +78,7 @@ struct tsne_hip_plan {
     int strip_rows = 0, n_strips = 0, n_parts = 0, list_words = 0, seg_stride = 0;
     int spin_limit = 0;             // polls before a wave of the attractive kernel gives up a wait
     bool blocked_ready = false;
+    bool recenter = false;          // the loop's updates re-centre the embedding (tsne_hip_plan_set_recenter)
 
     // The repulsive chain and the attractive kernel of a step are independent: the fused loop runs
     // the chain on this side stream (default priority) and joins before the update.
@@ -149,6 +150,10 @@ void release_blocked(tsne_hip_plan *p);
 int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s);
 int check_attractive_waits(tsne_hip_plan *p);
 int launch_sum_squares(const float *values, int64_t n, float *out, hipStream_t s);
+int launch_centre_sums(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s);
+// Error of the interpolated repulsive forces against exact sums on a sample of the points (quality.hip).
+int repulsive_error(tsne_hip_plan *p, const float *embedding, int slot, int sample_count, unsigned int seed,
+                    double *result, hipStream_t s);
 int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, float *gains, float *old_forces,
                   float eta, const float *normalization, float momentum, float exaggeration, int next_slot,
                   hipStream_t s);

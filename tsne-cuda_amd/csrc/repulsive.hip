@@ -297,6 +297,8 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
         if (next_slot >= 0) {
             sc->min_enc[next_slot] = 0xffffffffu;
             sc->max_enc[next_slot] = 0u;
+            sc->center_sum[next_slot][0] = 0.0;
+            sc->center_sum[next_slot][1] = 0.0;
         }
     }
     for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;

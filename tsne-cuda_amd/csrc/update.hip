@@ -39,6 +39,52 @@ __device__ __forceinline__ float step_coordinate(float &gain, float &u, float at
     return u;
 }
 
+// Re-centring (optional, no counterpart in the reference, whose loop never re-centres:
+// src/kernels/apply_forces.cu:11-57): the update subtracts from every new position the centre of the embedding
+// as it stood before the step (its coordinate sums were accumulated by the update before, or by
+// centre_sums_kernel at the start of a loop) and accumulates the sums of what it writes.  All forces are
+// translation invariant, so the trajectory is that of exact re-centring after every step, one step late.
+// Without the option the centre reads as (+0, +0) and x - 0 is x, bit for bit.
+struct Centre {
+    float x, y;
+};
+template <bool FUSED>
+__device__ __forceinline__ Centre load_centre(const LoopScalars *sc, int next_slot, int N, int recenter) {
+    Centre c{0.0f, 0.0f};
+    if (FUSED && recenter) {
+        c.x = (float)(sc->center_sum[next_slot ^ 1][0] / (double)N);
+        c.y = (float)(sc->center_sum[next_slot ^ 1][1] / (double)N);
+    }
+    return c;
+}
+// A thread's sums of the x and y coordinates it wrote into the next slot's sums: one pair of atomics per wave.
+__device__ __forceinline__ void publish_centre(LoopScalars *sc, int next_slot, float sx, float sy) {
+    double dx = (double)sx, dy = (double)sy;
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) {
+        dx += __shfl_xor(dx, m, kWave);
+        dy += __shfl_xor(dy, m, kWave);
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        atomicAdd(&sc->center_sum[next_slot][0], dx);
+        atomicAdd(&sc->center_sum[next_slot][1], dy);
+    }
+}
+
+__global__ __launch_bounds__(256) void centre_sums_kernel(const float *__restrict__ emb, int N, LoopScalars *sc,
+                                                          int slot) {
+    float sx = 0.0f, sy = 0.0f;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
+        sx += emb[i];
+        sy += emb[N + i];
+    }
+    publish_centre(sc, slot, sx, sy);
+}
+
+__global__ void centre_reset_kernel(LoopScalars *sc, int slot) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) sc->center_sum[slot][0] = sc->center_sum[slot][1] = 0.0;
+}
+
 template <bool FUSED>
 __global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, float *__restrict__ attr,
                                                      float *__restrict__ rep, float *__restrict__ gains,
@@ -46,18 +92,22 @@ __global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, fl
                                                      const float *__restrict__ z_ptr, int z_count, float z_offset,
                                                      float momentum,
                                                      float exaggeration, float2 *__restrict__ yxy, LoopScalars *sc,
-                                                     int next_slot) {
+                                                     int next_slot, int recenter) {
     float z_total = 0.0f;
     for (int k = 0; k < z_count; ++k) z_total += z_ptr[k];  // same order in every thread
     const float normalization = z_total - z_offset;
     float lo = INFINITY, hi = -INFINITY;
+    const Centre c = load_centre<FUSED>(sc, next_slot, N, recenter);
+    float sx = 0.0f, sy = 0.0f;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
         float gx = gains[i], gy = gains[N + i];
         float ux = old[i], uy = old[N + i];
         step_coordinate(gx, ux, attr[i], rep[i], exaggeration, normalization, momentum, eta);
         step_coordinate(gy, uy, attr[N + i], rep[N + i], exaggeration, normalization, momentum, eta);
-        const float x = emb[i] + ux;
-        const float y = emb[N + i] + uy;
+        const float x = (emb[i] + ux) - c.x;
+        const float y = (emb[N + i] + uy) - c.y;
+        sx += x;
+        sy += y;
         emb[i] = x;
         emb[N + i] = y;
         attr[i] = 0.0f;
@@ -92,6 +142,7 @@ __global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, fl
             }
             publish_bounds(sc, next_slot, lo, hi);
         }
+        if (recenter) publish_centre(sc, next_slot, sx, sy);
     }
 }
 
@@ -104,11 +155,14 @@ __global__ __launch_bounds__(256) void update_vec4_kernel(float *__restrict__ em
                                                           const float *__restrict__ z_ptr, int z_count,
                                                           float z_offset,
                                                           float momentum, float exaggeration,
-                                                          float2 *__restrict__ yxy, LoopScalars *sc, int next_slot) {
+                                                          float2 *__restrict__ yxy, LoopScalars *sc, int next_slot,
+                                                          int recenter) {
     float z_total = 0.0f;
     for (int k = 0; k < z_count; ++k) z_total += z_ptr[k];  // same order in every thread
     const float normalization = z_total - z_offset;
     float lo = INFINITY, hi = -INFINITY;
+    const Centre c = load_centre<FUSED>(sc, next_slot, N, recenter);
+    float sx = 0.0f, sy = 0.0f;
     const int n4 = N / 4;
     float4 *emb4 = reinterpret_cast<float4 *>(emb), *attr4 = reinterpret_cast<float4 *>(attr);
     float4 *rep4 = reinterpret_cast<float4 *>(rep), *gains4 = reinterpret_cast<float4 *>(gains);
@@ -128,8 +182,10 @@ __global__ __launch_bounds__(256) void update_vec4_kernel(float *__restrict__ em
         step_coordinate(gy.y, uy.y, ay.y, ry.y, exaggeration, normalization, momentum, eta);
         step_coordinate(gy.z, uy.z, ay.z, ry.z, exaggeration, normalization, momentum, eta);
         step_coordinate(gy.w, uy.w, ay.w, ry.w, exaggeration, normalization, momentum, eta);
-        const float4 nx = make_float4(ex.x + ux.x, ex.y + ux.y, ex.z + ux.z, ex.w + ux.w);
-        const float4 ny = make_float4(ey.x + uy.x, ey.y + uy.y, ey.z + uy.z, ey.w + uy.w);
+        const float4 nx = make_float4((ex.x + ux.x) - c.x, (ex.y + ux.y) - c.x, (ex.z + ux.z) - c.x, (ex.w + ux.w) - c.x);
+        const float4 ny = make_float4((ey.x + uy.x) - c.y, (ey.y + uy.y) - c.y, (ey.z + uy.z) - c.y, (ey.w + uy.w) - c.y);
+        sx += (nx.x + nx.y) + (nx.z + nx.w);
+        sy += (ny.x + ny.y) + (ny.z + ny.w);
         emb4[i] = nx;
         emb4[n4 + i] = ny;
         // The reference clears the force arrays here (src/kernels/apply_forces.cu:48-51); the stage-level
@@ -169,6 +225,7 @@ __global__ __launch_bounds__(256) void update_vec4_kernel(float *__restrict__ em
             }
             publish_bounds(sc, next_slot, lo, hi);
         }
+        if (recenter) publish_centre(sc, next_slot, sx, sy);
     }
 }
 
@@ -212,10 +269,10 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
         if (next_slot >= 0) {
             update_vec4_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count,
                                                             z_offset, momentum, exaggeration, p->yxy, p->scalars,
-                                                            next_slot);
+                                                            next_slot, p->recenter ? 1 : 0);
         } else {
             update_vec4_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count,
-                                                             z_offset, momentum, exaggeration, nullptr, nullptr, 0);
+                                                             z_offset, momentum, exaggeration, nullptr, nullptr, 0, 0);
         }
         TSNE_LAUNCHED(s);
         return 0;
@@ -223,11 +280,21 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
     const int blocks = std::min(div_up(N, 256), 2048);
     if (next_slot >= 0) {
         update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count, z_offset,
-                                                   momentum, exaggeration, p->yxy, p->scalars, next_slot);
+                                                   momentum, exaggeration, p->yxy, p->scalars, next_slot, p->recenter ? 1 : 0);
     } else {
         update_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count, z_offset,
-                                                    momentum, exaggeration, nullptr, nullptr, 0);
+                                                    momentum, exaggeration, nullptr, nullptr, 0, 0);
     }
+    TSNE_LAUNCHED(s);
+    return 0;
+}
+
+// Coordinate sums of `embedding` into the centre sums of `slot` (start of a re-centred loop).
+int launch_centre_sums(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s) {
+    centre_reset_kernel<<<1, 64, 0, s>>>(p->scalars, slot);
+    TSNE_LAUNCHED(s);
+    const int blocks = std::min(div_up(p->num_points, 256 * 4), 1024);
+    centre_sums_kernel<<<std::max(blocks, 1), 256, 0, s>>>(embedding, p->num_points, p->scalars, slot);
     TSNE_LAUNCHED(s);
     return 0;
 }

@@ -188,3 +188,31 @@ class TSNE(object):
         else:
             self.embedding = result
         return self.embedding
+
+    def trustworthiness(self, n_neighbors=12, max_sample=4096):
+        """Trustworthiness of the last fit's embedding (1 is best): how far the
+        ``n_neighbors`` nearest points of every point in the embedding are from
+        being its nearest points in the input space (the measure scikit-learn's
+        ``sklearn.manifold.trustworthiness`` computes).  Evaluated on all points
+        up to ``max_sample`` (at most 8192) of them, beyond that on a fixed
+        pseudo-random sample, whose indices are left in ``trust_sample_``.  Also
+        stored as ``trustworthiness_``.  The reference has no such output."""
+        if not hasattr(self, "embedding") or not hasattr(self, "points"):
+            raise RuntimeError("trustworthiness() needs a fit: call fit_transform first")
+        emb = self.embedding[-1] if self.embedding.ndim == 3 else self.embedding
+        emb = np.require(emb, np.float32, ['F_CONTIGUOUS', 'ALIGNED'])
+        n, d = self.points.shape
+        out = ctypes.c_double(0.0)
+        sample = np.zeros(int(max_sample), np.int32)
+        fn = self._lib.tsnecuda_trustworthiness
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                       ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
+        rc = fn(self.points.ctypes.data, emb.ctypes.data, n, d, int(n_neighbors), int(max_sample), self.gpu_device,
+                ctypes.byref(out), sample.ctypes.data)
+        if rc != 0:
+            self._lib.tsne_hip_last_error.restype = ctypes.c_char_p
+            raise RuntimeError(self._lib.tsne_hip_last_error().decode())
+        self.trust_sample_ = sample[:min(n, int(max_sample))].copy()
+        self.trustworthiness_ = float(out.value)
+        return self.trustworthiness_

@@ -35,6 +35,8 @@ def lib():
         L.tsne_hip_symmetrize.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
         L.tsne_hip_plan_create.argtypes = [ctypes.POINTER(_vp), c_int, c_int, c_int, c_int]
         L.tsne_hip_plan_check.argtypes = [_vp]
+        L.tsne_hip_plan_set_recenter.argtypes = [_vp, c_int]
+        L.tsne_hip_plan_set_recenter.restype = c_int
         L.tsne_hip_plan_destroy.argtypes = [_vp]
         L.tsne_hip_plan_destroy.restype = None
         L.tsne_hip_attractive.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp]
@@ -45,6 +47,8 @@ def lib():
         L.tsne_hip_iterate.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, c_int, c_int, c_int, c_float, c_float,
                                        c_float, c_float, _vp, _vp]
         L.tsne_hip_sum_squares.argtypes = [_vp, _vp, c_i64, _vp, _vp]
+        L.tsne_hip_repulsive_error.argtypes = [_vp, _vp, c_int, ctypes.POINTER(ctypes.c_double), _vp]
+        L.tsne_hip_repulsive_error.restype = c_int
         L.tsne_hip_profile_kernel_name.argtypes = [c_int]
         L.tsne_hip_profile_kernel_name.restype = ctypes.c_char_p
         L.tsne_hip_profile_begin.argtypes = [_vp]
@@ -174,6 +178,10 @@ class Plan(object):
         torch.cuda.synchronize(self.device)
         _check(lib().tsne_hip_plan_check(self._h))
 
+    def set_recenter(self, enable):
+        """Optional re-centring inside iterate_ (off by default, as in the reference)."""
+        _check(lib().tsne_hip_plan_set_recenter(self._h, 1 if enable else 0))
+
     def prepare_attractive(self, pij, idx):
         """Re-blocks (pij, idx) into the plan; afterwards attractive() and
         iterate_() may be called with pij = idx = None."""
@@ -223,6 +231,13 @@ class Plan(object):
         cnt = (ctypes.c_int * n)()
         _check(lib().tsne_hip_profile_end(self._h, ms, cnt))
         return {lib().tsne_hip_profile_kernel_name(i).decode(): (ms[i], cnt[i]) for i in range(n)}
+
+    def repulsive_error(self, embedding, sample_count):
+        """(relative L2 error of the interpolated repulsive forces, relative error of the
+        normalisation terms, points sampled) against exact sums on sampled points."""
+        out = (ctypes.c_double * 3)()
+        _check(lib().tsne_hip_repulsive_error(self._h, _ptr(_f32(embedding)), sample_count, out, _stream()))
+        return float(out[0]), float(out[1]), int(out[2])
 
     def sum_squares(self, values):
         out = torch.empty(1, dtype=torch.float32, device=self.device)
