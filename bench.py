@@ -117,7 +117,10 @@ def main():
     _, norm_s = timed(lambda: stages.max_normalize_(d2))
     cond, perp_s = timed(lambda: stages.perplexity(d2, fit["perplexity"], 1e-4))
     P, sym_s = timed(lambda: stages.symmetrize(cond, idx))
-    del cond, d2
+    # (the optional full form, (A + A^T) / 2N with the union pattern as CSR: timed for its roofline row only)
+    (_, csr_col, _), sym_full_s = timed(lambda: stages.symmetrize_full(cond, idx))
+    nnz_sym = int(csr_col.numel())
+    del cond, d2, csr_col
 
     # ---- gradient loop ----------------------------------------------------
     plan = stages.Plan(n, k)
@@ -175,6 +178,14 @@ def main():
         phase_rooflines["knn"] = {"bound": "mfma", "flop": flop, "achieved": flop / knn_s / 1e12, "unit": "TFLOP/s",
                                   "frac": flop / knn_s / 1e12 / 157.3, "tile_pairs_per_mille": knn_stats[2],
                                   "note": "fp32 matrix peak; time of the whole kNN call (sweep, re-rank, packing)"}
+
+    # One-shot stages that are HBM problems (bytes as SURVEY-style algorithmic traffic).
+    nnz = float(n) * k
+    for name, secs, b in (("perplexity", perp_s, 8.0 * nnz), ("symmetrize", sym_s, 12.0 * nnz),
+                          ("symmetrize_full", sym_full_s, 8.0 * nnz + 8.0 * nnz_sym + 4.0 * (n + 1))):
+        phase_rooflines[name] = {"bound": "hbm", "bytes": b, "achieved": b / secs / 1e9, "unit": "GB/s",
+                                 "frac": b / secs / 1e9 / HBM_PEAK_GBS}
+    phase_rooflines["symmetrize_full"]["nnz"] = nnz_sym
 
     if args.calibrate:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda").normal_()
@@ -281,7 +292,7 @@ def main():
         "fit_kl_divergence": kl_final,
         "fit_kl_divergence_oracle": oracle_kl,
         "phases_s": {"locality_order": order_s + gather_s, "knn": knn_s, "max_normalize": norm_s, "perplexity": perp_s, "symmetrize": sym_s,
-                     "reblock_pattern": reblock_s,
+                     "symmetrize_full_csr": sym_full_s, "reblock_pattern": reblock_s,
                      "gradient_loop_%d_steps" % args.steps: loop_s, "data_generation_host": gen_s},
         "roofline": {"bound": "hbm", "kernel": "attractive_blocked_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,

@@ -95,6 +95,11 @@ class Options {
     // src/kernels/apply_forces.cu:11-57).  Off by default; TSNE_RECENTER=1 in the environment also enables it.
     bool recenter_embedding = false;
 
+    // Not in the reference's live code: symmetrise P as (A + A^T) / 2N with the union pattern (its commented-out
+    // cuSPARSE routine, src/util/math_utils.cu:76-225) instead of the pattern-restricted form it runs
+    // (src/util/math_utils.cu:269-308).  Off by default; TSNE_SYMMETRIZE=full in the environment also enables it.
+    bool full_symmetrization = false;
+
     Options() {}
 
     Options(float *return_data, float *points, int num_points, int num_dims)

@@ -111,6 +111,19 @@ int tsne_hip_perplexity(const float *sq_dist, int num_points, int num_neighbors,
 int tsne_hip_symmetrize(const float *pij_non_symmetric, const int *indices, int num_points,
                         int num_neighbors, float *pij, void *stream);
 
+/* Full symmetrisation P = (A + A^T) / 2N, A[i, idx[i,s]] = p[i,s], as a CSR matrix with
+ * the union pattern of A and A^T (nothing is dropped, so the entries sum to 1; rows have
+ * ascending columns).  This is what the reference holds as a commented-out cuSPARSE
+ * routine (src/util/math_utils.cu:76-225: sort, transpose, csrgeam with both factors
+ * 1/(2N)); the gradient loops of both the reference and RunTsne use the pattern-restricted
+ * tsne_hip_symmetrize by default (TSNE_SYMMETRIZE=full in the environment switches RunTsne
+ * to this one).  Built with a device radix sort of the (row, column, value) triples and
+ * a segmented reduce.  row_ptr: num_points + 1 ints; col_idx / values: room for
+ * 2 * num_points * num_neighbors entries; *nnz (host, may be NULL) receives the number of
+ * entries written.  Allocates its work buffers and synchronises the stream. */
+int tsne_hip_symmetrize_full(const float *pij_non_symmetric, const int *indices, int num_points, int num_neighbors,
+                             int *row_ptr, int *col_idx, float *values, int64_t *nnz, void *stream);
+
 /* Scratch memory and constants for the gradient loop of one problem size.
  * n_boxes_per_dim is 130 in the reference (src/fit_tsne.cu:246-272); other
  * values (2..170) exist for testing on reduced grids.  Stands in for the
@@ -136,6 +149,17 @@ int tsne_hip_attractive_prepare(tsne_hip_plan *plan, const float *pij, const int
  * pij = indices = NULL: use the pattern given to tsne_hip_attractive_prepare. */
 int tsne_hip_attractive(tsne_hip_plan *plan, const float *pij, const int *indices, const float *embedding,
                         float *attractive_forces, void *stream);
+
+/* Attractive forces over a CSR pattern (any sparse P, e.g. the one tsne_hip_symmetrize_full
+ * builds): attr_i = sum_{e in row i} values[e] (y_i - y_j) / (1 + |y_i - y_j|^2), j = col_idx[e].
+ * Same reference counterpart as tsne_hip_attractive. */
+int tsne_hip_attractive_csr(tsne_hip_plan *plan, const int *row_ptr, const int *col_idx, const float *values,
+                            const float *embedding, float *attractive_forces, void *stream);
+
+/* Makes tsne_hip_iterate (called with pij = indices = NULL) take its attractive forces from
+ * a CSR pattern; the three arrays are borrowed and must stay valid; three NULLs clear it.
+ * Synchronises the device. */
+int tsne_hip_plan_set_csr_pattern(tsne_hip_plan *plan, const int *row_ptr, const int *col_idx, const float *values);
 
 /* FFT-interpolated repulsive forces and the normalisation Z = sum_i z_i - N
  * (written to the device scalar *normalization).  Replaces, for one iteration,

@@ -38,6 +38,7 @@ def lib():
         L.oracle_fit.restype = ctypes.c_float
         L.oracle_kl.restype = ctypes.c_double
         L.oracle_row_sum.restype = ctypes.c_float
+        L.oracle_symmetrize_full.restype = ctypes.c_int64
         _lib = L
     return _lib
 
@@ -123,6 +124,30 @@ def symmetrize(p, idx):
     P = np.empty((N, K), np.float32)
     lib().oracle_symmetrize(_opt(p), _opt(idx), N, K, _opt(P))
     return P
+
+
+def symmetrize_full(p, idx):
+    """(A + A^T) / 2N with the union pattern as CSR (row_ptr, col_idx, values), columns ascending."""
+    p = np.ascontiguousarray(p, np.float32)
+    idx = np.ascontiguousarray(idx, np.int32)
+    N, K = p.shape
+    row_ptr = np.empty(N + 1, np.int32)
+    col = np.empty(2 * N * K, np.int32)
+    val = np.empty(2 * N * K, np.float32)
+    nnz = int(lib().oracle_symmetrize_full(_opt(p), _opt(idx), N, K, _opt(row_ptr), _opt(col), _opt(val)))
+    return row_ptr, col[:nnz].copy(), val[:nnz].copy()
+
+
+def attractive_csr(row_ptr, col_idx, values, Y):
+    """Attractive forces over a CSR pattern; Y flat 2N -> flat 2N."""
+    row_ptr = np.ascontiguousarray(row_ptr, np.int32)
+    col_idx = np.ascontiguousarray(col_idx, np.int32)
+    values = np.ascontiguousarray(values, np.float32)
+    Y = np.ascontiguousarray(Y, np.float32).ravel()
+    N = row_ptr.size - 1
+    out = np.empty(2 * N, np.float32)
+    lib().oracle_attractive_csr(_opt(row_ptr), _opt(col_idx), _opt(values), _opt(Y), N, _opt(out))
+    return out
 
 
 def attractive(P, idx, Y):

@@ -26,7 +26,8 @@
 //   perplexity  row sums, entropy target, uniform closed form, sklearn bisection;
 //               its exp / log against double-precision exp / log (<= 2 units in the last place),
 //               its row-sum order against an exact (fsum) sum
-//   symmetrize  dense (A + A^T)/2N masked to the pattern
+//   symmetrize  dense (A + A^T)/2N masked to the pattern; the full (CSR) form against the dense
+//               matrix and scipy.sparse
 //   attractive  dense O(N^2) sum
 //   repulsive   direct node-to-node convolution on reduced grids, numpy FFT at
 //               full size, exact O(N^2) sums to interpolation accuracy
@@ -530,6 +531,66 @@ void oracle_symmetrize(const float *p, const int *idx, int N, int K, float *P) {
             for (int u = 0; u < K; ++u) acc += (idx[(size_t)j * K + u] == i) ? p[(size_t)j * K + u] : 0.0f;
             P[t] = (float)(acc / (2.0 * N));
         }
+    }
+}
+
+// Full symmetrisation (A + A^T) / 2N with the union pattern, CSR with ascending columns: what the reference
+// holds as a commented-out cuSPARSE routine (src/util/math_utils.cu:76-225: csrsort, csr2csc, csrgeam with
+// alpha = beta = 1 / (2N)) and the library offers as an option.  A[i, idx[i,s]] = p[i,s]; an entry's value is
+// the fp32 sum of what A and A^T hold there (own entry first), divided by 2.0 * N in double, rounded to float -
+// the arithmetic of oracle_symmetrize.  row_ptr: N + 1; col_idx / values: room for 2 N K.  Returns the count.
+int64_t oracle_symmetrize_full(const float *p, const int *idx, int N, int K, int *row_ptr, int *col_idx,
+                               float *values) {
+    struct Item {
+        int col;
+        float v;
+    };
+    // The triples are taken entry by entry, (i, j) then (j, i); rows are filled in that order and sorted stably,
+    // so equal (row, column) pairs are summed in the order in which they were generated.
+    std::vector<std::vector<Item>> rows(N);
+    for (int i = 0; i < N; ++i)
+        for (int s = 0; s < K; ++s) {
+            const size_t t = (size_t)i * K + s;
+            const int j = idx[t];
+            rows[i].push_back({j, p[t]});
+            rows[j].push_back({i, p[t]});
+        }
+    int64_t out = 0;
+    for (int i = 0; i < N; ++i) {
+        auto &r = rows[i];
+        std::stable_sort(r.begin(), r.end(), [](const Item &a, const Item &b) { return a.col < b.col; });
+        row_ptr[i] = (int)out;
+        for (size_t a = 0; a < r.size();) {
+            float sum = r[a].v;
+            size_t b = a + 1;
+            for (; b < r.size() && r[b].col == r[a].col; ++b) sum += r[b].v;
+            col_idx[out] = r[a].col;
+            values[out] = (float)((double)sum / (2.0 * N));
+            ++out;
+            a = b;
+        }
+    }
+    row_ptr[N] = (int)out;
+    return out;
+}
+
+// Attractive forces over a CSR pattern (same terms as oracle_attractive, row by row in stored order).
+void oracle_attractive_csr(const int *row_ptr, const int *col_idx, const float *values, const float *Y, int N,
+                           float *attr) {
+#pragma omp parallel for schedule(static)
+    for (int i = 0; i < N; ++i) {
+        const float ix = Y[i], iy = Y[N + i];
+        float ax = 0.0f, ay = 0.0f;
+        for (int e = row_ptr[i]; e < row_ptr[i + 1]; ++e) {
+            const int j = col_idx[e];
+            const float dx = ix - Y[j];
+            const float dy = iy - Y[N + j];
+            const float w = values[e] / (1 + dx * dx + dy * dy);
+            ax += w * dx;
+            ay += w * dy;
+        }
+        attr[i] = ax;
+        attr[N + i] = ay;
     }
 }
 

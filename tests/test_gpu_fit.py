@@ -222,6 +222,45 @@ def test_repulsion_monitor_lines(c0_problem, capfd, monkeypatch):
     assert 0.0 < err < 0.1
 
 
+def test_fit_with_full_symmetrisation(c0_problem, monkeypatch, capfd):
+    """TSNE_SYMMETRIZE=full: the gradient loop over (A + A^T) / 2N with the union pattern (CSR).  The fit's
+    objective is then taken over that pattern, whose mass is 1 (the default pattern drops ~a fifth of it
+    at K = 90), so it comes out higher; the embedding is as trustworthy as the default one's."""
+    from tsnecuda import TSNE
+    c = c0_problem
+    X = c["X"]
+    Y0 = synthetic_start(X.shape[0])
+    kw = dict(perplexity=30.0, num_neighbors=90, n_iter=500, perplexity_epsilon=1e-4)
+    base = TSNE(**kw)
+    base.fit_transform(X, y=Y0)
+    t_base = base.trustworthiness(12)
+    monkeypatch.setenv("TSNE_SYMMETRIZE", "full")
+    full = TSNE(verbose=1, print_interval=250, **kw)
+    emb = full.fit_transform(X, y=Y0)
+    out = capfd.readouterr().out
+    assert "non-zeros after full symmetrisation" in out
+    stored = int(out.split(" non-zeros after full symmetrisation")[0].split("(")[-1])
+    rp, cc, vv = oracle.symmetrize_full(c["p"], c["idx"])
+    assert stored == cc.size
+    assert np.isfinite(emb).all() and full.kl_divergence_ > 0
+    assert abs(full.trustworthiness(12) - t_base) <= 0.02
+    # the objective of the returned embedding over the CSR pattern, re-evaluated on the host (exact Z)
+    n = X.shape[0]
+    ex, ey = emb[:, 0].astype(np.float64), emb[:, 1].astype(np.float64)
+    rows = np.repeat(np.arange(n), np.diff(rp))
+    d2 = (ex[rows] - ex[cc]) ** 2 + (ey[rows] - ey[cc]) ** 2
+    dx, dy = ex[:, None] - ex[None, :], ey[:, None] - ey[None, :]
+    Z = (1.0 / (1.0 + dx * dx + dy * dy)).sum() - n
+    pos = vv > 0
+    kl = float((vv[pos].astype(np.float64) * (np.log(vv[pos].astype(np.float64)) + np.log1p(d2[pos]) + np.log(Z))).sum())
+    assert abs(full.kl_divergence_ - kl) <= 0.01 * kl
+
+
+def synthetic_start(n):
+    from tsnecuda import synthetic
+    return synthetic.initial_embedding(n)
+
+
 def test_dump_file_format(tmp_path, c0_problem):
     """Text dump: header "N 2" then N lines "x y" per dumped step
     (src/fit_tsne.cu:347-352,563-570)."""

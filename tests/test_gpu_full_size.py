@@ -85,6 +85,50 @@ def test_normalise_perplexity_symmetrise(c3):
     c3["P_h"], c3["idx_h"] = P_o, idx_h
 
 
+def test_full_symmetrisation(c3):
+    """(A + A^T) / 2N as CSR at a million points (180 M triples through the device radix sort): structure,
+    mass, symmetry of every entry, and 48 rows rebuilt on the host from the conditional probabilities."""
+    import time
+    st = c3["stages"]
+    cond, idx = c3["cond"], c3["idx"]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    row_ptr, col, val = st.symmetrize_full(cond, idx)
+    torch.cuda.synchronize()
+    nnz_sym = col.numel()
+    print("symmetrize_full c3: %.1f ms, %d non-zeros (%.2f x N K)" % ((time.perf_counter() - t0) * 1e3, nnz_sym,
+                                                                     nnz_sym / (N * K)))
+    assert N * K <= nnz_sym <= 2 * N * K
+    rp = row_ptr.long()
+    assert int(rp[0]) == 0 and int(rp[-1]) == nnz_sym and bool((rp[1:] - rp[:-1] >= K).all())
+    assert abs(float(val.sum(dtype=torch.float64)) - 1.0) <= 1e-5
+    rows = torch.repeat_interleave(torch.arange(N, device="cuda"), rp[1:] - rp[:-1])
+    keys = rows * N + col.long()
+    assert bool((keys[1:] > keys[:-1]).all())  # rows in order, columns ascending and distinct inside a row
+    # symmetry: the transposed keys, sorted, carry the same values
+    order = torch.argsort(col.long() * N + rows)
+    assert torch.equal(col.long()[order] * N + rows[order], keys)
+    assert torch.equal(val[order], val)
+    del keys, order
+    # sampled rows against the definition
+    cond_h = None
+    for r in list(range(0, 16)) + list(range(500000, 500016)) + list(range(N - 16, N)):
+        own_c = idx[r].long()
+        own_v = cond[r]
+        src = (idx == r).nonzero()  # (row, slot) of every entry that names r
+        inc_c, inc_v = src[:, 0], cond[src[:, 0], src[:, 1]]
+        dense = {}
+        for c_, v_ in zip(own_c.tolist(), own_v.tolist()):
+            dense[c_] = np.float32(v_)
+        for c_, v_ in zip(inc_c.tolist(), inc_v.tolist()):
+            dense[c_] = np.float32(dense.get(c_, np.float32(0.0)) + np.float32(v_))
+        lo, hi = int(rp[r]), int(rp[r + 1])
+        assert col[lo:hi].tolist() == sorted(dense)
+        want = np.array([np.float32(float(dense[c_]) / (2.0 * N)) for c_ in sorted(dense)], np.float32)
+        assert np.array_equal(val[lo:hi].cpu().numpy(), want)
+    c3["csr"] = (row_ptr, col, val)
+
+
 def test_forces_and_fused_steps(c3):
     st = c3["stages"]
     P_h, idx_h = c3["P"].cpu().numpy(), c3["idx"].cpu().numpy()

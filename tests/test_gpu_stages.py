@@ -89,6 +89,66 @@ def test_symmetrize(stages, c0_problem):
     np.testing.assert_allclose(P, c["P"], rtol=1e-6, atol=0)
 
 
+@pytest.mark.parametrize("n,k", [(2, 2), (7, 3), (300, 300), (5000, 90), (70000, 20), (20000, 1)])
+def test_symmetrize_full_csr(stages, c0_problem, n, k):
+    """(A + A^T) / 2N with the union pattern: the device radix sort + segmented reduce against the oracle's
+    CSR, bit for bit (row pointers, columns, values) - one tile and several tiles of the sort, dense rows,
+    K = 1 (every row: the explicit zero of the self entry only)."""
+    if (n, k) == (5000, 90):
+        p, idx = c0_problem["p"], c0_problem["idx"]
+    else:
+        # row i names the columns i + o for the k offsets o of one of seven offset sets (0 = itself first, the
+        # others distinct): distinct columns in every row, in-degrees that vary from row to row
+        rng = np.random.default_rng(n * 31 + k)
+        sets = np.stack([np.concatenate([[0], 1 + rng.choice(n - 1, size=k - 1, replace=False)]) for _ in range(7)])
+        idx = ((np.arange(n)[:, None] + sets[np.arange(n) % 7]) % n).astype(np.int32)
+        p = rng.random(idx.shape).astype(np.float32)
+        p[:, 0] = 0.0
+        p /= np.maximum(p.sum(1, keepdims=True), 1e-30)
+    want_ptr, want_col, want_val = oracle.symmetrize_full(p, idx)
+    row_ptr, col, val = stages.symmetrize_full(dev(p), dev(idx))
+    assert np.array_equal(row_ptr.cpu().numpy(), want_ptr)
+    assert np.array_equal(col.cpu().numpy(), want_col)
+    assert np.array_equal(val.cpu().numpy().view(np.uint32), want_val.view(np.uint32))
+    if k > 1:
+        assert abs(float(val.sum(dtype=torch.float64)) - 1.0) <= 1e-5
+    # forces over the CSR pattern, stage call and fused loop
+    nn = idx.shape[0]
+    rng = np.random.default_rng(1)
+    y = (rng.standard_normal(2 * nn) * 3.0).astype(np.float32)
+    plan = stages.Plan(nn, k)
+    got = plan.attractive_csr(row_ptr, col, val, dev(y)).cpu().numpy()
+    want = oracle.attractive_csr(want_ptr, want_col, want_val, y)
+    if np.linalg.norm(want) > 0:
+        assert rel_l2(got, want) <= 1e-4
+    plan.close()
+
+
+def test_iterate_over_the_full_csr_pattern(stages, c0_problem):
+    """Steps whose attractive forces come from the fully symmetrised CSR pattern, against the same steps
+    with the forces of the oracle's CSR evaluation: the embedding after three steps."""
+    c = c0_problem
+    n = c["X"].shape[0]
+    row_ptr, col, val = stages.symmetrize_full(dev(c["p"]), dev(c["idx"]))
+    plan = stages.Plan(n, c["K"])
+    plan.set_csr_pattern(row_ptr, col, val)
+    dy = dev(c["y0"])
+    gains, old = torch.ones_like(dy), torch.zeros_like(dy)
+    plan.iterate_(None, None, dy, gains, old, 0, 3)
+    # the oracle's loop, its attractive stage replaced by the CSR evaluation
+    y = c["y0"].copy()
+    g, u = np.ones_like(y), np.zeros_like(y)
+    rp, cc, vv = oracle.symmetrize_full(c["p"], c["idx"])
+    for _ in range(3):
+        rep, z = oracle.repulsive(y)
+        y, g, u = oracle.update(y, oracle.attractive_csr(rp, cc, vv, y), rep, g, u, 200.0, z, 0.5, 12.0)
+    assert rel_l2(dy.cpu().numpy(), y) <= 1e-4
+    plan.set_csr_pattern(None, None, None)
+    with pytest.raises(RuntimeError, match="none prepared"):
+        plan.iterate_(None, None, dy, gains, old, 0, 1)
+    plan.close()
+
+
 @pytest.mark.parametrize("step", [0, 30, 300])
 def test_attractive(stages, c0_problem, snapshots, step):
     c = c0_problem

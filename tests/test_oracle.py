@@ -233,6 +233,41 @@ def test_symmetrize_dense(small):
     assert P.sum() <= 1.0 + 1e-6  # one-directional pairs lose half their mass
 
 
+def test_symmetrize_full_against_dense_and_scipy(small):
+    import scipy.sparse as sp
+    n, k, idx, p = small["n"], small["k"], small["idx"], small["p"]
+    row_ptr, col, val = oracle.symmetrize_full(p, idx)
+    A = np.zeros((n, n), np.float64)
+    A[np.repeat(np.arange(n), k), idx.ravel()] = p.ravel()
+    want = (A + A.T) / (2.0 * n)
+    got = sp.csr_matrix((val, col, row_ptr), shape=(n, n))
+    assert got.has_sorted_indices and np.all(np.diff(row_ptr) >= k)
+    dense = got.toarray().astype(np.float64)
+    assert np.abs(dense - want).max() <= 1e-7 * want.max()
+    # the pattern is the union of A's and A^T's (the explicit zero of the self entry included)
+    pattern = np.zeros((n, n), bool)
+    pattern[np.repeat(np.arange(n), k), idx.ravel()] = True
+    stored = np.zeros((n, n), bool)
+    stored[np.repeat(np.arange(n), np.diff(row_ptr)), col] = True
+    assert np.array_equal(stored, pattern | pattern.T)
+    # nothing is dropped: the mass is 1, where the pattern-restricted form loses the unmirrored entries
+    assert abs(val.astype(np.float64).sum() - 1.0) <= 1e-5
+    assert small["P"].astype(np.float64).sum() < val.astype(np.float64).sum()
+    # ... and scipy's own (A + A^T) / 2N
+    As = sp.csr_matrix((p.ravel().astype(np.float64), idx.ravel(), np.arange(0, n * k + 1, k)), shape=(n, n))
+    ref = ((As + As.T) / (2.0 * n)).tocsr()
+    assert abs(ref - got).max() <= 1e-7 * want.max()
+    # forces over the CSR pattern against the dense sum
+    rng = np.random.default_rng(3)
+    y = (rng.standard_normal(2 * n) * 2.0).astype(np.float32)
+    attr = oracle.attractive_csr(row_ptr, col, val, y)
+    yx, yy = y[:n].astype(np.float64), y[n:].astype(np.float64)
+    dx, dy = yx[:, None] - yx[None, :], yy[:, None] - yy[None, :]
+    wgt = want / (1.0 + dx * dx + dy * dy)
+    dense_force = np.concatenate([(wgt * dx).sum(1), (wgt * dy).sum(1)])
+    assert rel_l2(attr, dense_force) < 1e-5
+
+
 # ---------------------------------------------------------- attractive ------
 def test_attractive_dense(small):
     n, k, idx, P, y = small["n"], small["k"], small["idx"], small["P"], small["y"]

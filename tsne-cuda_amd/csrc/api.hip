@@ -108,13 +108,21 @@ static bool overlap_enabled() {
 // step follows the update on its own stream without a hand-over, and every step leaves the caller's stream
 // joined with the side stream.  (With the update on the side stream behind the chain, as it was while the
 // attractive kernel was the longer of the two, a step took 2 % longer.)
+// Attractive forces of a step: the explicit N x K pattern if given, else the plan's CSR pattern if one is set,
+// else the re-blocked pattern.
+static int launch_step_attractive(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s) {
+    if (pij) return launch_attractive(p, pij, indices, p->attr, s);
+    if (p->csr_row_ptr) return launch_attractive_csr(p, p->csr_row_ptr, p->csr_col_idx, p->csr_values, p->attr, s);
+    return launch_attractive_blocked(p, p->attr, s);
+}
+
 int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
                 float *old_forces, float eta, float momentum, float exaggeration, int slot, float *normalization,
                 hipStream_t s) {
     const bool overlap = overlap_enabled() && !p->profiling && p->side_stream != nullptr;
     if (!overlap) {
         if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, s)) return 1;
-        if (pij ? launch_attractive(p, pij, indices, p->attr, s) : launch_attractive_blocked(p, p->attr, s)) return 1;
+        if (launch_step_attractive(p, pij, indices, s)) return 1;
         if (normalization && launch_finish_z(p, normalization, s)) return 1;
         return launch_update(p, embedding, p->attr, p->rep, gains, old_forces, eta, nullptr, momentum, exaggeration,
                              slot ^ 1, s);
@@ -125,7 +133,7 @@ int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *e
     if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, side)) return 1;
     if (normalization && launch_finish_z(p, normalization, side)) return 1;
     TSNE_TRY(hipEventRecord(p->join_event, side));
-    if (pij ? launch_attractive(p, pij, indices, p->attr, s) : launch_attractive_blocked(p, p->attr, s)) return 1;
+    if (launch_step_attractive(p, pij, indices, s)) return 1;
     TSNE_TRY(hipStreamWaitEvent(s, p->join_event, 0));
     return launch_update(p, embedding, p->attr, p->rep, gains, old_forces, eta, nullptr, momentum, exaggeration,
                          slot ^ 1, s);
@@ -422,7 +430,7 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
     if (check_plan(plan, "iterate")) return 1;
     TSNE_REQUIRE(embedding && gains && old_forces, "iterate: null pointer argument");
     TSNE_REQUIRE((pij == nullptr) == (indices == nullptr), "iterate: pij and indices must both be given or both be null");
-    TSNE_REQUIRE(pij || plan->blocked_ready, "iterate: no pattern given and none prepared");
+    TSNE_REQUIRE(pij || plan->blocked_ready || plan->csr_row_ptr, "iterate: no pattern given and none prepared");
     TSNE_REQUIRE(step_begin <= step_end, "iterate: step range [%d, %d) is reversed", step_begin, step_end);
     if (step_begin == step_end) return 0;
     // The loop runs on the plan's own stream, tied to the caller's stream by an event at either end.
@@ -490,6 +498,38 @@ int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches) {
         launches[id] += 1;
     }
     plan->events_used = 0;
+    return 0;
+}
+
+int tsne_hip_symmetrize_full(const float *pij_non_symmetric, const int *indices, int num_points, int num_neighbors,
+                             int *row_ptr, int *col_idx, float *values, int64_t *nnz, void *stream) {
+    TSNE_REQUIRE(pij_non_symmetric && indices && row_ptr && col_idx && values, "symmetrize_full: null pointer argument");
+    TSNE_REQUIRE(num_points > 0 && num_neighbors > 0, "symmetrize_full: empty problem (%d x %d)", num_points,
+                 num_neighbors);
+    return symmetrize_full(pij_non_symmetric, indices, num_points, num_neighbors, row_ptr, col_idx, values, nnz,
+                           (hipStream_t)stream);
+}
+
+int tsne_hip_attractive_csr(tsne_hip_plan *plan, const int *row_ptr, const int *col_idx, const float *values,
+                            const float *embedding, float *attractive_forces, void *stream) {
+    if (check_plan(plan, "attractive_csr")) return 1;
+    TSNE_REQUIRE(row_ptr && col_idx && values && embedding && attractive_forces, "attractive_csr: null pointer argument");
+    hipStream_t s = (hipStream_t)stream;
+    if (launch_pack_xy(plan, embedding, s)) return 1;
+    return launch_attractive_csr(plan, row_ptr, col_idx, values, attractive_forces, s);
+}
+
+int tsne_hip_plan_set_csr_pattern(tsne_hip_plan *plan, const int *row_ptr, const int *col_idx, const float *values) {
+    if (check_plan(plan, "plan_set_csr_pattern")) return 1;
+    TSNE_REQUIRE((row_ptr != nullptr) == (col_idx != nullptr) && (row_ptr != nullptr) == (values != nullptr),
+                 "plan_set_csr_pattern: give all three arrays or none");
+    // Captured steps hold the pattern they were captured with.
+    TSNE_TRY(hipDeviceSynchronize());
+    for (auto &g : plan->step_graphs) (void)hipGraphExecDestroy(g.exec);
+    plan->step_graphs.clear();
+    plan->csr_row_ptr = row_ptr;
+    plan->csr_col_idx = col_idx;
+    plan->csr_values = values;
     return 0;
 }
 

@@ -185,16 +185,33 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     // ---- P matrix --------------------------------------------------------
     clock.start();
     if (verbose) std::cout << "done.\nComputing Pij matrix... " << std::endl;
-    DeviceBuffer d_pij(sizeof(float) * nnz);
+    // TSNE_SYMMETRIZE=full (or Options::full_symmetrization): P = (A + A^T) / 2N with the union pattern, in CSR
+    // form, instead of the reference's pattern-restricted form; the attractive forces then run over the CSR rows.
+    const char *sym_env = std::getenv("TSNE_SYMMETRIZE");
+    const bool full_sym = opt.full_symmetrization || (sym_env && std::string(sym_env) == "full");
+    DeviceBuffer d_pij, d_row_ptr, d_col, d_val;
     {
         DeviceBuffer d_cond(sizeof(float) * nnz);
         TSNE_OR_DIE(tsnehip::launch_perplexity(d_dist.as<float>(), N, K, opt.perplexity,
                                                opt.perplexity_search_epsilon, d_cond.as<float>(), nullptr,
                                                stream),
                     "perplexity search");
-        TSNE_OR_DIE(tsnehip::launch_symmetrize(d_cond.as<float>(), d_idx.as<int>(), N, K, d_pij.as<float>(),
-                                               stream),
-                    "symmetrisation");
+        if (full_sym) {
+            DeviceBuffer row_ptr(sizeof(int) * ((size_t)N + 1)), col(sizeof(int) * 2 * nnz), val(sizeof(float) * 2 * nnz);
+            int64_t stored = 0;
+            TSNE_OR_DIE(tsnehip::symmetrize_full(d_cond.as<float>(), d_idx.as<int>(), N, K, row_ptr.as<int>(),
+                                                 col.as<int>(), val.as<float>(), &stored, stream),
+                        "full symmetrisation");
+            if (verbose) std::cout << "(" << stored << " non-zeros after full symmetrisation) " << std::flush;
+            d_row_ptr.swap(row_ptr);
+            d_col.swap(col);
+            d_val.swap(val);
+        } else {
+            DeviceBuffer pij(sizeof(float) * nnz);
+            TSNE_OR_DIE(tsnehip::launch_symmetrize(d_cond.as<float>(), d_idx.as<int>(), N, K, pij.as<float>(), stream),
+                        "symmetrisation");
+            d_pij.swap(pij);
+        }
         hip_or_die(hipStreamSynchronize(stream), "P matrix");
     }
     d_dist.release();
@@ -250,11 +267,20 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     // Re-block the sparse pattern for the LDS-staged attractive kernel; shapes it
     // cannot hold (very large K or N) keep the row-ordered kernel.
     // (The row-ordered pattern stays: the objective of the final embedding is evaluated on it.)
-    const int prepared = tsnehip::prepare_blocked(plan, d_pij.as<float>(), d_idx.as<int>(), stream);
-    if (prepared != 0 && prepared != tsnehip::kShapeNotSupported) die("re-blocking of the sparse pattern");
-    const bool blocked = prepared == 0;
-    if (!blocked && verbose)
-        std::cout << "(" << tsnehip::last_error() << "; using the row-ordered attractive kernel) " << std::flush;
+    bool blocked = false;
+    if (full_sym) {
+        plan->csr_row_ptr = d_row_ptr.as<int>();
+        plan->csr_col_idx = d_col.as<int>();
+        plan->csr_values = d_val.as<float>();
+    } else {
+        const int prepared = tsnehip::prepare_blocked(plan, d_pij.as<float>(), d_idx.as<int>(), stream);
+        if (prepared != 0 && prepared != tsnehip::kShapeNotSupported) die("re-blocking of the sparse pattern");
+        blocked = prepared == 0;
+        if (!blocked && verbose)
+            std::cout << "(" << tsnehip::last_error() << "; using the row-ordered attractive kernel) " << std::flush;
+    }
+    // No explicit N x K pattern goes to the steps when the plan holds the pattern itself (re-blocked or CSR).
+    const bool plan_pattern = blocked || full_sym;
 
     std::ofstream dump_file;
     if (opt.get_dump_points()) {
@@ -311,8 +337,8 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
                 hipStream_t batch_stream = plan->loop_stream;
                 hip_or_die(hipEventRecord(plan->enter_event, stream), "event");
                 hip_or_die(hipStreamWaitEvent(batch_stream, plan->enter_event, 0), "event");
-                TSNE_OR_DIE(tsnehip::launch_steps(plan, blocked ? nullptr : d_pij.as<float>(),
-                                                  blocked ? nullptr : d_idx.as<int>(), d_emb.as<float>(),
+                TSNE_OR_DIE(tsnehip::launch_steps(plan, plan_pattern ? nullptr : d_pij.as<float>(),
+                                                  plan_pattern ? nullptr : d_idx.as<int>(), d_emb.as<float>(),
                                                   d_gains.as<float>(), d_old.as<float>(), opt.learning_rate,
                                                   momentum, exaggeration, (int)count, slot, batch_stream),
                             "gradient steps");
@@ -324,8 +350,8 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         }
         if (!timing) {
             // Repulsive chain and attractive kernel side by side (plan's side stream), joined before the update.
-            TSNE_OR_DIE(tsnehip::launch_step(plan, blocked ? nullptr : d_pij.as<float>(),
-                                             blocked ? nullptr : d_idx.as<int>(), d_emb.as<float>(),
+            TSNE_OR_DIE(tsnehip::launch_step(plan, plan_pattern ? nullptr : d_pij.as<float>(),
+                                             plan_pattern ? nullptr : d_idx.as<int>(), d_emb.as<float>(),
                                              d_gains.as<float>(), d_old.as<float>(), opt.learning_rate, momentum,
                                              exaggeration, slot, want_norm ? d_norm.as<float>() : nullptr, stream),
                         "gradient step");
@@ -335,9 +361,11 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
             TSNE_OR_DIE(tsnehip::launch_repulsive(plan, d_emb.as<float>(), slot, plan->rep, nullptr, nullptr, stream),
                         "repulsive forces");
             hip_or_die(hipEventRecord(ev[1], stream), "event");
-            TSNE_OR_DIE(blocked ? tsnehip::launch_attractive_blocked(plan, plan->attr, stream)
-                                : tsnehip::launch_attractive(plan, d_pij.as<float>(), d_idx.as<int>(), plan->attr,
-                                                             stream),
+            TSNE_OR_DIE(full_sym ? tsnehip::launch_attractive_csr(plan, plan->csr_row_ptr, plan->csr_col_idx,
+                                                                  plan->csr_values, plan->attr, stream)
+                        : blocked ? tsnehip::launch_attractive_blocked(plan, plan->attr, stream)
+                                  : tsnehip::launch_attractive(plan, d_pij.as<float>(), d_idx.as<int>(), plan->attr,
+                                                               stream),
                         "attractive forces");
             hip_or_die(hipEventRecord(ev[2], stream), "event");
             if (want_norm) TSNE_OR_DIE(tsnehip::launch_finish_z(plan, d_norm.as<float>(), stream), "normalisation");
@@ -447,8 +475,10 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         TSNE_OR_DIE(tsnehip::launch_repulsive(plan, d_emb.as<float>(), slot, plan->rep, nullptr, nullptr, stream),
                     "final normalisation");
         TSNE_OR_DIE(tsnehip::launch_finish_z(plan, d_norm.as<float>(), stream), "final normalisation");
-        TSNE_OR_DIE(tsnehip::launch_kl_terms(d_pij.as<float>(), d_idx.as<int>(), d_emb.as<float>(), N, K,
-                                             d_kl.as<double>(), stream),
+        TSNE_OR_DIE(full_sym ? tsnehip::launch_kl_terms_csr(d_row_ptr.as<int>(), d_col.as<int>(), d_val.as<float>(),
+                                                            d_emb.as<float>(), N, d_kl.as<double>(), stream)
+                             : tsnehip::launch_kl_terms(d_pij.as<float>(), d_idx.as<int>(), d_emb.as<float>(), N, K,
+                                                        d_kl.as<double>(), stream),
                     "objective");
         hip_or_die(hipMemcpy(&z_final, d_norm.ptr, sizeof(float), hipMemcpyDeviceToHost), "objective");
         hip_or_die(hipMemcpy(terms, d_kl.ptr, sizeof(terms), hipMemcpyDeviceToHost), "objective");

@@ -78,6 +78,10 @@ struct tsne_hip_plan {
     int strip_rows = 0, n_strips = 0, n_parts = 0, list_words = 0, seg_stride = 0;
     int spin_limit = 0;             // polls before a wave of the attractive kernel gives up a wait
     bool blocked_ready = false;
+    // Optional CSR pattern (borrowed pointers; tsne_hip_plan_set_csr_pattern): when set, steps without an explicit
+    // N x K pattern take their attractive forces from it.
+    const int *csr_row_ptr = nullptr, *csr_col_idx = nullptr;
+    const float *csr_values = nullptr;
     bool recenter = false;          // the loop's updates re-centre the embedding (tsne_hip_plan_set_recenter)
 
     // The repulsive chain and the attractive kernel of a step are independent: the fused loop runs
@@ -148,6 +152,8 @@ constexpr int kShapeNotSupported = 2;
 int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s);
 void release_blocked(tsne_hip_plan *p);
 int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s);
+int launch_attractive_csr(tsne_hip_plan *p, const int *row_ptr, const int *col_idx, const float *values, float *attr,
+                          hipStream_t s);
 int check_attractive_waits(tsne_hip_plan *p);
 int launch_sum_squares(const float *values, int64_t n, float *out, hipStream_t s);
 int launch_centre_sums(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s);

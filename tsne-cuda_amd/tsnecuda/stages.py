@@ -33,6 +33,12 @@ def lib():
         L.tsne_hip_max_normalize_noalloc.restype = c_int
         L.tsne_hip_perplexity.argtypes = [_vp, c_int, c_int, c_float, c_float, _vp, _vp, _vp]
         L.tsne_hip_symmetrize.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
+        L.tsne_hip_symmetrize_full.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp, _vp, ctypes.POINTER(c_i64), _vp]
+        L.tsne_hip_symmetrize_full.restype = c_int
+        L.tsne_hip_attractive_csr.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp]
+        L.tsne_hip_attractive_csr.restype = c_int
+        L.tsne_hip_plan_set_csr_pattern.argtypes = [_vp, _vp, _vp, _vp]
+        L.tsne_hip_plan_set_csr_pattern.restype = c_int
         L.tsne_hip_plan_create.argtypes = [ctypes.POINTER(_vp), c_int, c_int, c_int, c_int]
         L.tsne_hip_plan_check.argtypes = [_vp]
         L.tsne_hip_plan_set_recenter.argtypes = [_vp, c_int]
@@ -150,6 +156,19 @@ def symmetrize(pij, idx):
     return out
 
 
+def symmetrize_full(pij, idx):
+    """(A + A^T) / 2N with the union pattern as CSR tensors (row_ptr, col_idx, values)."""
+    pij = _f32(pij)
+    n, k = pij.shape
+    row_ptr = torch.empty(n + 1, dtype=torch.int32, device=pij.device)
+    col = torch.empty(2 * n * k, dtype=torch.int32, device=pij.device)
+    val = torch.empty(2 * n * k, dtype=torch.float32, device=pij.device)
+    nnz = ctypes.c_int64(0)
+    _check(lib().tsne_hip_symmetrize_full(_ptr(pij), _ptr(idx), n, k, _ptr(row_ptr), _ptr(col), _ptr(val),
+                                          ctypes.byref(nnz), _stream()))
+    return row_ptr, col[:nnz.value], val[:nnz.value]
+
+
 class Plan(object):
     """Scratch memory of the gradient loop for one problem size."""
 
@@ -192,6 +211,18 @@ class Plan(object):
         _check(lib().tsne_hip_attractive(self._h, _ptr(None if pij is None else _f32(pij)), _ptr(idx),
                                          _ptr(_f32(embedding)), _ptr(out), _stream()))
         return out
+
+    def attractive_csr(self, row_ptr, col_idx, values, embedding):
+        out = torch.empty(2 * self.num_points, dtype=torch.float32, device=self.device)
+        _check(lib().tsne_hip_attractive_csr(self._h, _ptr(row_ptr), _ptr(col_idx), _ptr(_f32(values)),
+                                             _ptr(_f32(embedding)), _ptr(out), _stream()))
+        return out
+
+    def set_csr_pattern(self, row_ptr, col_idx, values):
+        """iterate_(None, None, ...) then takes its attractive forces from this CSR pattern (the tensors
+        must stay alive); three Nones clear it."""
+        self._csr = (row_ptr, col_idx, values)
+        _check(lib().tsne_hip_plan_set_csr_pattern(self._h, _ptr(row_ptr), _ptr(col_idx), _ptr(values)))
 
     def repulsive(self, embedding, details=False):
         n, g = self.num_points, self.n_nodes
