@@ -111,6 +111,20 @@ def main():
     dXs, gather_s = timed(lambda: stages.gather_rows(dX, order))
     del dX
     (idx, d2, knn_stats), knn_s = timed(lambda: stages.knn_select(dXs, k, 0))  # 0: what tsne_hip_knn does
+    # The optional approximate search (inverted file, floor(sqrt(N)) lists as the reference's FAISS index, 100
+    # lists probed per list: what TSNE_KNN=ivf runs): training and search timed, recall against the exact rows.
+    approx = None
+    if d <= 126 and n >= 4096:
+        import math
+        nlist = int(math.isqrt(n))
+        cen, train_s = timed(lambda: stages.ivf_train(dXs, nlist))
+        (idx_a, _, stats_a), search_s = timed(lambda: stages.knn_ivf(dXs, k, cen, min(100, nlist)))
+        rows = torch.arange(0, n, max(1, n // 4096), device="cuda")[:4096]
+        hits = (idx_a[rows, 1:, None] == idx[rows, None, 1:]).any(2).float().mean().item()
+        approx = {"nlist": nlist, "nprobe_per_list": min(100, nlist), "train_s": train_s, "search_s": search_s,
+                  "recall_at_%d" % (k - 1): hits, "recall_rows": int(rows.numel()),
+                  "tile_pairs_per_mille": stats_a[2]}
+        del idx_a, cen
     del dXs
     order_h = order.cpu().numpy().astype(np.int64)
     y0 = np.concatenate([y0[:n][order_h], y0[n:][order_h]])
@@ -299,6 +313,7 @@ def main():
                      "traffic_source": traffic_source, "bytes_per_launch": attr_bytes, "ms_per_launch": attr_ms},
         "kernels_us": kernels_us,
         "phase_rooflines": phase_rooflines,
+        "knn_approximate": approx,
         "cpu_baseline": cpu,
         "final_Z": float(z.item()),
     }

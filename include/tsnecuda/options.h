@@ -100,6 +100,20 @@ class Options {
     // (src/util/math_utils.cu:269-308).  Off by default; TSNE_SYMMETRIZE=full in the environment also enables it.
     bool full_symmetrization = false;
 
+    // Approximate neighbours through an inverted file, the structure of the reference's FAISS search
+    // (src/util/distance_utils.cu:85-120: floor(sqrt(N)) lists, 20 probed); the default here is the exact search.
+    // knn_nprobe: lists probed by each list (0: 100, which on 50-dimensional Gaussian clusters finds about as many
+    // of the true neighbours as FAISS's 20 lists per query).  TSNE_KNN=ivf and TSNE_KNN_NPROBE=<n> in the
+    // environment do the same.  Inputs of more than 126 dimensions keep the exact search.
+    bool approximate_neighbors = false;
+    int knn_nprobe = 0;
+
+    // FIt-SNE's rule for the size of the interpolation grid, which the reference carries as a comment
+    // (src/fit_tsne.cu:435) while it runs a fixed 130 boxes per dimension: every 50 steps the grid is set to
+    // max(125, spread of the embedding) boxes, rounded up in the reference's list of sizes (at most 170 here).
+    // Off by default; TSNE_ADAPTIVE_BOXES=1 in the environment also enables it.
+    bool adaptive_boxes = false;
+
     Options() {}
 
     Options(float *return_data, float *points, int num_points, int num_dims)

@@ -59,6 +59,30 @@ int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neig
 int tsne_hip_knn_select(const float *points, int num_points, int num_dims, int num_neighbors, int *indices,
                         float *sq_dist, void *stream, int sweep, int *stats);
 
+/* Approximate neighbours through an inverted file, the structure of the reference's own
+ * search (FAISS IndexIVFFlat, nlist = floor(sqrt(N)), nprobe = 20, L2:
+ * src/util/distance_utils.cu:85-120), for sizes at which the exact search dominates a fit.
+ *
+ * tsne_hip_ivf_train: nlist centroids (device, nlist x num_dims floats) from `iterations`
+ * Lloyd iterations on a pseudo-random sample of up to 64 points per list.  At most 128
+ * dimensions.  Synchronises the stream.
+ *
+ * tsne_hip_knn_ivf: every point is filed under its nearest centroid; a list probes the
+ * nprobe lists whose centroids are nearest to its own (itself included), and a query is
+ * compared with the points of the lists probed by the lists of its 128-point tile (consecutive
+ * points of the list-by-list numbering; mostly one list) and with the 8 tiles either side of
+ * its own; among those candidates the result is exact (same distances, order and self-first
+ * rule as tsne_hip_knn).  (FAISS probes the lists nearest to the query itself; here the
+ * probes hang on the query's list so that the queries of a tile, whose distances the
+ * matrix sweep computes together, share them.)  Given the centroids the result is a deterministic function of the points.
+ * At most 126 dimensions, num_points >= 8192, nprobe <= 32.  stats as in tsne_hip_knn_select
+ * ([1]: queries whose candidates failed the sweep's verification - near-duplicate points -
+ * and were answered by the exact sweep over all points instead).  Synchronises the stream. */
+int tsne_hip_ivf_train(const float *points, int num_points, int num_dims, int nlist, int iterations, float *centroids,
+                       void *stream);
+int tsne_hip_knn_ivf(const float *points, int num_points, int num_dims, int num_neighbors, const float *centroids,
+                     int nlist, int nprobe, int *indices, float *sq_dist, void *stream, int *stats);
+
 /* Locality ordering of the points: order[new] = old (int32, device, num_points
  * entries) such that points that are close in the input space get close numbers
  * (nearest of 64 to 256 pivots taken from the data, pivots chained greedily;
@@ -196,6 +220,17 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
  * update kernel: the forces are translation invariant, so this is re-centring after
  * every step, applied one step late and without a pass of its own. */
 int tsne_hip_plan_set_recenter(tsne_hip_plan *plan, int enable);
+
+/* Grid size of the interpolation scheme, changeable between steps.  The reference fixes
+ * 125 boxes per dimension, rounded up to 130 in its list of sizes (src/fit_tsne.cu:246-266),
+ * and carries FIt-SNE's adaptive rule as a comment (src/fit_tsne.cu:435):
+ * max(min_num_intervals, (max_coord - min_coord) / intervals_per_integer), rounded up in
+ * that list.  tsne_hip_boxes_for_spread applies that rule (125 and 1) to a coordinate
+ * spread and returns 130, 140, 150 or - past the list entries the 1024-point transforms
+ * can hold - 170; tsne_hip_plan_set_boxes makes a plan use a size in [2, 170] from its
+ * next step on (it waits for the device and drops captured steps when the size changes). */
+int tsne_hip_plan_set_boxes(tsne_hip_plan *plan, int n_boxes_per_dim);
+int tsne_hip_boxes_for_spread(float spread);
 
 /* Whether a kernel of this plan has reported trouble since the last call (no
  * counterpart in the reference).  Call it after synchronising the streams the

@@ -70,6 +70,22 @@ def knn(X, K, rows=None):
     return idx, d2
 
 
+def knn_ivf(X, K, centroids, nprobe, return_probes=False):
+    """The library's approximate (inverted-file) search: (idx, d2[, list of every point, probes of every
+    list]) in the caller's numbering."""
+    X = np.ascontiguousarray(X, np.float32)
+    centroids = np.ascontiguousarray(centroids, np.float32)
+    N, D = X.shape
+    nlist = centroids.shape[0]
+    idx = np.empty((N, K), np.int32)
+    d2 = np.empty((N, K), np.float32)
+    list_of = np.empty(N, np.int32)
+    probes = np.empty((nlist, nprobe), np.int32)
+    lib().oracle_knn_ivf(_opt(X), N, D, K, _opt(centroids), nlist, nprobe, _opt(idx), _opt(d2), _opt(list_of),
+                         _opt(probes))
+    return (idx, d2, list_of, probes) if return_probes else (idx, d2)
+
+
 def max_normalize(d2):
     out = np.array(d2, np.float32, copy=True, order="C")
     m = lib().oracle_max_normalize(_opt(out), ctypes.c_int64(out.size))

@@ -9,6 +9,7 @@
 //
 //   oracle_knn            exact kNN that stands in for the FAISS call at
 //                         src/util/distance_utils.cu:79-121 (definition below)
+//   oracle_knn_ivf        the library's approximate (inverted-file) search, structured as the FAISS call above
 //   oracle_max_normalize  src/util/math_utils.cu:66-74
 //   oracle_perplexity     src/kernels/perplexity_search.cu:10-141
 //   oracle_symmetrize     src/util/math_utils.cu:269-308
@@ -22,6 +23,8 @@
 //
 // Pinning status (what fixes each function independently of this file):
 //   knn         brute force over numpy float32 arithmetic + sklearn brute kNN
+//   knn_ivf     a numpy restatement of the candidate rule on small inputs; with every list probed it must
+//               reduce to the exact search; recall against the exact search
 //   max_norm    closed form
 //   perplexity  row sums, entropy target, uniform closed form, sklearn bisection;
 //               its exp / log against double-precision exp / log (<= 2 units in the last place),
@@ -270,6 +273,97 @@ void oracle_knn_rows(const float *X, int N, int D, int K, int row_begin, int row
 
 void oracle_knn(const float *X, int N, int D, int K, int *idx, float *d2) {
     oracle_knn_rows(X, N, D, K, 0, N, idx, d2);
+}
+
+// Approximate neighbours through an inverted file: the library's approximate mode, which keeps the structure
+// and parameters of the reference's FAISS IndexIVFFlat search (src/util/distance_utils.cu:85-120: nlist lists,
+// nprobe probed, L2) - FAISS itself is not among the reference's sources (un-vendored, v1.9.0), so this restates
+// the library's documented rule, and what it is held to is that rule plus its recall against the exact search:
+//   * every point is filed under its nearest centroid, by (distance, list number), distances accumulated as in
+//     the exact search (one fma per dimension);
+//   * a list probes the nprobe lists whose centroids are nearest to its own centroid (same order; itself
+//     first), and a point probes what its list probes;
+//   * the points are renumbered list by list, old numbers ascending inside a list; tiles are runs of 128
+//     consecutive new numbers;
+//   * the candidates of a query are the points of its tile's 8 neighbours either side in the numbering and of
+//     every tile that overlaps a list probed by the list of some query of its tile;
+//   * among them the K - 1 nearest by (distance, new number), the query itself first.
+// Output in the caller's (old) numbering.  list_out (optional): N list numbers; list_probes_out (optional):
+// nlist x nprobe.
+void oracle_knn_ivf(const float *X, int N, int D, int K, const float *centroids, int nlist, int nprobe, int *idx_out,
+                    float *d2_out, int *list_out, int *list_probes_out) {
+    auto nearest = [&](const float *q, int count, int *out) {
+        std::vector<Cand> all(nlist);
+        for (int c = 0; c < nlist; ++c) {
+            float acc = 0.0f;
+            for (int d = 0; d < D; ++d) {
+                const float df = q[d] - centroids[(size_t)c * D + d];
+                acc = std::fmaf(df, df, acc);
+            }
+            all[c] = Cand{acc, c};
+        }
+        std::partial_sort(all.begin(), all.begin() + count, all.end(), cand_less);
+        for (int r = 0; r < count; ++r) out[r] = all[r].j;
+    };
+    std::vector<int> list_of(N), lprobes((size_t)nlist * nprobe);
+#pragma omp parallel for schedule(static)
+    for (int i = 0; i < N; ++i) nearest(X + (size_t)i * D, 1, &list_of[i]);
+#pragma omp parallel for schedule(static)
+    for (int l = 0; l < nlist; ++l) nearest(centroids + (size_t)l * D, nprobe, &lprobes[(size_t)l * nprobe]);
+    if (list_out) std::memcpy(list_out, list_of.data(), list_of.size() * sizeof(int));
+    if (list_probes_out) std::memcpy(list_probes_out, lprobes.data(), lprobes.size() * sizeof(int));
+    std::vector<int> order(N);
+    for (int i = 0; i < N; ++i) order[i] = i;
+    std::stable_sort(order.begin(), order.end(),
+                     [&](int a, int b) { return list_of[a] < list_of[b]; });
+    std::vector<int> list_start(nlist + 1, 0);
+    for (int i = 0; i < N; ++i) list_start[list_of[i] + 1] += 1;
+    for (int l = 0; l < nlist; ++l) list_start[l + 1] += list_start[l];
+    const int T = (N + 127) / 128;
+#pragma omp parallel
+    {
+        std::vector<char> probed(nlist), visit(T);
+        std::vector<Cand> cands;
+#pragma omp for schedule(dynamic, 1)
+        for (int qt = 0; qt < T; ++qt) {
+            std::fill(probed.begin(), probed.end(), 0);
+            std::fill(visit.begin(), visit.end(), 0);
+            const int q0 = qt * 128, q1 = std::min(N, q0 + 128);
+            for (int r = q0; r < q1; ++r)
+                for (int s = 0; s < nprobe; ++s) probed[lprobes[(size_t)list_of[order[r]] * nprobe + s]] = 1;
+            for (int t = std::max(0, qt - 8); t <= std::min(T - 1, qt + 8); ++t) visit[t] = 1;
+            for (int l = 0; l < nlist; ++l)
+                if (probed[l] && list_start[l + 1] > list_start[l])
+                    for (int t = list_start[l] / 128; t <= (list_start[l + 1] - 1) / 128; ++t) visit[t] = 1;
+            for (int r = q0; r < q1; ++r) {
+                const float *xq = X + (size_t)order[r] * D;
+                cands.clear();
+                for (int t = 0; t < T; ++t) {
+                    if (!visit[t]) continue;
+                    for (int c = t * 128; c < std::min(N, t * 128 + 128); ++c) {
+                        if (c == r) continue;
+                        const float *xc = X + (size_t)order[c] * D;
+                        float acc = 0.0f;
+                        for (int d = 0; d < D; ++d) {
+                            const float df = xq[d] - xc[d];
+                            acc = std::fmaf(df, df, acc);
+                        }
+                        cands.push_back(Cand{acc, c});
+                    }
+                }
+                const int keep = std::min<int>(K - 1, (int)cands.size());
+                std::partial_sort(cands.begin(), cands.begin() + keep, cands.end(), cand_less);
+                int *oi = idx_out + (size_t)order[r] * K;
+                float *od = d2_out + (size_t)order[r] * K;
+                oi[0] = order[r];
+                od[0] = 0.0f;
+                for (int s = 1; s < K; ++s) {
+                    oi[s] = s - 1 < keep ? order[cands[s - 1].j] : -1;
+                    od[s] = s - 1 < keep ? cands[s - 1].d : INFINITY;
+                }
+            }
+        }
+    }
 }
 
 // src/util/math_utils.cu:66-74: divide every entry by the largest absolute value.

@@ -256,6 +256,57 @@ def test_fit_with_full_symmetrisation(c0_problem, monkeypatch, capfd):
     assert abs(full.kl_divergence_ - kl) <= 0.01 * kl
 
 
+def test_fit_with_approximate_neighbours(monkeypatch, capfd):
+    """TSNE_KNN=ivf: the neighbour search through the inverted file (floor(sqrt(N)) lists, as the
+    reference's FAISS index).  The embedding of clustered data is as trustworthy as with exact neighbours."""
+    from tsnecuda import TSNE, synthetic
+    X, fit = synthetic.make_config("c3", n=40000)
+    Y0 = synthetic_start(X.shape[0])
+    kw = dict(perplexity=30.0, num_neighbors=90, n_iter=400, perplexity_epsilon=1e-4)
+    exact = TSNE(**kw)
+    exact.fit_transform(X, y=Y0)
+    t_exact = exact.trustworthiness(12)
+    monkeypatch.setenv("TSNE_KNN", "ivf")
+    monkeypatch.setenv("TSNE_KNN_NPROBE", "40")
+    approx = TSNE(verbose=1, print_interval=200, **kw)
+    emb = approx.fit_transform(X, y=Y0)
+    out = capfd.readouterr().out
+    assert "(inverted file: 200 lists, 40 probed per list, " in out
+    per_mille = int(out.split("probed per list, ")[1].split(" per mille")[0])
+    assert 0 < per_mille < 600
+    assert np.isfinite(emb).all()
+    t_approx = approx.trustworthiness(12)
+    print("trustworthiness: exact neighbours %.4f, inverted file %.4f" % (t_exact, t_approx))
+    assert t_approx >= t_exact - 0.03
+
+
+def test_fit_with_adaptive_grid(monkeypatch, capfd):
+    """TSNE_ADAPTIVE_BOXES=1: every 50 steps the grid follows the spread of the embedding.  From a start that
+    is 160 units wide the first check moves from 130 to 170 boxes; the interpolation error of the repulsive
+    forces reported then is lower than with the reference's fixed grid."""
+    from tsnecuda import TSNE, synthetic
+    X, fit = synthetic.make_config("c0")
+    n = X.shape[0]
+    Y0 = (np.random.default_rng(2).random((n, 2)) * 160.0 - 80.0).astype(np.float32)
+    monkeypatch.setenv("TSNE_REPULSION_MONITOR", "400")
+    kw = dict(perplexity=30.0, num_neighbors=90, n_iter=101, verbose=1, print_interval=100, early_exaggeration=1.0,
+              learning_rate=1.0, perplexity_epsilon=1e-4)
+
+    def monitored_error():
+        TSNE(**kw).fit_transform(X, y=Y0)
+        out = capfd.readouterr().out
+        line = [l for l in out.split("\n") if l.startswith("[Step 100] Repulsion interpolation error")][0]
+        return out, float(line.split("forces ")[1].split(",")[0])
+
+    out_fixed, err_fixed = monitored_error()
+    assert "Interpolation grid" not in out_fixed
+    monkeypatch.setenv("TSNE_ADAPTIVE_BOXES", "1")
+    out_adaptive, err_adaptive = monitored_error()
+    assert "[Step 50] Interpolation grid: 170 boxes per dimension (spread " in out_adaptive
+    print("repulsion error at step 100: fixed grid %.3g, adaptive %.3g" % (err_fixed, err_adaptive))
+    assert err_adaptive < err_fixed
+
+
 def synthetic_start(n):
     from tsnecuda import synthetic
     return synthetic.initial_embedding(n)

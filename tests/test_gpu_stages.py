@@ -262,6 +262,44 @@ def test_iterate_with_recentring(stages, c0_problem, prepared):
     plan.close()
 
 
+def test_grid_size_changes_between_steps(stages, c0_problem):
+    """The plan's interpolation grid can change between steps (the adaptive rule the reference carries
+    as a comment, src/fit_tsne.cu:435): after every change the repulsive forces and fused steps follow the
+    oracle run with that grid size - growing, shrinking (nothing of the larger grid may leak into the
+    smaller one) and back to the reference's 130."""
+    c = c0_problem
+    n = c["X"].shape[0]
+    rng = np.random.default_rng(21)
+    y = (rng.standard_normal(2 * n) * 20).astype(np.float32)
+    plan = stages.Plan(n, c["K"])
+    dy = dev(y)
+    for nb in (130, 150, 36, 170, 130):
+        plan.set_boxes(nb)
+        rep, z, w, yt, phi = plan.repulsive(dy, details=True)
+        rep_o, z_o, w_o, yt_o, phi_o = oracle.repulsive(y, nb=nb, details=True)
+        assert w.shape == w_o.shape
+        assert rel_l2(rep.cpu().numpy(), rep_o) <= 1e-4, nb
+        assert abs(float(z) - z_o) <= 1e-5 * abs(z_o), nb
+    dP, di = dev(c["P"]), dev(c["idx"])
+    plan.prepare_attractive(dP, di)
+    y0 = c["y0"]
+    dy = dev(y0)
+    gains, old = torch.ones_like(dy), torch.zeros_like(dy)
+    plan.iterate_(None, None, dy, gains, old, 0, 4)          # captured or not: 130 boxes
+    plan.set_boxes(140)
+    plan.iterate_(None, None, dy, gains, old, 4, 8)          # the same steps must not replay the old grid
+    g_h, o_h = np.ones(2 * n, np.float32), np.zeros(2 * n, np.float32)
+    y_o, _ = oracle.iterate(c["P"], c["idx"], y0, 4, gains=g_h, old_forces=o_h)
+    y_o, _ = oracle.iterate(c["P"], c["idx"], y_o, 4, step_begin=4, gains=g_h, old_forces=o_h, nb=140)
+    assert rel_l2(dy.cpu().numpy(), y_o) <= 1e-4
+    with pytest.raises(RuntimeError, match="n_boxes_per_dim must be"):
+        plan.set_boxes(171)
+    plan.close()
+    # the rule: 125 boxes at least -> 130 in the reference's list; one box per unit of spread above that
+    assert [stages.boxes_for_spread(s) for s in (0.0, 10.0, 125.0, 130.0, 130.5, 140.0, 149.9, 150.1, 1e6,
+                                                 float("nan"))] == [130, 130, 130, 130, 140, 140, 150, 170, 170, 130]
+
+
 @pytest.mark.parametrize("n,d,k,perp", [
     (2, 2, 2, 1.5),         # smallest problem: self plus one neighbour
     (50, 3, 50, 10.0),      # K == N, fewer points than one candidate tile
@@ -636,6 +674,43 @@ def test_knn_tile_skipping_is_exact(stages, scale, d):
         idx_o, d2_o = oracle.knn(Xs_h, k, rows=(first, first + 96))
         assert np.array_equal(idx_v[first:first + 96].cpu().numpy(), idx_o)
         assert np.array_equal(d2_v[first:first + 96].cpu().numpy(), d2_o)
+
+
+@pytest.mark.parametrize("n,d,k,nlist,nprobe", [(20000, 16, 30, 141, 20), (9000, 50, 90, 94, 5), (30000, 3, 10, 173, 1), (40000, 50, 90, 200, 60)])
+def test_knn_ivf_matches_the_oracle_given_the_centroids(stages, n, d, k, nlist, nprobe):
+    """The approximate (inverted-file) search: centroids trained on the GPU, then - the centroids given - the
+    search is a deterministic function of the points, which the oracle restates: identical neighbours and
+    distances, bit for bit.  Recall against the exact search is reported and bounded."""
+    from tsnecuda import synthetic
+    X = synthetic.gaussian_clusters(n, d=d, clusters=6, center_scale=4.0, seed=n + d)
+    dX = dev(X)
+    cen = stages.ivf_train(dX, nlist)
+    cen_h = cen.cpu().numpy()
+    assert cen_h.shape == (nlist, d) and np.isfinite(cen_h).all()
+    # trained centroids describe the data better than the points they started from would: every list is used
+    idx, d2, stats = stages.knn_ivf(dX, k, cen, nprobe)
+    assert stats[0] == 1 and stats[1] == 0  # matrix sweep, no query answered by the exact fallback
+    idx_o, d2_o, list_of, probes = oracle.knn_ivf(X, k, cen_h, nprobe, return_probes=True)
+    assert np.array_equal(idx.cpu().numpy(), idx_o)
+    assert np.array_equal(d2.cpu().numpy().view(np.uint32), d2_o.view(np.uint32))
+    assert np.unique(list_of).size > 0.8 * nlist
+    exact, _ = stages.knn(dX, k)
+    exact = exact.cpu().numpy()
+    got = idx.cpu().numpy()
+    recall = np.mean([len(np.intersect1d(got[i, 1:], exact[i, 1:])) for i in range(0, n, 7)]) / (k - 1)
+    print("knn_ivf n=%d d=%d nlist=%d nprobe=%d: recall %.4f, %d per mille of the tile pairs" % (n, d, nlist, nprobe,
+                                                                                                recall, stats[2]))
+    assert recall > (0.6 if nprobe >= 5 else 0.4)
+
+
+def test_knn_ivf_argument_errors(stages):
+    X = dev(np.random.default_rng(0).standard_normal((9000, 8)).astype(np.float32))
+    cen = stages.ivf_train(X, 30)
+    with pytest.raises(RuntimeError, match="nprobe must be"):
+        stages.knn_ivf(X, 10, cen, 31)
+    wide = dev(np.zeros((9000, 200), np.float32))
+    with pytest.raises(RuntimeError, match="at most 12"):
+        stages.ivf_train(wide, 30)
 
 
 def test_knn_chunked_sweep_calibrates_its_margin(stages):

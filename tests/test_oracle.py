@@ -82,6 +82,50 @@ def test_knn_ties_and_duplicates():
     assert np.array_equal(sub_idx, idx[2:5]) and np.array_equal(sub_d2, d2[2:5])
 
 
+def test_knn_ivf_rule_and_limits():
+    """The approximate search's restatement: with every list probed it is the exact search; with few lists
+    probed its candidate rule is what a numpy restatement of the rule gives; recall grows with nprobe."""
+    rng = np.random.default_rng(5)
+    n, d, k, nlist = 1500, 6, 12, 24
+    X = synthetic.gaussian_clusters(n, d=d, clusters=5, center_scale=3.0, seed=11)
+    cen = X[rng.choice(n, nlist, replace=False)].copy()
+    exact_idx, exact_d = oracle.knn(X, k)
+    idx_all, d_all = oracle.knn_ivf(X, k, cen, nlist)
+    # ties aside (none in this data), probing everything is the exact search
+    assert np.array_equal(idx_all, exact_idx) and np.array_equal(d_all, exact_d)
+    recalls = []
+    for nprobe in (1, 3, 8):
+        idx, d2, list_of, probes = oracle.knn_ivf(X, k, cen, nprobe, return_probes=True)
+        # a point's list: its nearest centroid; a list's probes: the centroids nearest to its own (itself
+        # first) - numpy, float64, away from ties
+        dc = ((X[:, None, :].astype(np.float64) - cen[None].astype(np.float64)) ** 2).sum(-1)
+        assert np.array_equal(list_of, dc.argmin(1))
+        cc = ((cen[:, None, :].astype(np.float64) - cen[None].astype(np.float64)) ** 2).sum(-1)
+        assert np.array_equal(probes[:, 0], np.arange(nlist))
+        assert np.array_equal(np.sort(probes, 1), np.sort(np.argsort(cc, 1)[:, :nprobe], 1))
+        # the candidate rule, restated: renumber by (list, old number), 128-point tiles, a query's candidates
+        order = np.lexsort((np.arange(n), list_of))
+        lists_sorted = list_of[order]
+        T = (n + 127) // 128
+        for r in rng.choice(n, 40, replace=False):  # r: a new number
+            qt = r // 128
+            mates = order[qt * 128:min(n, qt * 128 + 128)]
+            probed = np.unique(probes[list_of[mates]])
+            tiles = set(range(max(0, qt - 8), min(T - 1, qt + 8) + 1))
+            for l in probed:
+                members = np.flatnonzero(lists_sorted == l)
+                if members.size:
+                    tiles.update(range(members[0] // 128, members[-1] // 128 + 1))
+            cand = np.array([c for c in range(n) if c // 128 in tiles and c != r])
+            dd = ((X[order[r]].astype(np.float64) - X[order[cand]].astype(np.float64)) ** 2).sum(1)
+            best = cand[np.lexsort((cand, dd))[:k - 1]]
+            assert np.array_equal(idx[order[r], 1:], order[best])
+            assert idx[order[r], 0] == order[r] and d2[order[r], 0] == 0.0
+        hits = sum(len(np.intersect1d(idx[i, 1:], exact_idx[i, 1:])) for i in range(n))
+        recalls.append(hits / (n * (k - 1)))
+    assert recalls[0] <= recalls[1] <= recalls[2] and recalls[2] > 0.9
+
+
 def test_max_normalize(small):
     dn, dmax, d2 = small["dn"], small["dmax"], small["d2"]
     assert dmax == d2.max()

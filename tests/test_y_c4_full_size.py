@@ -80,6 +80,32 @@ def test_c4_order_and_knn_rows_bit_exact(c4):
     for b in range(0, N, 2000000):  # distinct neighbours per row (sorted in slabs: a full sort needs 7 GB more)
         srt = torch.sort(idx[b:b + 2000000], dim=1).values
         assert bool((srt[:, 1:] != srt[:, :-1]).all())
+    # The approximate search on the same points (inverted file, floor(sqrt(N)) = 3162 lists as the reference's
+    # FAISS index, 100 lists probed per list): its time, its recall against the exact rows, and what must hold
+    # of any subset search - rank by rank no neighbour is nearer than the exact one, and a row that found the
+    # exact neighbours reports the exact distances.
+    st = c4["stages"]
+    dXs = torch.from_numpy(c4["Xs"]).cuda()
+    torch.cuda.synchronize()
+    t0 = time.time()
+    cen = st.ivf_train(dXs, 3162)
+    torch.cuda.synchronize()
+    t1 = time.time()
+    idx_a, d2_a, stats_a = st.knn_ivf(dXs, K, cen, 100)
+    torch.cuda.synchronize()
+    t2 = time.time()
+    del dXs
+    sample = torch.arange(0, N, N // 20000, device="cuda")[:20000]
+    found = (idx_a[sample, 1:, None] == idx[sample, None, 1:]).any(2)
+    recall = float(found.float().mean())
+    print("c4 approximate kNN: train %.2f s, search %.2f s, %d per mille of the tile pairs, recall@%d %.4f"
+          % (t1 - t0, t2 - t1, stats_a[2], K - 1, recall), flush=True)
+    assert stats_a[0] == 1 and stats_a[1] == 0 and recall > 0.25
+    assert torch.equal(idx_a[:, 0], torch.arange(N, device="cuda", dtype=torch.int32))
+    assert bool((d2_a[sample] >= d2[sample]).all())
+    whole = found.all(1)
+    assert bool((d2_a[sample][whole] == d2[sample][whole]).all())
+    del idx_a, d2_a
     c4.pop("Xs")
 
 

@@ -320,7 +320,8 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
     p->n_nodes = n_boxes_per_dim * kInterp;
     p->device = device;
     p->lagrange = make_lagrange();
-    const size_t G2 = (size_t)p->n_nodes * p->n_nodes;
+    // The grid buffers hold the largest grid: tsne_hip_plan_set_boxes may change the size between steps.
+    const size_t G2 = (size_t)(kMaxBoxes * kInterp) * (kMaxBoxes * kInterp);
     const size_t spec = (size_t)2 * kFft * kNodePad;
     const size_t N = (size_t)num_points;
     p->max_chunks = (int)(N / kChunkPoints) + kMaxTiles + 1;
@@ -543,6 +544,34 @@ int tsne_hip_plan_set_recenter(tsne_hip_plan *plan, int enable) {
     }
     plan->recenter = enable != 0;
     return 0;
+}
+
+int tsne_hip_plan_set_boxes(tsne_hip_plan *plan, int n_boxes_per_dim) {
+    if (check_plan(plan, "plan_set_boxes")) return 1;
+    TSNE_REQUIRE(n_boxes_per_dim >= 2 && n_boxes_per_dim <= kMaxBoxes,
+                 "plan_set_boxes: n_boxes_per_dim must be in [2, %d] (got %d)", kMaxBoxes, n_boxes_per_dim);
+    if (n_boxes_per_dim == plan->n_boxes) return 0;
+    // Nothing of the old grid survives a step: the charges are cleared by the pass that consumes them, every
+    // other grid buffer is written before it is read, and all of them are sized for the largest grid.
+    // Captured steps carry the grid size as kernel arguments and launch shapes.
+    TSNE_TRY(hipSetDevice(plan->device));
+    TSNE_TRY(hipDeviceSynchronize());
+    for (auto &g : plan->step_graphs) (void)hipGraphExecDestroy(g.exec);
+    plan->step_graphs.clear();
+    plan->n_boxes = n_boxes_per_dim;
+    plan->n_nodes = n_boxes_per_dim * kInterp;
+    return 0;
+}
+
+int tsne_hip_boxes_for_spread(float spread) {
+    // src/fit_tsne.cu:248-266 (the list of grid sizes) and :435 (the rule, commented out there; FIt-SNE's
+    // max(min_num_intervals, spread / intervals_per_integer) with 125 and 1).
+    static const int allowed[] = {25, 36, 50, 55, 60, 65, 70, 75, 80, 85, 90, 96, 100, 110, 120, 130, 140, 150};
+    float want = 125.0f;
+    if (spread == spread && spread > want) want = spread;  // (a NaN spread keeps the minimum)
+    for (int a : allowed)
+        if ((float)a >= want) return a;
+    return kMaxBoxes;  // the transform length ends the list here (its next entries: 175, 200, 1125)
 }
 
 int tsne_hip_plan_check(tsne_hip_plan *plan) {

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <cstring>
 #include <cstdio>
 #include <cstdlib>
 
@@ -38,6 +39,14 @@ bool sync_kernels_enabled();
 inline int div_up(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
 constexpr int kWave = 64;
+
+// Host-side inverse of the order-preserving float -> uint32 map below.
+inline float ordered_to_float_host(unsigned int u) {
+    const unsigned int bits = (u & 0x80000000u) ? (u & 0x7fffffffu) : ~u;
+    float f;
+    std::memcpy(&f, &bits, sizeof(f));
+    return f;
+}
 
 #ifdef __HIPCC__
 // Order-preserving map between float and uint32 so min/max can use integer atomics.

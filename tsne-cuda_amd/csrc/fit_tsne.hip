@@ -174,8 +174,25 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     clock.start();
     if (verbose) std::cout << "done.\nKNN Computation... " << std::flush;
     DeviceBuffer d_idx(sizeof(int) * nnz), d_dist(sizeof(float) * nnz), d_scratch(sizeof(float));
-    TSNE_OR_DIE(tsnehip::run_knn(d_points.as<float>(), N, D, K, d_idx.as<int>(), d_dist.as<float>(), stream),
-                "kNN");
+    // Exact by default.  Options::approximate_neighbors or TSNE_KNN=ivf: inverted file with floor(sqrt(N)) lists,
+    // as the reference's FAISS search (src/util/distance_utils.cu:85-120); wider inputs than it takes stay exact.
+    const char *knn_env = std::getenv("TSNE_KNN");
+    const bool approximate = (opt.approximate_neighbors || (knn_env && std::string(knn_env) == "ivf")) && D <= 126 &&
+                             N >= 4096;
+    if (approximate) {
+        int nprobe = env_int("TSNE_KNN_NPROBE", opt.knn_nprobe);
+        if (nprobe <= 0) nprobe = 100;
+        int nlist = 0, knn_stats[3] = {0, 0, 0};
+        TSNE_OR_DIE(tsnehip::run_knn_approximate(d_points.as<float>(), N, D, K, nprobe, d_idx.as<int>(),
+                                                 d_dist.as<float>(), &nlist, knn_stats, stream),
+                    "approximate kNN");
+        if (verbose)
+            std::cout << "(inverted file: " << nlist << " lists, " << std::min(nprobe, nlist) << " probed per list, "
+                      << knn_stats[2] << " per mille of the tile pairs compared) " << std::flush;
+    } else {
+        TSNE_OR_DIE(tsnehip::run_knn(d_points.as<float>(), N, D, K, d_idx.as<int>(), d_dist.as<float>(), stream),
+                    "kNN");
+    }
     d_points.release();
     TSNE_OR_DIE(tsnehip::launch_max_normalize(d_dist.as<float>(), (int64_t)nnz, d_scratch.as<float>(), stream),
                 "max-normalisation");
@@ -303,6 +320,10 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     const bool want_snap = opt.return_style == RETURN_STYLE::SNAPSHOT && opt.return_data != nullptr;
     const bool want_stop = opt.min_gradient_norm > 0.0f;
     const int monitor_points = verbose ? env_int("TSNE_REPULSION_MONITOR", 0) : 0;
+    // Options::adaptive_boxes or TSNE_ADAPTIVE_BOXES=1: every kGridCheckSteps steps the grid follows the spread
+    // of the embedding (src/fit_tsne.cu:435, commented out in the reference, which keeps 130 boxes).
+    const bool adaptive_boxes = opt.adaptive_boxes || env_int("TSNE_ADAPTIVE_BOXES", 0) != 0;
+    constexpr size_t kGridCheckSteps = 50;
     hipEvent_t ev[4];
     if (verbose)
         for (auto &e : ev) hip_or_die(hipEventCreate(&e), "event creation");
@@ -323,6 +344,19 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         const bool printing = verbose && step % print_interval == 0;
         const bool timing = printing;  // phase timers sample the steps that already synchronise
 
+        if (adaptive_boxes && step > 0 && step % kGridCheckSteps == 0) {
+            unsigned int enc[4];  // min_enc[2], max_enc[2]: the bounds the next step will use are in `slot`
+            hip_or_die(hipStreamSynchronize(stream), "grid size");
+            hip_or_die(hipMemcpy(enc, plan->scalars, sizeof(enc), hipMemcpyDeviceToHost), "grid size");
+            const float spread = tsnehip::ordered_to_float_host(enc[2 + slot]) - tsnehip::ordered_to_float_host(enc[slot]);
+            const int boxes = tsne_hip_boxes_for_spread(spread);
+            if (boxes != plan->n_boxes) {
+                if (verbose)
+                    std::cout << "[Step " << step << "] Interpolation grid: " << boxes << " boxes per dimension (spread "
+                              << spread << ")" << std::endl;
+                TSNE_OR_DIE(tsne_hip_plan_set_boxes(plan, boxes), "grid size");
+            }
+        }
         const bool want_norm = step + 1 == iterations || want_stop;
         if (!verbose && !want_stop && !want_dump && !want_snap) {
             // Nothing looks at the steps in between: everything up to the schedule switch, or up to the last
@@ -332,6 +366,7 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
             size_t run_end = iterations - 1;
             if (!late && opt.force_magnify_iters >= 0)
                 run_end = std::min(run_end, (size_t)opt.force_magnify_iters);
+            if (adaptive_boxes) run_end = std::min(run_end, (step / kGridCheckSteps + 1) * kGridCheckSteps);
             if (run_end > step + 1) {
                 const size_t count = std::min<size_t>(run_end - step, 1u << 30);
                 hipStream_t batch_stream = plan->loop_stream;

@@ -42,6 +42,7 @@
 //    every tile's candidates over several workgroups; a merge kernel reduces
 //    their lists to what a single list would have kept.
 #include "common.h"
+#include "stages.h"
 
 #include <algorithm>
 #include <climits>
@@ -614,6 +615,13 @@ struct SweepArgs {
     int parts;
     u64 *part_keys;
     int select_slack;  // entries beyond `want` a compaction in mid-sweep may keep (see wave_select)
+    // Approximate search (register-resident sweep only; null = exact): the points are numbered list by list of
+    // an inverted file, and after its neighbourhood in the numbering a query tile only visits the tiles that
+    // overlap the lists some query of the tile probes.  probe_tile_lists: per query tile a bitmap over the
+    // lists (probe_list_words words); probe_list_tiles: first and last tile of every list (first > last: empty).
+    const unsigned int *probe_tile_lists;
+    int probe_list_words, probe_nlist;
+    const int *probe_list_tiles;
 };
 
 // ---------------------------------------------------------------------------
@@ -909,9 +917,24 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                 __syncthreads();
                 const float tmax = fmaxf(tmax_part[0], tmax_part[1]);
                 const float ra = args.radius[qt];
-                for (int t = tid; t < T; t += 256)
-                    if ((t < h0 || t > h1) && tile_may_matter(qcenter, ra, args.centers_t, args.radius, D, T, t, tmax))
-                        atomicOr(&bitmap[t >> 5], 1u << (t & 31));
+                if (args.probe_tile_lists) {
+                    // Approximate search: only tiles of probed lists are eligible (the ball test still drops
+                    // those among them that cannot matter, which changes nothing in the result).
+                    const unsigned int *mine = args.probe_tile_lists + (size_t)qt * args.probe_list_words;
+                    for (int l = tid; l < args.probe_nlist; l += 256) {
+                        if (!((mine[l >> 5] >> (l & 31)) & 1u)) continue;
+                        const int t0 = args.probe_list_tiles[2 * l], t1 = args.probe_list_tiles[2 * l + 1];
+                        for (int t = t0; t <= t1; ++t)
+                            if ((t < h0 || t > h1) &&
+                                tile_may_matter(qcenter, ra, args.centers_t, args.radius, D, T, t, tmax))
+                                atomicOr(&bitmap[t >> 5], 1u << (t & 31));
+                    }
+                } else {
+                    for (int t = tid; t < T; t += 256)
+                        if ((t < h0 || t > h1) &&
+                            tile_may_matter(qcenter, ra, args.centers_t, args.radius, D, T, t, tmax))
+                            atomicOr(&bitmap[t >> 5], 1u << (t & 31));
+                }
                 __syncthreads();
                 nxt = next_tile();
                 if (nxt >= 0) {
@@ -1489,7 +1512,7 @@ int run_valu_sweep(const float *points, const float *Xt, int N, int Npad, int D,
 // stats (optional, 3 ints): [0] = 1 if the matrix-instruction sweep ran, [1] = queries redone by the VALU sweep,
 // [2] = per mille of the (query tile, candidate tile) pairs the matrix sweep computed.
 int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s, int mode,
-                 int *stats) {
+                 int *stats, const KnnProbes *probes) {
     if (stats) stats[0] = stats[1] = stats[2] = 0;
     if (N <= 0 || D <= 0 || K <= 0) {
         set_error("knn: num_points, num_dims and num_neighbors must be positive (got %d, %d, %d)", N, D, K);
@@ -1541,6 +1564,11 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     bool use_mfma = mode == 2 || (mode == 0 && mfma_fits && N >= 8192);
     if (mode == 2 && !mfma_fits) {
         set_error("knn: the matrix-instruction sweep does not fit %d dimensions / %d neighbours", D, K);
+        return 1;
+    }
+    if (probes && (!use_mfma || chunked)) {
+        set_error("knn: the approximate search runs on the register-resident matrix sweep only (at most 126 "
+                  "dimensions; got %d dimensions, %d neighbours)", D, K);
         return 1;
     }
 
@@ -1637,6 +1665,10 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         args.qtile_step = step;
         args.parts = parts;
         args.part_keys = part_keys.as<u64>();
+        args.probe_tile_lists = probes ? probes->tile_lists : nullptr;
+        args.probe_list_words = probes ? probes->list_words : 0;
+        args.probe_nlist = probes ? probes->nlist : 0;
+        args.probe_list_tiles = probes ? probes->list_tiles : nullptr;
         if (chunked) {
             const size_t lds = sweep_lds(keep);
             TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_chunked_sweep_kernel),
@@ -1733,7 +1765,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
 }
 
 int run_knn(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s) {
-    return run_knn_mode(points, N, D, K, indices, sq_dist, s, 0, nullptr);
+    return run_knn_mode(points, N, D, K, indices, sq_dist, s, 0, nullptr, nullptr);
 }
 
 }  // namespace tsnehip

@@ -8,10 +8,9 @@
 
 #include "../../include/tsnecuda/tsne_stages.h"
 #include "plan.h"
+#include "stages.h"
 
 namespace tsnehip {
-
-namespace {
 
 // `count` distinct pseudo-random indices below n, ascending: a full-period linear congruential sequence modulo
 // the next power of two, values >= n skipped (a permutation of [0, 2^b), so no index repeats).
@@ -34,6 +33,8 @@ std::vector<int> sample_indices(int n, int count, unsigned int seed) {
     std::sort(out.begin(), out.end());
     return out;
 }
+
+namespace {
 
 struct DeviceArray {
     void *ptr = nullptr;

@@ -26,6 +26,10 @@ def lib():
         L.tsne_hip_knn.argtypes = [_vp, c_int, c_int, c_int, _vp, _vp, _vp]
         L.tsne_hip_knn_select.argtypes = [_vp, c_int, c_int, c_int, _vp, _vp, _vp, c_int, ctypes.POINTER(c_int)]
         L.tsne_hip_knn_select.restype = c_int
+        L.tsne_hip_ivf_train.argtypes = [_vp, c_int, c_int, c_int, c_int, _vp, _vp]
+        L.tsne_hip_ivf_train.restype = c_int
+        L.tsne_hip_knn_ivf.argtypes = [_vp, c_int, c_int, c_int, _vp, c_int, c_int, _vp, _vp, _vp, ctypes.POINTER(c_int)]
+        L.tsne_hip_knn_ivf.restype = c_int
         L.tsne_hip_locality_order.argtypes = [_vp, c_int, c_int, _vp, _vp]
         L.tsne_hip_gather_rows.argtypes = [_vp, _vp, c_int, c_int, _vp, _vp]
         L.tsne_hip_max_normalize.argtypes = [_vp, c_i64, _vp]
@@ -43,6 +47,10 @@ def lib():
         L.tsne_hip_plan_check.argtypes = [_vp]
         L.tsne_hip_plan_set_recenter.argtypes = [_vp, c_int]
         L.tsne_hip_plan_set_recenter.restype = c_int
+        L.tsne_hip_plan_set_boxes.argtypes = [_vp, c_int]
+        L.tsne_hip_plan_set_boxes.restype = c_int
+        L.tsne_hip_boxes_for_spread.argtypes = [c_float]
+        L.tsne_hip_boxes_for_spread.restype = c_int
         L.tsne_hip_plan_destroy.argtypes = [_vp]
         L.tsne_hip_plan_destroy.restype = None
         L.tsne_hip_attractive.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp]
@@ -109,6 +117,28 @@ def knn_select(points, num_neighbors, sweep):
     return idx, dist, (int(stats[0]), int(stats[1]), int(stats[2]))
 
 
+def ivf_train(points, nlist, iterations=10):
+    """nlist k-means centroids (nlist x D) for the inverted-file search."""
+    points = _f32(points)
+    n, d = points.shape
+    centroids = torch.empty((nlist, d), dtype=torch.float32, device=points.device)
+    _check(lib().tsne_hip_ivf_train(_ptr(points), n, d, nlist, iterations, _ptr(centroids), _stream()))
+    return centroids
+
+
+def knn_ivf(points, num_neighbors, centroids, nprobe=20):
+    """Approximate neighbours through the inverted file given by `centroids`.
+    Returns (indices, sq_dist, stats) in the caller's numbering."""
+    points, centroids = _f32(points), _f32(centroids)
+    n, d = points.shape
+    idx = torch.empty((n, num_neighbors), dtype=torch.int32, device=points.device)
+    dist = torch.empty((n, num_neighbors), dtype=torch.float32, device=points.device)
+    stats = (ctypes.c_int * 3)()
+    _check(lib().tsne_hip_knn_ivf(_ptr(points), n, d, num_neighbors, _ptr(centroids), centroids.shape[0], nprobe,
+                                  _ptr(idx), _ptr(dist), _stream(), stats))
+    return idx, dist, (int(stats[0]), int(stats[1]), int(stats[2]))
+
+
 def locality_order(points):
     """order[new] = old (int32): the renumbering RunTsne applies on entry."""
     points = _f32(points)
@@ -169,6 +199,12 @@ def symmetrize_full(pij, idx):
     return row_ptr, col[:nnz.value], val[:nnz.value]
 
 
+def boxes_for_spread(spread):
+    """FIt-SNE's grid-size rule with the reference's constants (125 boxes at least, one per unit
+    of spread, rounded up in its list of sizes; 170 at most)."""
+    return int(lib().tsne_hip_boxes_for_spread(ctypes.c_float(spread)))
+
+
 class Plan(object):
     """Scratch memory of the gradient loop for one problem size."""
 
@@ -200,6 +236,11 @@ class Plan(object):
     def set_recenter(self, enable):
         """Optional re-centring inside iterate_ (off by default, as in the reference)."""
         _check(lib().tsne_hip_plan_set_recenter(self._h, 1 if enable else 0))
+
+    def set_boxes(self, n_boxes_per_dim):
+        """Size of the interpolation grid from the next step on (the reference runs 130)."""
+        _check(lib().tsne_hip_plan_set_boxes(self._h, n_boxes_per_dim))
+        self.n_nodes = 3 * n_boxes_per_dim
 
     def prepare_attractive(self, pij, idx):
         """Re-blocks (pij, idx) into the plan; afterwards attractive() and
