@@ -153,7 +153,7 @@ def test_forces_and_fused_steps(c3):
 
 
 def test_blocked_attractive_with_more_than_1024_column_partitions():
-    """4.5 M points are 1099 column partitions of 4096: the re-blocking's scans
+    """4.5 M points are 2198 column partitions of 2048: the re-blocking's scans
     give every thread several partition slots.  A pattern without any locality
     (every strip references every partition, most runs far shorter than a work
     item) against the row-ordered kernel and, on its first and last rows, the

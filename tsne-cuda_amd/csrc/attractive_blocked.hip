@@ -236,9 +236,10 @@ __global__ void clear_pmax_kernel(float *p_max) {
 // which they only entered after every staging wave had written it: a buffer's
 // counters never run ahead by a generation, so the thresholds are exact.
 // A streaming wave therefore never waits for another streaming wave, and waits for
-// the staging waves only when they are less than one partition ahead.  The LDS
-// executes one wave's operations in order, so a counter update that follows a
-// wave's reads or writes of a buffer is seen after them; the counters only grow.
+// the staging waves only when they are less than one partition ahead.  A count
+// is made after a release fence and a wait ends with an acquire fence, both at
+// workgroup scope and on the LDS address space only (the entry loads from memory
+// stay in flight across them; measured cost: none); the counters only grow.
 // Every wait is a bounded poll.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int rl, float vx, float vy,
@@ -268,12 +269,15 @@ __device__ __forceinline__ void wait_for_count(const unsigned int *counter, unsi
         if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= need) break;
         __builtin_amdgcn_s_sleep(1);
     }
-    asm volatile("" ::: "memory");
+    // Acquire, for LDS only: the buffer accesses that follow are not issued before the count has been seen.
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 // One count from this wave, after everything it has issued to the LDS so far.
 __device__ __forceinline__ void count_wave(unsigned int *counter, int lane) {
-    asm volatile("" ::: "memory");
+    // Release, for LDS only (the wave's loads from memory stay in flight): every LDS access issued so far has
+    // been performed before the count is.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     if (lane == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     asm volatile("" ::: "memory");
 }

@@ -185,11 +185,12 @@ __global__ __launch_bounds__(256) void bounds_kernel(const float *__restrict__ v
 // The row index of the node grid is the x node.
 //
 // The reference issues 36 global atomics per point.  Nodes belong to exactly
-// one box, so here the points are first grouped by 10 x 10-box tile with a
-// counting sort (count, scan, scatter: positions only, the P matrix keeps its
-// order); then a workgroup takes up to 1024 points of one tile, accumulates
-// them into a private 30 x 30-node tile in LDS with (integer) LDS atomics, and
-// adds the non-zero nodes of its tile to the grid with one global atomic each.
+// one box, so here the points are first grouped by tile of kTileBoxes x
+// kTileBoxes (5 x 5) boxes with a counting sort (count, scan, scatter:
+// positions only, the P matrix keeps its order); then a workgroup takes up to
+// 1024 points of one tile, accumulates their moments per box in a private LDS
+// tile with (integer) LDS atomics, and adds the node sums that follow from the
+// moments to the grid with one global atomic each.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ int box_of(float v, const Bounds &bd, int n_boxes) {
 #pragma clang fp contract(off)
