@@ -232,6 +232,14 @@ int tsne_hip_plan_set_recenter(tsne_hip_plan *plan, int enable);
 int tsne_hip_plan_set_boxes(tsne_hip_plan *plan, int n_boxes_per_dim);
 int tsne_hip_boxes_for_spread(float spread);
 
+/* Inside a gradient loop the repulsive evaluation keeps its grouping of the points by grid tile
+ * from step to step while few points have left the neighbourhood of their tile, instead of
+ * counting and scattering all points every step (the reference has no such stage: its spread is
+ * 36 global atomics per point, src/kernels/nbodyfft.cu:107-139).  out[0..2]: repulsive evaluations
+ * of this plan so far, those that grouped the points afresh, and points that were spread on the
+ * slow path because they had strayed from their tile.  Waits for the device's pending work. */
+int tsne_hip_plan_grouping_stats(tsne_hip_plan *plan, unsigned int *out);
+
 /* Whether a kernel of this plan has reported trouble since the last call (no
  * counterpart in the reference).  Call it after synchronising the streams the
  * plan was used on.  The one condition reported today: waves of the re-blocked

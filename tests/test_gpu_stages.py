@@ -226,6 +226,47 @@ def test_iterate_short(stages, c0_problem, start, steps):
     plan.close()
 
 
+@pytest.mark.parametrize("eta,steps", [(200.0, 40), (3000.0, 12)])
+def test_iterate_keeps_the_grouping_by_tile(stages, c0_problem, monkeypatch, eta, steps):
+    """Inside a loop the repulsive chain keeps its grouping of the points by grid tile while few points
+    have left the neighbourhood of their tile.  40 steps at the usual learning rate, of which a good part
+    reuse the grouping, and 12 at a learning rate that throws points across several boxes per step (strays,
+    spread on the slow path, and early re-grouping), against the oracle's loop and against a plan that
+    groups afresh every step (TSNE_KEEP_GROUPING=0); a stage-level call in between (which always groups
+    afresh) must not disturb the loop's state."""
+    c = c0_problem
+    n = c["X"].shape[0]
+    y_o, z_o = oracle.iterate(c["P"], c["idx"], c["y0"], steps, eta=eta)
+
+    def run(keep):
+        monkeypatch.setenv("TSNE_KEEP_GROUPING", "1" if keep else "0")
+        plan = stages.Plan(n, c["K"])
+        plan.prepare_attractive(dev(c["P"]), dev(c["idx"]))
+        dy = dev(c["y0"])
+        gains, old = torch.ones_like(dy), torch.zeros_like(dy)
+        half = steps // 2
+        plan.iterate_(None, None, dy, gains, old, 0, half, eta=eta)
+        plan.repulsive(torch.flip(dy, [0]))  # an unrelated embedding through the stage call
+        z = plan.iterate_(None, None, dy, gains, old, half, steps, eta=eta)
+        stats = plan.grouping_stats()
+        plan.close()
+        return dy.cpu().numpy(), float(z.item()), stats
+
+    y_keep, z_keep, (runs, sorts, strays) = run(True)
+    y_fresh, z_fresh, (runs_f, sorts_f, strays_f) = run(False)
+    err_keep, err_fresh = rel_l2(y_keep, y_o), rel_l2(y_fresh, y_o)
+    print("eta %g: %d evaluations, %d groupings, %d strays; against the oracle %.2e (grouping kept) %.2e (afresh)"
+          % (eta, runs, sorts, strays, err_keep, err_fresh))
+    assert runs == steps + 1 and runs_f == steps + 1 and sorts_f == runs_f and strays_f == 0
+    assert 3 <= sorts <= (steps * 3 // 4 if eta < 1000 else steps)
+    if eta > 1000:
+        assert strays > 0
+    # (at the large learning rate the trajectory itself amplifies rounding differences: both plans sit equally
+    # far from the oracle)
+    assert err_keep <= max(2e-4, 2.0 * err_fresh) and err_fresh <= 1e-3
+    assert abs(z_keep - z_o) <= 1e-3 * abs(z_o)
+
+
 @pytest.mark.parametrize("prepared", [False, True])
 def test_iterate_with_recentring(stages, c0_problem, prepared):
     """The optional re-centring (not in the reference): every update subtracts the centre the

@@ -121,7 +121,7 @@ int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *e
                 hipStream_t s) {
     const bool overlap = overlap_enabled() && !p->profiling && p->side_stream != nullptr;
     if (!overlap) {
-        if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, s)) return 1;
+        if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, s, true)) return 1;
         if (launch_step_attractive(p, pij, indices, s)) return 1;
         if (normalization && launch_finish_z(p, normalization, s)) return 1;
         return launch_update(p, embedding, p->attr, p->rep, gains, old_forces, eta, nullptr, momentum, exaggeration,
@@ -130,7 +130,7 @@ int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *e
     hipStream_t side = p->side_stream;
     TSNE_TRY(hipEventRecord(p->fork_event, s));  // everything up to the previous step's update
     TSNE_TRY(hipStreamWaitEvent(side, p->fork_event, 0));
-    if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, side)) return 1;
+    if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, side, true)) return 1;
     if (normalization && launch_finish_z(p, normalization, side)) return 1;
     TSNE_TRY(hipEventRecord(p->join_event, side));
     if (launch_step_attractive(p, pij, indices, s)) return 1;
@@ -284,6 +284,7 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     release_blocked(p);
     (void)hipFree(p->yxy);
     (void)hipFree(p->tile_xy);
+    (void)hipFree(p->tile_perm);
     (void)hipFree(p->tile_count);
     (void)hipFree(p->tile_cursor);
     (void)hipFree(p->point_code);
@@ -320,6 +321,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
     p->n_nodes = n_boxes_per_dim * kInterp;
     p->device = device;
     p->lagrange = make_lagrange();
+    if (const char *v = std::getenv("TSNE_KEEP_GROUPING")) p->keep_grouping = v[0] != '0';
     // The grid buffers hold the largest grid: tsne_hip_plan_set_boxes may change the size between steps.
     const size_t G2 = (size_t)(kMaxBoxes * kInterp) * (kMaxBoxes * kInterp);
     const size_t spec = (size_t)2 * kFft * kNodePad;
@@ -333,6 +335,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
     // yxy carries one spare pair so that two-point (float4) loads may straddle the end.
     bool ok = hipMalloc(&p->yxy, sizeof(float2) * (N + 2)) == hipSuccess &&
               hipMalloc(&p->tile_xy, sizeof(float2) * N) == hipSuccess &&
+              hipMalloc(&p->tile_perm, sizeof(int) * N) == hipSuccess &&
               hipMalloc(&p->tile_count, sizeof(int) * kMaxTiles) == hipSuccess &&
               hipMalloc(&p->tile_cursor, sizeof(int) * kMaxTiles) == hipSuccess &&
               hipMalloc(&p->point_code, sizeof(unsigned int) * N) == hipSuccess &&
@@ -560,6 +563,16 @@ int tsne_hip_plan_set_boxes(tsne_hip_plan *plan, int n_boxes_per_dim) {
     plan->step_graphs.clear();
     plan->n_boxes = n_boxes_per_dim;
     plan->n_nodes = n_boxes_per_dim * kInterp;
+    // (a grouping of the points by tile belongs to the grid it was made on)
+    TSNE_TRY(hipMemset(&plan->scalars->reuse_sort, 0, sizeof(int)));
+    return 0;
+}
+
+int tsne_hip_plan_grouping_stats(tsne_hip_plan *plan, unsigned int *out) {
+    if (check_plan(plan, "plan_grouping_stats")) return 1;
+    TSNE_REQUIRE(out, "plan_grouping_stats: null output");
+    TSNE_TRY(hipSetDevice(plan->device));
+    TSNE_TRY(hipMemcpy(out, &plan->scalars->chain_runs, 3 * sizeof(unsigned int), hipMemcpyDeviceToHost));
     return 0;
 }
 

@@ -92,6 +92,15 @@ struct LoopScalars {
     // Workgroups of the re-blocked attractive kernel in which a wave gave up waiting for an LDS counter (their
     // rows come out as NaN).  Never non-zero unless the kernel's roles lose step; the host checks it after a loop.
     unsigned int wait_timeouts;
+    // The grouping of the points by spreading tile is kept over the steps for as long as few points have left
+    // the neighbourhood of their tile: `strays` counts the points of the current step's spread that had (they are
+    // spread with global atomics instead), `sort_age` the steps since the grouping was made, and `reuse_sort`,
+    // set at the end of a step's chain, tells the next step's kernels to keep it.
+    unsigned int strays;
+    int sort_age;
+    int reuse_sort;
+    // Running totals since the plan was made: chain evaluations, those that grouped the points afresh, strays.
+    unsigned int chain_runs, chain_sorts, strays_total;
     // Optional re-centring (off unless the plan asks for it): per bounds slot, the sums of the x and of the y
     // coordinates of the embedding that slot's bounds describe.
     double center_sum[2][2];

@@ -393,7 +393,8 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
         } else {
             // Sampled steps run the phases one after the other so that the phase timers mean something.
             hip_or_die(hipEventRecord(ev[0], stream), "event");
-            TSNE_OR_DIE(tsnehip::launch_repulsive(plan, d_emb.as<float>(), slot, plan->rep, nullptr, nullptr, stream),
+            TSNE_OR_DIE(tsnehip::launch_repulsive(plan, d_emb.as<float>(), slot, plan->rep, nullptr, nullptr, stream,
+                                                  true),
                         "repulsive forces");
             hip_or_die(hipEventRecord(ev[1], stream), "event");
             TSNE_OR_DIE(full_sym ? tsnehip::launch_attractive_csr(plan, plan->csr_row_ptr, plan->csr_col_idx,

@@ -56,10 +56,12 @@ struct tsne_hip_plan {
     int *tile_cursor = nullptr;    // first position of every tile's run in tile_xy
     unsigned int *point_code = nullptr;  // N: (tile << 22 | rank among its workgroup's points of that tile), by the count kernel
     int *wg_tile_base = nullptr;   // kSortBlocks x kMaxTiles: where a workgroup's points start inside a tile's run
-    int4 *chunks = nullptr;        // (tile, first point, count, -) per spreading workgroup
+    int *tile_perm = nullptr;      // N: the point at every position of tile_xy (kept while the grouping is reused)
+    int4 *chunks = nullptr;        // (tile, first point, count, box offset of the first point in the tile's LDS region)
     int *num_chunks = nullptr;  // [0] chunks of the current step, [1] ticket counter of the tile count kernel
     int max_chunks = 0;
     int spread_grid = 512;         // workgroups of the spreading kernel (two per CU)
+    bool keep_grouping = true;     // loops may carry the grouping by tile from step to step (TSNE_KEEP_GROUPING=0: never)
     float4 *node_charges = nullptr;     // n_nodes^2, one float4 (4 terms) per node
     float4 *node_potentials = nullptr;  // n_nodes^2
     float2 *row_spectra = nullptr;      // 2 plane pairs x kFft x kNodePad (transposed)
@@ -122,8 +124,10 @@ int profile_mark(tsne_hip_plan *p, int id, hipStream_t s);
 // `slot` selects which pair of bounds in LoopScalars the launch reads.
 int launch_bounds_reset(tsne_hip_plan *p, int slot, hipStream_t s);
 int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s);
+// keep_grouping: the call is a step of a gradient loop over this embedding buffer, so the grouping of the points by
+// spreading tile may be carried over from the step before (the kernels decide on the device); otherwise it is redone.
 int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *rep, float *point_potentials,
-                     float *charges_out, hipStream_t s);
+                     float *charges_out, hipStream_t s, bool keep_grouping = false);
 // Writes Z = z_sum - N to the device scalar *normalization.
 int launch_finish_z(tsne_hip_plan *p, float *normalization, hipStream_t s);
 int launch_pack_xy(tsne_hip_plan *p, const float *embedding, hipStream_t s);

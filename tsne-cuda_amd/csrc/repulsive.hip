@@ -151,6 +151,7 @@ __global__ void bounds_reset_kernel(LoopScalars *sc, int slot) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         sc->min_enc[slot] = 0xffffffffu;
         sc->max_enc[slot] = 0u;
+        sc->reuse_sort = 0;  // a new embedding: whatever grouping by tile the plan holds is not its
     }
 }
 
@@ -287,7 +288,7 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
                                                          int *__restrict__ tile_cursor, int4 *__restrict__ chunks,
                                                          int *__restrict__ num_chunks, int *__restrict__ ticket,
                                                          unsigned int *__restrict__ point_code,
-                                                         int *__restrict__ wg_tile_base) {
+                                                         int *__restrict__ wg_tile_base, int keep_grouping) {
     __shared__ int hist[kMaxTiles];
     __shared__ int pts[1024], chk[1024];
     __shared__ int last;
@@ -302,6 +303,8 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
             sc->center_sum[next_slot][1] = 0.0;
         }
     }
+    // The grouping of the step before is kept (nobody writes the flag while this kernel runs).
+    if (keep_grouping && sc->reuse_sort) return;
     for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;
     __syncthreads();
     const Bounds bd = load_bounds(sc, slot, n_boxes);
@@ -340,15 +343,19 @@ __global__ __launch_bounds__(1024) void tile_scatter_kernel(const float *__restr
                                                            const int *__restrict__ tile_cursor,
                                                            const unsigned int *__restrict__ point_code,
                                                            const int *__restrict__ wg_tile_base,
-                                                           float2 *__restrict__ tile_xy) {
+                                                           float2 *__restrict__ tile_xy, int *__restrict__ tile_perm,
+                                                           const LoopScalars *sc, int keep_grouping) {
     __shared__ int base[kMaxTiles];
+    if (keep_grouping && sc->reuse_sort) return;
     // (entries of wg_tile_base for tiles this workgroup has no point in are never read)
     for (int b = threadIdx.x; b < n_tiles; b += blockDim.x)
         base[b] = tile_cursor[b] + wg_tile_base[(size_t)blockIdx.x * kMaxTiles + b];
     __syncthreads();
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
         const unsigned int code = point_code[i];
-        tile_xy[base[code >> kRankBits] + (int)(code & ((1u << kRankBits) - 1u))] = make_float2(emb[i], emb[N + i]);
+        const int pos = base[code >> kRankBits] + (int)(code & ((1u << kRankBits) - 1u));
+        tile_xy[pos] = make_float2(emb[i], emb[N + i]);
+        tile_perm[pos] = i;
     }
 }
 
@@ -401,21 +408,33 @@ __device__ __forceinline__ float box_lower(int b, const Bounds &bd) {
 // up to 4096 of them sum below 2^62.  The node sums are formed from the moments in fp64 when the tile is
 // flushed, which is exact to fp64 rounding where the per-point products were rounded to fp32.
 constexpr int kMoments = 21;
-constexpr int kTileBoxes2 = kTileBoxes * kTileBoxes;
+// The moments of a tile are kept for a region of the tile's 5 x 5 boxes plus a rim of kHalo boxes: when the
+// grouping by tile is carried over from an earlier step, the points of a tile have moved a little, and the region
+// is placed where the tile's points are now (the box of the chunk's first point minus the offset that point had
+// when the grouping was made).  Points that have left even the rim ("strays") add their 36 node contributions
+// with global atomics and are counted; too many of them and the next step groups the points afresh.
+constexpr int kHalo = 1;
+constexpr int kRegionBoxes = kTileBoxes + 2 * kHalo;
+constexpr int kRegionBoxes2 = kRegionBoxes * kRegionBoxes;
+constexpr int kMaxSortAge = 32;  // steps a grouping is kept at most
+constexpr int kStrayShift = 10;  // ... and only while at most N / 2^10 points strayed in the last step (36 global atomics each)
 __device__ __forceinline__ constexpr int moment_index(int i, int j) { return j <= 2 ? j * 5 + i : 15 + (j - 3) * 3 + i; }
 
 __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__restrict__ tile_xy,
-                                                     const int4 *__restrict__ chunks,
-                                                     const int *__restrict__ num_chunks, const LoopScalars *sc,
+                                                     const int *__restrict__ tile_perm,
+                                                     const float2 *__restrict__ yxy, int4 *chunks,
+                                                     const int *__restrict__ num_chunks, LoopScalars *sc,
                                                      int slot, int n_boxes, LagrangeConsts lc,
-                                                     float *__restrict__ w) {
-    __shared__ unsigned long long acc[kMoments * kTileBoxes2];  // one plane per moment
+                                                     float *__restrict__ w, int keep_grouping) {
+    __shared__ unsigned long long acc[kMoments * kRegionBoxes2];  // one plane per moment
+    __shared__ int origin[2];
     const int nc = *num_chunks;
     const int c0 = (int)((long long)blockIdx.x * nc / gridDim.x);
     const int c1 = (int)((long long)(blockIdx.x + 1) * nc / gridDim.x);
     if (c0 >= c1) return;
+    const bool reuse = keep_grouping && sc->reuse_sort;
     const int tid = threadIdx.x;
-    for (int e = tid; e < kMoments * kTileBoxes2; e += kSpreadThreads) acc[e] = 0ull;
+    for (int e = tid; e < kMoments * kRegionBoxes2; e += kSpreadThreads) acc[e] = 0ull;
     const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
     const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
@@ -429,62 +448,147 @@ __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__
         coef[m][1] = -(sk + sl) / d;
         coef[m][2] = 1.0 / d;
     }
-    // Unconditional, clamped loads: a chunk holds at least one point.
-    auto fetch = [&](const int4 &ch, float2 (&pt)[2]) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) pt[u] = tile_xy[ch.y + min(tid + u * kSpreadThreads, ch.z - 1)];
-    };
-    int4 ch = chunks[c0];
-    float2 pt[2];
-    fetch(ch, pt);
-    __syncthreads();  // the tile is zero
-    int cur_tile = ch.x, in_tile = 0;
-    for (int c = c0; c < c1; ++c) {
-        const bool last = c + 1 == c1;
-        int4 next_ch = ch;
-        float2 next_pt[2] = {pt[0], pt[1]};
-        if (!last) {
-            next_ch = chunks[c + 1];
-            fetch(next_ch, next_pt);
-        }
-        const int bx0 = (cur_tile % tiles_per_dim) * kTileBoxes;
-        const int by0 = (cur_tile / tiles_per_dim) * kTileBoxes;
+    // Unconditional, clamped loads: a chunk holds at least one point.  With a grouping carried over, the
+    // positions are the current ones of the points the grouping lists (the interleaved copy the update keeps):
+    // a chunk's list of points is fetched two chunks ahead, its positions one chunk ahead, so that neither load
+    // is waited for where it is issued.
+    const float2 *src = reuse ? yxy : tile_xy;
+    auto fetch_index = [&](const int4 &ch, int (&idx)[2]) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
+            const int pos = ch.y + min(tid + u * kSpreadThreads, ch.z - 1);
+            idx[u] = reuse ? tile_perm[pos] : pos;
+        }
+    };
+    auto fetch = [&](const int (&idx)[2], float2 (&pt)[2]) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) pt[u] = src[idx[u]];
+    };
+    int4 ch = chunks[c0];
+    int4 next_ch = c0 + 1 < c1 ? chunks[c0 + 1] : ch;
+    float2 pt[2];
+    int next_idx[2];
+    {
+        int idx[2];
+        fetch_index(ch, idx);
+        fetch_index(next_ch, next_idx);
+        fetch(idx, pt);
+    }
+    int cur_tile = ch.x, in_tile = 0;
+    bool new_run = true;
+    unsigned int strays = 0u;
+    int ox0 = 0, oy0 = 0;
+    for (int c = c0; c < c1; ++c) {
+        const bool last = c + 1 == c1;
+        float2 next_pt[2] = {pt[0], pt[1]};
+        int4 after_ch = next_ch;
+        int after_idx[2] = {next_idx[0], next_idx[1]};
+        if (!last) {
+            fetch(next_idx, next_pt);
+            if (c + 2 < c1) {
+                after_ch = chunks[c + 2];
+                fetch_index(after_ch, after_idx);
+            }
+        }
+        int pbx[2], pby[2];
+        float pcu[2], pcv[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            bin_and_coord(pt[u].x, bd, n_boxes, pbx[u], pcu[u]);
+            bin_and_coord(pt[u].y, bd, n_boxes, pby[u], pcv[u]);
+        }
+        // The chunk's anchor: the summed box coordinates of its first 64 points (the clamped loads make that 64
+        // whatever the chunk holds).  Stored relative to the region when the grouping is made; on later steps the
+        // region goes where the same points' sum puts it, i.e. it follows the mean movement of those points.
+        if ((new_run || !reuse) && tid < kWave) {
+            int sx = pbx[0], sy = pby[0];
+#pragma unroll
+            for (int m = kWave / 2; m >= 1; m >>= 1) {
+                sx += __shfl_xor(sx, m, kWave);
+                sy += __shfl_xor(sy, m, kWave);
+            }
+            if (tid == 0) {
+                const int fx = (cur_tile % tiles_per_dim) * kTileBoxes - kHalo;
+                const int fy = (cur_tile / tiles_per_dim) * kTileBoxes - kHalo;
+                if (!reuse) {
+                    origin[0] = fx;
+                    origin[1] = fy;
+                    reinterpret_cast<int *>(chunks)[4 * c + 3] = ((sx - kWave * fx) << 16) | (sy - kWave * fy);
+                } else {
+                    // floor((sum now - sum then) / 64 + 1/2), for either sign
+                    origin[0] = (sx - (ch.w >> 16) + kWave / 2 + kWave * 1024) / kWave - 1024;
+                    origin[1] = (sy - (ch.w & 0xffff) + kWave / 2 + kWave * 1024) / kWave - 1024;
+                }
+            }
+        }
+        if (new_run) {
+            __syncthreads();  // the region's place is known (and the region is zero)
+            ox0 = origin[0];
+            oy0 = origin[1];
+            new_run = false;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            bool stray = false;
             if (tid + u * kSpreadThreads < ch.z) {
-                int bx, by;
+                const int bx = pbx[u], by = pby[u];
                 float pu[5], pv[5];
                 pu[0] = pv[0] = 1.0f;
-                bin_and_coord(pt[u].x, bd, n_boxes, bx, pu[1]);
-                bin_and_coord(pt[u].y, bd, n_boxes, by, pv[1]);
+                pu[1] = pcu[u];
+                pv[1] = pcv[u];
+                const int lx = bx - ox0, ly = by - oy0;
+                if ((unsigned int)lx < (unsigned int)kRegionBoxes && (unsigned int)ly < (unsigned int)kRegionBoxes) {
 #pragma unroll
-                for (int k = 2; k < 5; ++k) {
-                    pu[k] = pu[k - 1] * pu[1];
-                    pv[k] = pv[k - 1] * pv[1];
+                    for (int k = 2; k < 5; ++k) {
+                        pu[k] = pu[k - 1] * pu[1];
+                        pv[k] = pv[k - 1] * pv[1];
+                    }
+                    unsigned long long *dst = acc + lx * kRegionBoxes + ly;
+#pragma unroll
+                    for (int j = 0; j < 5; ++j)
+#pragma unroll
+                        for (int i = 0; i < 5; ++i)
+                            if (j <= 2 || i <= 2)
+                                add_fixed(dst + moment_index(i, j) * kRegionBoxes2, pu[i] * pv[j], to_fixed);
+                } else {
+                    // A stray: its nine nodes directly (src/kernels/nbodyfft.cu:107-139).
+                    stray = true;
+                    const float x = pt[u].x, y = pt[u].y;
+                    float Lx[kInterp], Ly[kInterp];
+#pragma unroll
+                    for (int m = 0; m < kInterp; ++m) {
+                        Lx[m] = (float)(coef[m][0] + (coef[m][1] + coef[m][2] * pu[1]) * pu[1]);
+                        Ly[m] = (float)(coef[m][0] + (coef[m][1] + coef[m][2] * pv[1]) * pv[1]);
+                    }
+#pragma unroll
+                    for (int a = 0; a < kInterp; ++a)
+#pragma unroll
+                        for (int b = 0; b < kInterp; ++b) {
+                            const float lw = Lx[a] * Ly[b];
+                            float *out = w + ((size_t)(bx * kInterp + a) * G + (by * kInterp + b)) * kTerms;
+                            atomicAdd(out + 0, lw);
+                            atomicAdd(out + 1, lw * x);
+                            atomicAdd(out + 2, lw * y);
+                            atomicAdd(out + 3, lw * (x * x + y * y));
+                        }
                 }
-                unsigned long long *dst = acc + (bx - bx0) * kTileBoxes + (by - by0);
-#pragma unroll
-                for (int j = 0; j < 5; ++j)
-#pragma unroll
-                    for (int i = 0; i < 5; ++i)
-                        if (j <= 2 || i <= 2)
-                            add_fixed(dst + moment_index(i, j) * kTileBoxes2, pu[i] * pv[j], to_fixed);
             }
+            strays += stray ? 1u : 0u;
         }
         ++in_tile;
         if (last || next_ch.x != cur_tile || in_tile == kChunksPerFlush) {
             __syncthreads();
             // One thread per (box, node of the box): five sums over the nine monomial pairs, then the four terms.
-            for (int e = tid; e < kTileBoxes2 * kInterp * kInterp; e += kSpreadThreads) {
+            for (int e = tid; e < kRegionBoxes2 * kInterp * kInterp; e += kSpreadThreads) {
                 const int box = e / (kInterp * kInterp), a = (e / kInterp) % kInterp, b = e % kInterp;
                 const unsigned long long *src = acc + box;
                 if (src[0] == 0ull) continue;  // moment (0, 0) is the number of points in the box
-                const int bxl = box / kTileBoxes, byl = box % kTileBoxes;
-                const int gx = (bx0 + bxl) * kInterp + a, gy = (by0 + byl) * kInterp + b;
-                if (gx >= G || gy >= G) continue;
+                const int bxg = ox0 + box / kRegionBoxes, byg = oy0 + box % kRegionBoxes;
+                const int gx = bxg * kInterp + a, gy = byg * kInterp + b;
+                if (gx < 0 || gy < 0 || gx >= G || gy >= G) continue;  // (boxes with points lie inside the grid)
                 double M[kMoments];
 #pragma unroll
-                for (int m = 0; m < kMoments; ++m) M[m] = (double)(long long)src[m * kTileBoxes2] * from_fixed;
+                for (int m = 0; m < kMoments; ++m) M[m] = (double)(long long)src[m * kRegionBoxes2] * from_fixed;
                 double s00 = 0.0, s10 = 0.0, s01 = 0.0, s20 = 0.0, s02 = 0.0;
 #pragma unroll
                 for (int i = 0; i < 3; ++i)
@@ -498,7 +602,7 @@ __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__
                         s02 += cc * M[moment_index(i, j + 2)];
                     }
                 const double bw = bd.box_width;
-                const double xl = box_lower(bx0 + bxl, bd), yl = box_lower(by0 + byl, bd);
+                const double xl = box_lower(bxg, bd), yl = box_lower(byg, bd);
                 float *out = w + ((size_t)gx * G + gy) * kTerms;
                 atomicAdd(out + 0, (float)s00);
                 atomicAdd(out + 1, (float)(xl * s00 + bw * s10));
@@ -507,14 +611,26 @@ __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__
                                            bw * bw * (s20 + s02)));
             }
             __syncthreads();
-            for (int e = tid; e < kMoments * kTileBoxes2; e += kSpreadThreads) acc[e] = 0ull;
-            if (!last) __syncthreads();
+            for (int e = tid; e < kMoments * kRegionBoxes2; e += kSpreadThreads) acc[e] = 0ull;
+            // (the barrier of the next run's start, or the kernel's end, follows)
             cur_tile = next_ch.x;
             in_tile = 0;
+            new_run = true;
         }
         ch = next_ch;
         pt[0] = next_pt[0];
         pt[1] = next_pt[1];
+        next_ch = after_ch;
+        next_idx[0] = after_idx[0];
+        next_idx[1] = after_idx[1];
+    }
+    // Strays are rare: one atomic per wave that met any.
+    const unsigned long long any = __ballot(strays != 0u);
+    if (any) {
+        unsigned int total = strays;
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) total += __shfl_xor(total, m, kWave);
+        if ((tid & (kWave - 1)) == 0) atomicAdd(&sc->strays, total);
     }
 }
 
@@ -719,8 +835,21 @@ __global__ __launch_bounds__(256) void gather_forces_kernel(const float *__restr
                                                             LagrangeConsts lc,
                                                             const float4 *__restrict__ node_potentials,
                                                             float *__restrict__ rep, float *__restrict__ phi_out,
-                                                            LoopScalars *sc) {
+                                                            LoopScalars *sc, int keep_grouping) {
     __shared__ float partial[256 / kWave];
+    // Last kernel of the chain: whether the next step keeps this step's grouping of the points by tile.  (The
+    // spread kernel has finished counting; the chain's kernels of this step have all read the flag.)
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        const bool reused = keep_grouping && sc->reuse_sort;
+        const int age = reused ? sc->sort_age + 1 : 0;
+        const unsigned int strays = sc->strays;
+        sc->strays = 0u;
+        sc->sort_age = age;
+        sc->chain_runs += 1u;
+        sc->chain_sorts += reused ? 0u : 1u;
+        sc->strays_total += strays;
+        sc->reuse_sort = (keep_grouping && strays <= (unsigned int)(N >> kStrayShift) && age < kMaxSortAge) ? 1 : 0;
+    }
     const Bounds bd = load_bounds(sc_in, slot, n_boxes);
     const int G = n_boxes * kInterp;
     float z = 0.0f;
@@ -796,7 +925,8 @@ int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_
 // `embedding` in `slot`; leaves sum_i z_i in scalars->z_part and resets the other
 // bounds slot.  charges_out (optional) receives a copy of the node charges.
 int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *rep, float *point_potentials,
-                     float *charges_out, hipStream_t s) {
+                     float *charges_out, hipStream_t s, bool keep_grouping) {
+    const int keep = keep_grouping && p->keep_grouping ? 1 : 0;
     const int N = p->num_points, G = p->n_nodes, nb = p->n_boxes;
     const int tiles_per_dim = (nb + kTileBoxes - 1) / kTileBoxes;
     // Few, large workgroups: every workgroup ends with one global atomic per tile counter, and
@@ -806,18 +936,20 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     if (profile_mark(p, kKernelTileCount, s)) return 1;
     tile_count_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, slot ^ 1, nb, p->tile_count,
                                                    p->tile_cursor, p->chunks, p->num_chunks, p->num_chunks + 1,
-                                                   p->point_code, p->wg_tile_base);
+                                                   p->point_code, p->wg_tile_base, keep);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelTileScatter, s)) return 1;
     tile_scatter_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, tiles_per_dim * tiles_per_dim, p->tile_cursor,
-                                                     p->point_code, p->wg_tile_base, p->tile_xy);
+                                                     p->point_code, p->wg_tile_base, p->tile_xy, p->tile_perm,
+                                                     p->scalars, keep);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelSpread, s)) return 1;
     // Resident workgroups share the chunk list (its length is only known on the device; with fewer chunks
     // than workgroups the surplus ones exit at once).
     const int spread_blocks = std::min(N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1, p->spread_grid);
-    spread_kernel<<<spread_blocks, kSpreadThreads, 0, s>>>(p->tile_xy, p->chunks, p->num_chunks, p->scalars, slot, nb,
-                                                p->lagrange, reinterpret_cast<float *>(p->node_charges));
+    spread_kernel<<<spread_blocks, kSpreadThreads, 0, s>>>(p->tile_xy, p->tile_perm, p->yxy, p->chunks,
+                                                           p->num_chunks, p->scalars, slot, nb, p->lagrange,
+                                                           reinterpret_cast<float *>(p->node_charges), keep);
     TSNE_LAUNCHED(s);
     if (charges_out)
         TSNE_TRY(hipMemcpyAsync(charges_out, p->node_charges, sizeof(float4) * (size_t)G * G,
@@ -835,7 +967,7 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelGather, s)) return 1;
     gather_forces_kernel<<<std::min(div_up(N, 256), 1024), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
-                                                        p->node_potentials, rep, point_potentials, p->scalars);
+                                                        p->node_potentials, rep, point_potentials, p->scalars, keep);
     TSNE_LAUNCHED(s);
     return 0;
 }

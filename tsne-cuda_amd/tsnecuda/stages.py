@@ -47,6 +47,8 @@ def lib():
         L.tsne_hip_plan_check.argtypes = [_vp]
         L.tsne_hip_plan_set_recenter.argtypes = [_vp, c_int]
         L.tsne_hip_plan_set_recenter.restype = c_int
+        L.tsne_hip_plan_grouping_stats.argtypes = [_vp, _vp]
+        L.tsne_hip_plan_grouping_stats.restype = c_int
         L.tsne_hip_plan_set_boxes.argtypes = [_vp, c_int]
         L.tsne_hip_plan_set_boxes.restype = c_int
         L.tsne_hip_boxes_for_spread.argtypes = [c_float]
@@ -236,6 +238,13 @@ class Plan(object):
     def set_recenter(self, enable):
         """Optional re-centring inside iterate_ (off by default, as in the reference)."""
         _check(lib().tsne_hip_plan_set_recenter(self._h, 1 if enable else 0))
+
+    def grouping_stats(self):
+        """(repulsive evaluations so far, those that grouped the points by tile afresh, points spread
+        on the slow path because they had strayed from their tile)."""
+        out = (ctypes.c_uint * 3)()
+        _check(lib().tsne_hip_plan_grouping_stats(self._h, out))
+        return int(out[0]), int(out[1]), int(out[2])
 
     def set_boxes(self, n_boxes_per_dim):
         """Size of the interpolation grid from the next step on (the reference runs 130)."""
