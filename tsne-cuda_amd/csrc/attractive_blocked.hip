@@ -30,6 +30,7 @@
 // only the order of the additions inside a row differs.
 #include <algorithm>
 #include <cstdlib>
+#include <vector>
 
 #include "plan.h"
 
@@ -120,7 +121,8 @@ constexpr int kResidueStride = kResidues + 1;  // odd: the 32 counters of differ
 constexpr size_t kReblockLds = sizeof(unsigned int) * 2 * kBalancedParts * kResidueStride;
 
 __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
-                                                         int N, int K, int strip_rows, int list_words,
+                                                         int N, int K, const int *__restrict__ strip_row0,
+                                                         int list_words,
                                                          int seg_stride, float *__restrict__ ent_p,
                                                          unsigned int *__restrict__ seg, float *__restrict__ p_max) {
     __shared__ unsigned int cursor[kMaxParts];
@@ -130,8 +132,8 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
     unsigned int *residue_cursor = residue_count + kBalancedParts * kResidueStride;  // same shape
     const int tid = threadIdx.x;
     const int strip = blockIdx.x;
-    const int row0 = strip * strip_rows;
-    const int nrows = min(strip_rows, N - row0);
+    const int row0 = strip_row0[strip];
+    const int nrows = strip_row0[strip + 1] - row0;
     const size_t base = (size_t)row0 * K;
     const unsigned int count = (unsigned int)nrows * (unsigned int)K;
     for (int b = tid; b < kMaxParts; b += kBlock) cursor[b] = 0;
@@ -144,7 +146,7 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
     scan_slots(mine, first, scan, tid);
 #pragma unroll
     for (int i = 0; i < kSlotsPerThread; ++i) cursor[tid * kSlotsPerThread + i] = first[i];
-    // Layout of a strip's list: {-, partitions referenced, -, -}, then for the k-th referenced partition the
+    // Layout of a strip's list: {first row, partitions referenced, rows, -}, then for the k-th referenced partition the
     // first entry of its run (n_parts + 4 words, unused ones hold ~0), then the partitions themselves in the
     // same order (n_parts words).
     unsigned int *hdr = seg + (size_t)strip * seg_stride;
@@ -163,7 +165,11 @@ __global__ __launch_bounds__(kBlock) void reblock_kernel(const float *__restrict
             fresh_of[tid * kSlotsPerThread + i] = (unsigned short)order[i];
         }
     for (unsigned int b = n_fresh + tid; b < (unsigned int)list_words; b += kBlock) run_start[b] = ~0u;
-    if (tid == 0) hdr[1] = n_fresh;
+    if (tid == 0) {
+        hdr[0] = (unsigned int)row0;
+        hdr[1] = n_fresh;
+        hdr[2] = (unsigned int)nrows;
+    }
     const bool balanced = n_fresh <= (unsigned int)kBalancedParts;
     if (balanced) {
         for (unsigned int b = tid; b < 2u * kBalancedParts * kResidueStride; b += kBlock) residue_count[b] = 0u;
@@ -290,7 +296,7 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
                                                                     const float2 *__restrict__ yxy,
                                                                     LoopScalars *__restrict__ scalars,
                                                                     float *__restrict__ attr, int N, int K,
-                                                                    int strip_rows, int list_words, int seg_stride,
+                                                                    int list_words, int seg_stride,
                                                                     int spin_limit_arg) {
     const int spin_limit = RUNTIME_LIMIT ? spin_limit_arg : kSpinLimit;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -302,14 +308,14 @@ __global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int strip = blockIdx.x;
-    const int row0 = strip * strip_rows;
-    const int nrows = min(strip_rows, N - row0);
     // The list is read through the constant address space: it is never written while this
     // kernel runs, and constant-space loads at uniform addresses are scalar loads, which do not
     // queue behind the vector loads in flight.
     typedef const __attribute__((address_space(4))) unsigned int *ConstWords;
     ConstWords hdr = (ConstWords)(seg + (size_t)strip * seg_stride);
+    const int row0 = (int)hdr[0];
     const int n_fresh = (int)hdr[1];
+    const int nrows = (int)hdr[2];
     ConstWords run_start = hdr + 4;  // ~0 after the last run
     ConstWords fresh_parts = run_start + list_words;
     const float pm = scalars->vmax;
@@ -459,6 +465,92 @@ static_assert(kBlockedLds <= 160 * 1024, "one workgroup must fit the 160 KB of L
 
 }  // namespace
 
+// ---------------------------------------------------------------------------
+// Strip boundaries.  What a strip costs the force kernel is its entries plus a fixed price for every column
+// partition it references (staging the partition, and a second pass over the item in which its run starts):
+// measured at a million points, 0.42 us per partition against 0.21 ns per entry, i.e. a partition costs what
+// about 2000 entries do.  With equal strips the few that straddle two clusters of the data reference twice the
+// partitions of the others and finish 40 % later, and the launch lasts as long as its slowest workgroup.  When
+// all strips run at once (no more strips than CUs) their boundaries are therefore chosen so that the predicted
+// costs are equal: the rows are cut into micro-strips of 64, a kernel finds the partitions every micro-strip
+// references (a bitmap), and the host merges consecutive micro-strips greedily under the smallest cost limit
+// that needs no more strips than there are CUs (bisection on the limit).
+// ---------------------------------------------------------------------------
+namespace {
+
+constexpr int kMicroRows = 64;
+constexpr long long kPartCostEntries = 2000;
+
+__global__ __launch_bounds__(256) void micro_strip_parts_kernel(const int *__restrict__ idx, int N, int K, int words,
+                                                                unsigned int *__restrict__ bitmaps) {
+    extern __shared__ unsigned int bits[];
+    for (int w = threadIdx.x; w < words; w += 256) bits[w] = 0u;
+    __syncthreads();
+    const int row0 = blockIdx.x * kMicroRows;
+    const int nrows = min(kMicroRows, N - row0);
+    const size_t base = (size_t)row0 * K;
+    for (int e = threadIdx.x; e < nrows * K; e += 256) {
+        const int part = idx[base + e] / kPartPoints;
+        atomicOr(&bits[part >> 5], 1u << (part & 31));
+    }
+    __syncthreads();
+    for (int w = threadIdx.x; w < words; w += 256) bitmaps[(size_t)blockIdx.x * words + w] = bits[w];
+}
+
+}  // namespace
+
+// row0 (n_strips + 1 entries, ascending, row0[0] = 0, row0[n_strips] = N) of strips with at most kStripMax rows
+// and equal predicted cost, at most max_strips of them.
+static int balanced_strips(const int *indices, int N, int K, int n_parts, int max_strips, std::vector<int> &row0,
+                           hipStream_t s) {
+    const int micro = div_up(N, kMicroRows), words = div_up(n_parts, 32);
+    unsigned int *d_bits = nullptr;
+    TSNE_TRY(hipMalloc(&d_bits, sizeof(unsigned int) * (size_t)micro * words));
+    micro_strip_parts_kernel<<<micro, 256, sizeof(unsigned int) * words, s>>>(indices, N, K, words, d_bits);
+    std::vector<unsigned int> bits((size_t)micro * words);
+    hipError_t err = hipGetLastError();
+    if (err == hipSuccess) err = hipStreamSynchronize(s);
+    if (err == hipSuccess)
+        err = hipMemcpy(bits.data(), d_bits, sizeof(unsigned int) * bits.size(), hipMemcpyDeviceToHost);
+    (void)hipFree(d_bits);
+    TSNE_TRY(err);
+    std::vector<unsigned int> acc(words);
+    // Greedy merge under a cost limit; returns the number of strips (boundaries in `out` when given).
+    auto cut = [&](long long limit, std::vector<int> *out) {
+        int strips = 0, m = 0;
+        if (out) out->assign(1, 0);
+        while (m < micro) {
+            std::fill(acc.begin(), acc.end(), 0u);
+            int rows = 0, parts = 0;
+            while (m < micro) {
+                const int add_rows = std::min(kMicroRows, N - m * kMicroRows);
+                int new_parts = parts;
+                const unsigned int *b = &bits[(size_t)m * words];
+                for (int w = 0; w < words; ++w) new_parts += __builtin_popcount(b[w] & ~acc[w]);
+                const long long cost = (long long)(rows + add_rows) * K + kPartCostEntries * new_parts;
+                if (rows > 0 && (rows + add_rows > kStripMax || cost > limit)) break;
+                for (int w = 0; w < words; ++w) acc[w] |= b[w];
+                rows += add_rows;
+                parts = new_parts;
+                ++m;
+            }
+            ++strips;
+            if (out) out->push_back(m * kMicroRows < N ? m * kMicroRows : N);
+        }
+        return strips;
+    };
+    long long lo = 0, hi = (long long)kStripMax * K + kPartCostEntries * n_parts;  // hi always suffices when N fits
+    while (lo + 1 < hi) {
+        const long long mid = lo + (hi - lo) / 2;
+        if (cut(mid, nullptr) <= max_strips)
+            hi = mid;
+        else
+            lo = mid;
+    }
+    cut(hi, &row0);
+    return 0;
+}
+
 void release_blocked(tsne_hip_plan *p) {
     // Steps may still be running (tsne_hip_iterate is asynchronous) and captured steps hold the addresses
     // about to be freed: wait for the plan's own streams and the device before anything is destroyed.
@@ -469,8 +561,10 @@ void release_blocked(tsne_hip_plan *p) {
     p->step_graphs.clear();
     (void)hipFree(p->ent_p);
     (void)hipFree(p->seg);
+    (void)hipFree(p->strip_row0);
     p->ent_p = nullptr;
     p->seg = nullptr;
+    p->strip_row0 = nullptr;
     p->blocked_ready = false;
 }
 
@@ -494,8 +588,18 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
         set_error("attractive_prepare: num_neighbors = %d is too large for the blocked format", K);
         return kShapeNotSupported;
     }
-    p->strip_rows = strip_rows;
-    p->n_strips = div_up(N, strip_rows);
+    // Equal strips, or - when they all run at once - strips of equal predicted cost.
+    std::vector<int> row0;
+    if (div_up(N, kStripMax) <= cus && N > cus * kMicroRows && std::getenv("TSNE_EQUAL_STRIPS") == nullptr) {
+        if (balanced_strips(indices, N, K, n_parts, cus, row0, s)) return 1;
+    } else {
+        for (int r = 0; r < N; r += strip_rows) row0.push_back(r);
+        row0.push_back(N);
+    }
+    p->n_strips = (int)row0.size() - 1;
+    strip_rows = 0;
+    for (int i = 0; i < p->n_strips; ++i) strip_rows = std::max(strip_rows, row0[i + 1] - row0[i]);
+    p->strip_rows = strip_rows;  // the longest strip
     p->n_parts = n_parts;
     // A strip's list: the run starts (padded: the force kernel reads two past the last run) and the partitions.
     p->list_words = (n_parts + 4 + 3) & ~3;
@@ -504,7 +608,9 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     const size_t items_per_strip = ((size_t)strip_rows * K + kItemEntries - 1) / kItemEntries;
     const size_t nnz = items_per_strip * p->n_strips * kItemEntries;
     bool ok = hipMalloc(&p->ent_p, 2 * sizeof(float) * nnz) == hipSuccess &&
-              hipMalloc(&p->seg, sizeof(unsigned int) * (size_t)p->n_strips * p->seg_stride) == hipSuccess;
+              hipMalloc(&p->seg, sizeof(unsigned int) * (size_t)p->n_strips * p->seg_stride) == hipSuccess &&
+              hipMalloc(&p->strip_row0, sizeof(int) * row0.size()) == hipSuccess &&
+              hipMemcpy(p->strip_row0, row0.data(), sizeof(int) * row0.size(), hipMemcpyHostToDevice) == hipSuccess;
     if (!ok) {
         release_blocked(p);
         set_error("attractive_prepare: out of device memory for the re-blocked pattern (%zu bytes)", nnz * 8);
@@ -514,7 +620,7 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     TSNE_LAUNCHED(s);
     TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(reblock_kernel),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kReblockLds));
-    reblock_kernel<<<p->n_strips, kBlock, kReblockLds, s>>>(pij, indices, N, K, strip_rows, p->list_words, p->seg_stride, p->ent_p,
+    reblock_kernel<<<p->n_strips, kBlock, kReblockLds, s>>>(pij, indices, N, K, p->strip_row0, p->list_words, p->seg_stride, p->ent_p,
                                                   p->seg,
                                                   &p->scalars->vmax);
     TSNE_LAUNCHED(s);
@@ -537,7 +643,7 @@ int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s) {
     if (profile_mark(p, kKernelAttractive, s)) return 1;
     const auto kernel = p->spin_limit == kSpinLimit ? attractive_blocked_kernel<false> : attractive_blocked_kernel<true>;
     kernel<<<p->n_strips, kBlock, kBlockedLds, s>>>(p->ent_p, p->seg, p->yxy, p->scalars, attr, p->num_points,
-                                                    p->num_neighbors, p->strip_rows, p->list_words, p->seg_stride,
+                                                    p->num_neighbors, p->list_words, p->seg_stride,
                                                     p->spin_limit);
     TSNE_LAUNCHED(s);
     return 0;

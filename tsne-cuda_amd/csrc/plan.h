@@ -77,7 +77,8 @@ struct tsne_hip_plan {
                                     // 8 bytes each, grouped by (row strip, column partition), in items of
                                     // consecutive entries that are interleaved over the strips
     unsigned int *seg = nullptr;    // per strip seg_stride words: counts, run starts, partitions in opening order
-    int strip_rows = 0, n_strips = 0, n_parts = 0, list_words = 0, seg_stride = 0;
+    int strip_rows = 0, n_strips = 0, n_parts = 0, list_words = 0, seg_stride = 0;  // strip_rows: of the longest strip
+    int *strip_row0 = nullptr;      // n_strips + 1: first row of every strip
     int spin_limit = 0;             // polls before a wave of the attractive kernel gives up a wait
     bool blocked_ready = false;
     // Optional CSR pattern (borrowed pointers; tsne_hip_plan_set_csr_pattern): when set, steps without an explicit

@@ -51,22 +51,42 @@ __device__ __forceinline__ float2 csub(float2 a, float2 b) { return make_float2(
 // in LDS.  L is the sub-transform length of the stage.  Forward stages run
 // L = 1024, 256, 64, 16, 4; inverse stages run the same butterflies backwards
 // with L = 4, 16, 64, 256, 1024.
+//
+// A thread works on butterfly q = tid mod 256 of every transform it visits (the workgroups have a multiple of 256
+// threads), so the three twiddles it needs in each of the five stages are the same for all of them: they are
+// loaded once, ahead of the data, and stay in registers.  (Loaded where they are used, every stage waits for a
+// trip to memory; beside the attractive kernel, which keeps the memory system busy, that trip is long.)
+struct StageTwiddles {
+    float2 w[kLog2Fft / 2][3];  // [stage, L = 1024 first][power]
+};
+__device__ __forceinline__ StageTwiddles load_twiddles(const float2 *tw, int tid) {
+    StageTwiddles t;
+    const int q = tid & 255;
+#pragma unroll
+    for (int si = 0; si < kLog2Fft / 2; ++si) {
+        const int log2L = kLog2Fft - 2 * si;
+        const int k = q & ((1 << (log2L - 2)) - 1);
+        const int stride = kFft >> log2L;
+        t.w[si][0] = tw[k * stride];
+        t.w[si][1] = tw[2 * k * stride];
+        t.w[si][2] = tw[3 * k * stride];
+    }
+    return t;
+}
+
 template <bool INVERSE>
-__device__ __forceinline__ void radix4_stage(float2 *s, int nfft, int log2L, const float2 *tw, int tid,
+__device__ __forceinline__ void radix4_stage(float2 *s, int nfft, int log2L, const float2 (&w)[3], int tid,
                                              int nthreads) {
     const int L = 1 << log2L;
     const int q4 = L >> 2;
     const int log2q4 = log2L - 2;
-    const int stride = kFft >> log2L;
+    const float2 w1 = w[0], w2 = w[1], w3 = w[2];
     for (int id = tid; id < nfft * (kFft / 4); id += nthreads) {
         const int f = id >> 8;
-        const int q = id & 255;
+        const int q = id & 255;  // == tid & 255: nthreads is a multiple of 256
         const int k = q & (q4 - 1);
         const int b = q >> log2q4;
         float2 *a = s + f * kFft + b * L + k;
-        const float2 w1 = tw[k * stride];
-        const float2 w2 = tw[2 * k * stride];
-        const float2 w3 = tw[3 * k * stride];
         float2 a0 = a[0], a1 = a[q4], a2 = a[2 * q4], a3 = a[3 * q4];
         if (!INVERSE) {
             const float2 t0 = cadd(a0, a2), t1 = csub(a0, a2), t2 = cadd(a1, a3), t3 = csub(a1, a3);
@@ -87,17 +107,17 @@ __device__ __forceinline__ void radix4_stage(float2 *s, int nfft, int log2L, con
     }
 }
 
-__device__ __forceinline__ void fft_forward(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+__device__ __forceinline__ void fft_forward(float2 *s, int nfft, const StageTwiddles &tw, int tid, int nthreads) {
 #pragma unroll
     for (int l = kLog2Fft; l >= 2; l -= 2) {
-        radix4_stage<false>(s, nfft, l, tw, tid, nthreads);
+        radix4_stage<false>(s, nfft, l, tw.w[(kLog2Fft - l) / 2], tid, nthreads);
         __syncthreads();
     }
 }
-__device__ __forceinline__ void fft_inverse(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+__device__ __forceinline__ void fft_inverse(float2 *s, int nfft, const StageTwiddles &tw, int tid, int nthreads) {
 #pragma unroll
     for (int l = 2; l <= kLog2Fft; l += 2) {
-        radix4_stage<true>(s, nfft, l, tw, tid, nthreads);
+        radix4_stage<true>(s, nfft, l, tw.w[(kLog2Fft - l) / 2], tid, nthreads);
         __syncthreads();
     }
 }
@@ -651,14 +671,15 @@ __device__ __forceinline__ float kernel_value(float lo, float h, int a, int b) {
     return (float)(1.0 / (s * s));
 }
 
+template <int THREADS>
 __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *sc, int slot, int n_boxes,
-                                                  const float2 *__restrict__ tw, float *__restrict__ kernel_rows,
+                                                  const StageTwiddles &tw, float *__restrict__ kernel_rows,
                                                   float2 (*s)[kFft]) {
     const int tid = threadIdx.x;
     const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
     const int a0 = block * 4;
-    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
+    for (int e = tid; e < 2 * kFft; e += THREADS) {
         const int f = e >> kLog2Fft, m = e & (kFft - 1);
         const int b = m < kFft / 2 ? m : kFft - m;
         const int ra = a0 + 2 * f;
@@ -670,8 +691,8 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
         s[f][m] = v;
     }
     __syncthreads();
-    fft_forward(&s[0][0], 2, tw, tid, kRowThreads);
-    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
+    fft_forward(&s[0][0], 2, tw, tid, THREADS);
+    for (int e = tid; e < 2 * kFft; e += THREADS) {
         const int f = e >> kLog2Fft, pos = e & (kFft - 1);
         const int v = rev4(pos);
         if (v <= kFft / 2) {
@@ -683,31 +704,35 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
 }
 
 // ---------------------------------------------------------------------------
-// Row pass: transforms two grid rows (x nodes m0, m0+1), both plane pairs,
-// along the y-node axis; clears the charges it consumed so that the next step
-// starts from zero without a memset.  Output is transposed:
+// Row pass: transforms ROWS grid rows (x nodes m0 ...), both plane pairs, along the y-node axis; clears the
+// charges it consumed so that the next step starts from zero without a memset.  Output is transposed:
 // row_spectra[pair][pos][m], pos = digit-reversed frequency position.
+//
+// Two rows per workgroup (512 threads, 32 KB of LDS) is what the loop uses.  One row per workgroup (256 threads,
+// 16 KB, so that two fit into the 35 KB of LDS a CU has left beside the attractive kernel's workgroup and the
+// whole launch is resident at once) measured 51 us against 61 us beside that kernel and 21 us against 17 us
+// alone, and 2 % fewer iterations per second: what slows the pass down there is not the number of rounds.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kRowThreads) void conv_rows_forward_kernel(float4 *__restrict__ w, int G, int n_boxes,
-                                                                const LoopScalars *sc, int slot,
-                                                                const float2 *__restrict__ twiddles,
-                                                                float2 *__restrict__ row_spectra,
-                                                                float *__restrict__ kernel_rows) {
-    // 32 KB of LDS, twiddles straight from memory (an 8 KB table every CU keeps in its L1): small
-    // enough to run next to the attractive kernel's workgroup on the same CU.
-    __shared__ float2 s[4][kFft];  // [row * 2 + pair]
-    const float2 *tw = twiddles;
+template <int ROWS>
+__global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *__restrict__ w, int G, int n_boxes,
+                                                                       const LoopScalars *sc, int slot,
+                                                                       const float2 *__restrict__ twiddles,
+                                                                       float2 *__restrict__ row_spectra,
+                                                                       float *__restrict__ kernel_rows) {
+    constexpr int kThreads = 256 * ROWS;
+    __shared__ float2 s[2 * ROWS][kFft];  // [row * 2 + pair]
+    const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
     const int tid = threadIdx.x;
-    // The workgroups past the row pairs produce the kernel's row spectra (needed by the column
+    // The workgroups past the rows produce the kernel's row spectra (needed by the column
     // pass only): the two jobs are independent and share the launch.
-    const int row_blocks = (G + 1) / 2;
+    const int row_blocks = (G + ROWS - 1) / ROWS;
     if ((int)blockIdx.x >= row_blocks) {
-        kernel_rows_block(blockIdx.x - row_blocks, sc, slot, n_boxes, tw, kernel_rows, s);
+        kernel_rows_block<kThreads>(blockIdx.x - row_blocks, sc, slot, n_boxes, tw, kernel_rows, s);
         return;
     }
-    const int m0 = blockIdx.x * 2;
+    const int m0 = blockIdx.x * ROWS;
     const float s3 = r2_plane_scale(sc, slot);
-    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
+    for (int e = tid; e < ROWS * kFft; e += kThreads) {
         const int r = e >> kLog2Fft, n = e & (kFft - 1);
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (n < G && m0 + r < G) {
@@ -719,12 +744,16 @@ __global__ __launch_bounds__(kRowThreads) void conv_rows_forward_kernel(float4 *
         s[r * 2 + 1][n] = make_float2(v.y, v.z);       // planes x and y
     }
     __syncthreads();
-    fft_forward(&s[0][0], 4, tw, tid, kRowThreads);
-    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
+    fft_forward(&s[0][0], 2 * ROWS, tw, tid, kThreads);
+    for (int e = tid; e < 2 * kFft; e += kThreads) {
         const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
-        const float2 r0 = s[0 + pair][pos], r1 = s[2 + pair][pos];
-        float4 *dst = reinterpret_cast<float4 *>(row_spectra + ((size_t)pair * kFft + pos) * kNodePad + m0);
-        *dst = make_float4(r0.x, r0.y, r1.x, r1.y);
+        float2 *dst = row_spectra + ((size_t)pair * kFft + pos) * kNodePad + m0;
+        if (ROWS == 2) {
+            const float2 r0 = s[0 + pair][pos], r1 = s[2 + pair][pos];
+            *reinterpret_cast<float4 *>(dst) = make_float4(r0.x, r0.y, r1.x, r1.y);
+        } else {
+            *dst = s[pair][pos];
+        }
     }
 }
 
@@ -745,7 +774,7 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
     constexpr int kPairsInFlight = 2;
     constexpr int kData = 2 * kPairsInFlight;  // transforms of data per round
     __shared__ float2 s[kData + 1][kFft];
-    const float2 *tw = twiddles;
+    const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
     const int tid = threadIdx.x;
     const int c0 = blockIdx.x * 2;
     {
@@ -800,7 +829,7 @@ __global__ __launch_bounds__(kRowThreads) void conv_rows_inverse_kernel(const fl
                                                                 const float2 *__restrict__ twiddles,
                                                                 float4 *__restrict__ node_potentials) {
     __shared__ float2 s[4][kFft];  // [row * 2 + pair]; twiddles from memory, as in the forward pass
-    const float2 *tw = twiddles;
+    const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
     const int tid = threadIdx.x;
     const int m0 = blockIdx.x * 2;
     for (int e = tid; e < 2 * kFft; e += kRowThreads) {
@@ -955,8 +984,8 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
         TSNE_TRY(hipMemcpyAsync(charges_out, p->node_charges, sizeof(float4) * (size_t)G * G,
                                 hipMemcpyDeviceToDevice, s));
     if (profile_mark(p, kKernelConvRowsForward, s)) return 1;
-    conv_rows_forward_kernel<<<div_up(G, 2) + div_up(G, 4), kRowThreads, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
-                                                                         p->twiddles, p->row_spectra, p->kernel_rows);
+    conv_rows_forward_kernel<2><<<div_up(G, 2) + div_up(G, 4), 512, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
+                                                                            p->twiddles, p->row_spectra, p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
     conv_columns_kernel<<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
