@@ -443,8 +443,14 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
     TSNE_TRY(hipStreamWaitEvent(s, plan->enter_event, 0));
     // Bounds and the interleaved copy of the starting embedding; from then on
     // the update kernel keeps both current.
+    // A call that takes up where the last one left off (same buffer, next step) keeps the chain's grouping of the
+    // points by tile; should the caller have changed the positions in between, the grouping is merely a poor one
+    // (the spread kernel finds the strays and the next step groups afresh).
+    const bool continues = embedding == plan->loop_embedding && step_begin == plan->loop_next_step;
+    plan->loop_embedding = embedding;
+    plan->loop_next_step = step_end;
     int slot = 0;
-    if (launch_bounds(plan, embedding, slot, s)) return 1;
+    if (launch_bounds(plan, embedding, slot, s, !continues)) return 1;
     if (plan->recenter && launch_centre_sums(plan, embedding, slot, s)) return 1;
     if (launch_pack_xy(plan, embedding, s)) return 1;
     // Schedule of src/fit_tsne.cu:416-420: two stretches of constant parameters; the step that reports the

@@ -61,6 +61,8 @@ struct tsne_hip_plan {
     int *num_chunks = nullptr;  // [0] chunks of the current step, [1] ticket counter of the tile count kernel
     int max_chunks = 0;
     int spread_grid = 512;         // workgroups of the spreading kernel (two per CU)
+    const float *loop_embedding = nullptr;  // where tsne_hip_iterate last left off: the buffer and the step after its last
+    int loop_next_step = -1;
     bool keep_grouping = true;     // loops may carry the grouping by tile from step to step (TSNE_KEEP_GROUPING=0: never)
     float4 *node_charges = nullptr;     // n_nodes^2, one float4 (4 terms) per node
     float4 *node_potentials = nullptr;  // n_nodes^2
@@ -123,8 +125,9 @@ int profile_mark(tsne_hip_plan *p, int id, hipStream_t s);
 
 // Stage launchers shared between the stage-level ABI and the fused loop.
 // `slot` selects which pair of bounds in LoopScalars the launch reads.
-int launch_bounds_reset(tsne_hip_plan *p, int slot, hipStream_t s);
-int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s);
+// new_embedding: the plan's grouping of the points by grid tile (if any) was made for other positions and is dropped.
+int launch_bounds_reset(tsne_hip_plan *p, int slot, hipStream_t s, bool new_embedding = true);
+int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s, bool new_embedding = true);
 // keep_grouping: the call is a step of a gradient loop over this embedding buffer, so the grouping of the points by
 // spreading tile may be carried over from the step before (the kernels decide on the device); otherwise it is redone.
 int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *rep, float *point_potentials,

@@ -47,79 +47,126 @@ __device__ __forceinline__ float2 cmul_conj(float2 a, float2 b) {  // a * conj(b
 __device__ __forceinline__ float2 cadd(float2 a, float2 b) { return make_float2(a.x + b.x, a.y + b.y); }
 __device__ __forceinline__ float2 csub(float2 a, float2 b) { return make_float2(a.x - b.x, a.y - b.y); }
 
-// One radix-4 stage over `nfft` transforms of length 1024 stored back to back
-// in LDS.  L is the sub-transform length of the stage.  Forward stages run
-// L = 1024, 256, 64, 16, 4; inverse stages run the same butterflies backwards
-// with L = 4, 16, 64, 256, 1024.
+// The transforms of length 1024 are five radix-4 levels (sub-transform lengths 1024, 256, 64, 16, 4 forwards, the
+// same backwards for the inverse), run as three passes over the LDS: levels 1024 + 256 and 64 + 16 are fused - a
+// thread holds the 16 elements that the two levels combine among themselves in registers - and level 4 is a pass
+// of its own.  Data flow and element order are those of five in-place radix-4 passes; what the fusion saves is two
+// of the five trips through the LDS and two of the five barriers of what is a chain of dependent, latency-bound
+// steps.  The three twiddles a thread needs per level and butterfly depend on its number only (thread mod 64 is
+// the butterfly it works on in every transform it visits), so they are loaded once, ahead of the data, and stay
+// in registers.
 //
-// A thread works on butterfly q = tid mod 256 of every transform it visits (the workgroups have a multiple of 256
-// threads), so the three twiddles it needs in each of the five stages are the same for all of them: they are
-// loaded once, ahead of the data, and stay in registers.  (Loaded where they are used, every stage waits for a
-// trip to memory; beside the attractive kernel, which keeps the memory system busy, that trip is long.)
+// A transform occupies 1056 LDS slots: one slot of padding after every 32 elements, so that the strides the
+// levels use (64, 4 and 1 elements between the lanes of a wave, 8-byte elements) fall on different banks - with
+// a plain layout the lanes of the 16- and 4-point levels hit each bank eight deep.
+constexpr int kFftPad = kFft + kFft / 32;
+__device__ __forceinline__ int pad(int i) { return i + (i >> 5); }
+
 struct StageTwiddles {
-    float2 w[kLog2Fft / 2][3];  // [stage, L = 1024 first][power]
+    float2 a[2][4][3];  // fused pass 0 (lengths 1024 + 256) and 1 (64 + 16): level of length L, [element mod 4][power]
+    float2 b[2][3];     // ... level of length L / 4
 };
 __device__ __forceinline__ StageTwiddles load_twiddles(const float2 *tw, int tid) {
     StageTwiddles t;
-    const int q = tid & 255;
+    const int lane = tid & 63;
 #pragma unroll
-    for (int si = 0; si < kLog2Fft / 2; ++si) {
-        const int log2L = kLog2Fft - 2 * si;
-        const int k = q & ((1 << (log2L - 2)) - 1);
+    for (int fs = 0; fs < 2; ++fs) {
+        const int log2L = kLog2Fft - 4 * fs;
+        const int q16 = 1 << (log2L - 4);
+        const int k = lane & (q16 - 1);
         const int stride = kFft >> log2L;
-        t.w[si][0] = tw[k * stride];
-        t.w[si][1] = tw[2 * k * stride];
-        t.w[si][2] = tw[3 * k * stride];
+#pragma unroll
+        for (int jl = 0; jl < 4; ++jl)
+#pragma unroll
+            for (int pw = 0; pw < 3; ++pw) t.a[fs][jl][pw] = tw[(pw + 1) * (k + jl * q16) * stride];
+#pragma unroll
+        for (int pw = 0; pw < 3; ++pw) t.b[fs][pw] = tw[(pw + 1) * k * stride * 4];
     }
     return t;
 }
 
-template <bool INVERSE>
-__device__ __forceinline__ void radix4_stage(float2 *s, int nfft, int log2L, const float2 (&w)[3], int tid,
-                                             int nthreads) {
-    const int L = 1 << log2L;
-    const int q4 = L >> 2;
-    const int log2q4 = log2L - 2;
-    const float2 w1 = w[0], w2 = w[1], w3 = w[2];
-    for (int id = tid; id < nfft * (kFft / 4); id += nthreads) {
-        const int f = id >> 8;
-        const int q = id & 255;  // == tid & 255: nthreads is a multiple of 256
-        const int k = q & (q4 - 1);
-        const int b = q >> log2q4;
-        float2 *a = s + f * kFft + b * L + k;
-        float2 a0 = a[0], a1 = a[q4], a2 = a[2 * q4], a3 = a[3 * q4];
+// Radix-4 butterflies on four registers: decimation in frequency forwards (twiddles after the sums), decimation in
+// time for the inverse (conjugate twiddles first).
+__device__ __forceinline__ void butterfly_forward(float2 &x0, float2 &x1, float2 &x2, float2 &x3, const float2 (&w)[3]) {
+    const float2 t0 = cadd(x0, x2), t1 = csub(x0, x2), t2 = cadd(x1, x3), t3 = csub(x1, x3);
+    x0 = cadd(t0, t2);
+    x1 = cmul(make_float2(t1.x + t3.y, t1.y - t3.x), w[0]);
+    x2 = cmul(csub(t0, t2), w[1]);
+    x3 = cmul(make_float2(t1.x - t3.y, t1.y + t3.x), w[2]);
+}
+__device__ __forceinline__ void butterfly_inverse(float2 &x0, float2 &x1, float2 &x2, float2 &x3, const float2 (&w)[3]) {
+    const float2 a1 = cmul_conj(x1, w[0]), a2 = cmul_conj(x2, w[1]), a3 = cmul_conj(x3, w[2]);
+    const float2 u0 = cadd(x0, a2), u1 = csub(x0, a2), u2 = cadd(a1, a3), u3 = csub(a1, a3);
+    x0 = cadd(u0, u2);
+    x1 = make_float2(u1.x - u3.y, u1.y + u3.x);
+    x2 = csub(u0, u2);
+    x3 = make_float2(u1.x + u3.y, u1.y - u3.x);
+}
+
+// Fused pass FS over `nfft` transforms stored kFftPad slots apart: 64 threads per transform, 16 elements each.
+template <bool INVERSE, int FS>
+__device__ __forceinline__ void radix16_pass(float2 *s, int nfft, const StageTwiddles &tw, int tid, int nthreads) {
+    constexpr int log2L = kLog2Fft - 4 * FS;
+    constexpr int L = 1 << log2L, q16 = L >> 4;
+    for (int id = tid; id < nfft * 64; id += nthreads) {
+        const int f = id >> 6, t = id & 63;  // t == tid & 63: nthreads is a multiple of 64
+        const int k = t & (q16 - 1), b = t >> (log2L - 4);
+        float2 *base = s + f * kFftPad;
+        const int i0 = b * L + k;
+        float2 x[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) x[j] = base[pad(i0 + j * q16)];
         if (!INVERSE) {
-            const float2 t0 = cadd(a0, a2), t1 = csub(a0, a2), t2 = cadd(a1, a3), t3 = csub(a1, a3);
-            a[0] = cadd(t0, t2);
-            a[q4] = cmul(make_float2(t1.x + t3.y, t1.y - t3.x), w1);
-            a[2 * q4] = cmul(csub(t0, t2), w2);
-            a[3 * q4] = cmul(make_float2(t1.x - t3.y, t1.y + t3.x), w3);
+#pragma unroll
+            for (int jl = 0; jl < 4; ++jl) butterfly_forward(x[jl], x[jl + 4], x[jl + 8], x[jl + 12], tw.a[FS][jl]);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) butterfly_forward(x[4 * m], x[4 * m + 1], x[4 * m + 2], x[4 * m + 3], tw.b[FS]);
         } else {
-            a1 = cmul_conj(a1, w1);
-            a2 = cmul_conj(a2, w2);
-            a3 = cmul_conj(a3, w3);
-            const float2 u0 = cadd(a0, a2), u1 = csub(a0, a2), u2 = cadd(a1, a3), u3 = csub(a1, a3);
-            a[0] = cadd(u0, u2);
-            a[q4] = make_float2(u1.x - u3.y, u1.y + u3.x);
-            a[2 * q4] = csub(u0, u2);
-            a[3 * q4] = make_float2(u1.x + u3.y, u1.y - u3.x);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) butterfly_inverse(x[4 * m], x[4 * m + 1], x[4 * m + 2], x[4 * m + 3], tw.b[FS]);
+#pragma unroll
+            for (int jl = 0; jl < 4; ++jl) butterfly_inverse(x[jl], x[jl + 4], x[jl + 8], x[jl + 12], tw.a[FS][jl]);
         }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) base[pad(i0 + j * q16)] = x[j];
     }
 }
 
-__device__ __forceinline__ void fft_forward(float2 *s, int nfft, const StageTwiddles &tw, int tid, int nthreads) {
-#pragma unroll
-    for (int l = kLog2Fft; l >= 2; l -= 2) {
-        radix4_stage<false>(s, nfft, l, tw.w[(kLog2Fft - l) / 2], tid, nthreads);
-        __syncthreads();
+// The level of length 4 (no twiddles): 256 threads per transform, four neighbouring elements each.
+template <bool INVERSE>
+__device__ __forceinline__ void radix4_last_pass(float2 *s, int nfft, int tid, int nthreads) {
+    const float2 one[3] = {make_float2(1.f, 0.f), make_float2(1.f, 0.f), make_float2(1.f, 0.f)};
+    for (int id = tid; id < nfft * (kFft / 4); id += nthreads) {
+        const int f = id >> 8, q = id & 255;
+        float2 *base = s + f * kFftPad;
+        float2 x0 = base[pad(4 * q)], x1 = base[pad(4 * q + 1)], x2 = base[pad(4 * q + 2)], x3 = base[pad(4 * q + 3)];
+        if (!INVERSE)
+            butterfly_forward(x0, x1, x2, x3, one);
+        else
+            butterfly_inverse(x0, x1, x2, x3, one);
+        base[pad(4 * q)] = x0;
+        base[pad(4 * q + 1)] = x1;
+        base[pad(4 * q + 2)] = x2;
+        base[pad(4 * q + 3)] = x3;
     }
 }
+
+// Forward: natural order in, base-4 digit-reversed order out; inverse: the other way round.  Both end with a barrier.
+__device__ __forceinline__ void fft_forward(float2 *s, int nfft, const StageTwiddles &tw, int tid, int nthreads) {
+    radix16_pass<false, 0>(s, nfft, tw, tid, nthreads);
+    __syncthreads();
+    radix16_pass<false, 1>(s, nfft, tw, tid, nthreads);
+    __syncthreads();
+    radix4_last_pass<false>(s, nfft, tid, nthreads);
+    __syncthreads();
+}
 __device__ __forceinline__ void fft_inverse(float2 *s, int nfft, const StageTwiddles &tw, int tid, int nthreads) {
-#pragma unroll
-    for (int l = 2; l <= kLog2Fft; l += 2) {
-        radix4_stage<true>(s, nfft, l, tw.w[(kLog2Fft - l) / 2], tid, nthreads);
-        __syncthreads();
-    }
+    radix4_last_pass<true>(s, nfft, tid, nthreads);
+    __syncthreads();
+    radix16_pass<true, 1>(s, nfft, tw, tid, nthreads);
+    __syncthreads();
+    radix16_pass<true, 0>(s, nfft, tw, tid, nthreads);
+    __syncthreads();
 }
 
 struct Bounds {
@@ -167,11 +214,11 @@ __device__ __forceinline__ void bin_and_weights(float v, const Bounds &bd, int n
 // (src/fit_tsne.cu:430-432), kept on the device in an order-preserving integer
 // encoding so that blocks can combine with integer atomics.
 // ---------------------------------------------------------------------------
-__global__ void bounds_reset_kernel(LoopScalars *sc, int slot) {
+__global__ void bounds_reset_kernel(LoopScalars *sc, int slot, int new_embedding) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         sc->min_enc[slot] = 0xffffffffu;
         sc->max_enc[slot] = 0u;
-        sc->reuse_sort = 0;  // a new embedding: whatever grouping by tile the plan holds is not its
+        if (new_embedding) sc->reuse_sort = 0;  // whatever grouping by tile the plan holds is not this embedding's
     }
 }
 
@@ -314,15 +361,6 @@ __global__ __launch_bounds__(1024) void tile_count_kernel(const float *__restric
     __shared__ int last;
     const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
     const int n_tiles = tiles_per_dim * tiles_per_dim;
-    if (blockIdx.x == 0 && threadIdx.x < kZParts) sc->z_part[threadIdx.x] = 0.0f;
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
-        if (next_slot >= 0) {
-            sc->min_enc[next_slot] = 0xffffffffu;
-            sc->max_enc[next_slot] = 0u;
-            sc->center_sum[next_slot][0] = 0.0;
-            sc->center_sum[next_slot][1] = 0.0;
-        }
-    }
     // The grouping of the step before is kept (nobody writes the flag while this kernel runs).
     if (keep_grouping && sc->reuse_sort) return;
     for (int b = threadIdx.x; b < n_tiles; b += blockDim.x) hist[b] = 0;
@@ -444,10 +482,19 @@ __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__
                                                      const int *__restrict__ tile_perm,
                                                      const float2 *__restrict__ yxy, int4 *chunks,
                                                      const int *__restrict__ num_chunks, LoopScalars *sc,
-                                                     int slot, int n_boxes, LagrangeConsts lc,
+                                                     int slot, int next_slot, int n_boxes, LagrangeConsts lc,
                                                      float *__restrict__ w, int keep_grouping) {
     __shared__ unsigned long long acc[kMoments * kRegionBoxes2];  // one plane per moment
     __shared__ int origin[2];
+    // The step's resets: the partial sums of z (the gather kernel at the chain's end adds to them) and the
+    // bounds slot the coming update will fill.
+    if (blockIdx.x == 0 && threadIdx.x < kZParts) sc->z_part[threadIdx.x] = 0.0f;
+    if (blockIdx.x == 0 && threadIdx.x == 0 && next_slot >= 0) {
+        sc->min_enc[next_slot] = 0xffffffffu;
+        sc->max_enc[next_slot] = 0u;
+        sc->center_sum[next_slot][0] = 0.0;
+        sc->center_sum[next_slot][1] = 0.0;
+    }
     const int nc = *num_chunks;
     const int c0 = (int)((long long)blockIdx.x * nc / gridDim.x);
     const int c1 = (int)((long long)(blockIdx.x + 1) * nc / gridDim.x);
@@ -674,7 +721,7 @@ __device__ __forceinline__ float kernel_value(float lo, float h, int a, int b) {
 template <int THREADS>
 __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *sc, int slot, int n_boxes,
                                                   const StageTwiddles &tw, float *__restrict__ kernel_rows,
-                                                  float2 (*s)[kFft]) {
+                                                  float2 (*s)[kFftPad]) {
     const int tid = threadIdx.x;
     const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
@@ -688,7 +735,7 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
             if (ra < G) v.x = kernel_value(bd.lo, bd.h, ra, b);
             if (ra + 1 < G) v.y = kernel_value(bd.lo, bd.h, ra + 1, b);
         }
-        s[f][m] = v;
+        s[f][pad(m)] = v;
     }
     __syncthreads();
     fft_forward(&s[0][0], 2, tw, tid, THREADS);
@@ -697,7 +744,7 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
         const int v = rev4(pos);
         if (v <= kFft / 2) {
             const int ra = a0 + 2 * f;
-            const float2 val = s[f][pos];
+            const float2 val = s[f][pad(pos)];
             *reinterpret_cast<float2 *>(kernel_rows + (size_t)v * kNodePad + ra) = val;
         }
     }
@@ -720,7 +767,7 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
                                                                        float2 *__restrict__ row_spectra,
                                                                        float *__restrict__ kernel_rows) {
     constexpr int kThreads = 256 * ROWS;
-    __shared__ float2 s[2 * ROWS][kFft];  // [row * 2 + pair]
+    __shared__ float2 s[2 * ROWS][kFftPad];  // [row * 2 + pair]
     const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
     const int tid = threadIdx.x;
     // The workgroups past the rows produce the kernel's row spectra (needed by the column
@@ -740,8 +787,8 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
             v = *src;
             *src = make_float4(0.f, 0.f, 0.f, 0.f);
         }
-        s[r * 2 + 0][n] = make_float2(v.x, v.w * s3);  // planes 1 and r^2 / m^2
-        s[r * 2 + 1][n] = make_float2(v.y, v.z);       // planes x and y
+        s[r * 2 + 0][pad(n)] = make_float2(v.x, v.w * s3);  // planes 1 and r^2 / m^2
+        s[r * 2 + 1][pad(n)] = make_float2(v.y, v.z);       // planes x and y
     }
     __syncthreads();
     fft_forward(&s[0][0], 2 * ROWS, tw, tid, kThreads);
@@ -749,10 +796,10 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
         const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
         float2 *dst = row_spectra + ((size_t)pair * kFft + pos) * kNodePad + m0;
         if (ROWS == 2) {
-            const float2 r0 = s[0 + pair][pos], r1 = s[2 + pair][pos];
+            const float2 r0 = s[0 + pair][pad(pos)], r1 = s[2 + pair][pad(pos)];
             *reinterpret_cast<float4 *>(dst) = make_float4(r0.x, r0.y, r1.x, r1.y);
         } else {
-            *dst = s[pair][pos];
+            *dst = s[pair][pad(pos)];
         }
     }
 }
@@ -773,7 +820,7 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
     // Twiddles come straight from memory.  Layout: [pair in flight][col], then the kernel columns.
     constexpr int kPairsInFlight = 2;
     constexpr int kData = 2 * kPairsInFlight;  // transforms of data per round
-    __shared__ float2 s[kData + 1][kFft];
+    __shared__ float2 s[kData + 1][kFftPad];
     const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
     const int tid = threadIdx.x;
     const int c0 = blockIdx.x * 2;
@@ -788,7 +835,7 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
                 v.x = kernel_rows[(size_t)v0 * kNodePad + a];
                 v.y = kernel_rows[(size_t)v1 * kNodePad + a];
             }
-            s[kData][m] = v;
+            s[kData][pad(m)] = v;
         }
     }
     for (int pair0 = 0; pair0 < 2; pair0 += kPairsInFlight) {
@@ -796,25 +843,25 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
             const int t = e >> kLog2Fft, m = e & (kFft - 1);  // t = pair in flight * 2 + col
             float2 v = make_float2(0.f, 0.f);
             if (m < G) v = row_spectra[((size_t)(pair0 + (t >> 1)) * kFft + c0 + (t & 1)) * kNodePad + m];
-            s[t][m] = v;
+            s[t][pad(m)] = v;
         }
         __syncthreads();
         // (the kernel columns are transformed with the first round)
         fft_forward(&s[0][0], pair0 == 0 ? kData + 1 : kData, tw, tid, 512);
         for (int e = tid; e < kData * kFft; e += 512) {
             const int t = e >> kLog2Fft, m = e & (kFft - 1);
-            const float2 kk = s[kData][m];
+            const float2 kk = s[kData][pad(m)];
             const float kv = (t & 1) ? kk.y : kk.x;
-            float2 v = s[t][m];
+            float2 v = s[t][pad(m)];
             v.x *= kv;
             v.y *= kv;
-            s[t][m] = v;
+            s[t][pad(m)] = v;
         }
         __syncthreads();
         fft_inverse(&s[0][0], kData, tw, tid, 512);
         for (int e = tid; e < kData * kFft; e += 512) {
             const int t = e >> kLog2Fft, m = e & (kFft - 1);
-            if (m < G) col_results[((size_t)(pair0 + (t >> 1)) * kFft + c0 + (t & 1)) * kNodePad + m] = s[t][m];
+            if (m < G) col_results[((size_t)(pair0 + (t >> 1)) * kFft + c0 + (t & 1)) * kNodePad + m] = s[t][pad(m)];
         }
         __syncthreads();
     }
@@ -828,7 +875,7 @@ __global__ __launch_bounds__(kRowThreads) void conv_rows_inverse_kernel(const fl
                                                                 const LoopScalars *sc, int slot,
                                                                 const float2 *__restrict__ twiddles,
                                                                 float4 *__restrict__ node_potentials) {
-    __shared__ float2 s[4][kFft];  // [row * 2 + pair]; twiddles from memory, as in the forward pass
+    __shared__ float2 s[4][kFftPad];  // [row * 2 + pair]
     const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
     const int tid = threadIdx.x;
     const int m0 = blockIdx.x * 2;
@@ -836,8 +883,8 @@ __global__ __launch_bounds__(kRowThreads) void conv_rows_inverse_kernel(const fl
         const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
         const float4 v =
             *reinterpret_cast<const float4 *>(col_results + ((size_t)pair * kFft + pos) * kNodePad + m0);
-        s[0 + pair][pos] = make_float2(v.x, v.y);
-        s[2 + pair][pos] = make_float2(v.z, v.w);
+        s[0 + pair][pad(pos)] = make_float2(v.x, v.y);
+        s[2 + pair][pad(pos)] = make_float2(v.z, v.w);
     }
     __syncthreads();
     fft_inverse(&s[0][0], 4, tw, tid, kRowThreads);
@@ -846,7 +893,7 @@ __global__ __launch_bounds__(kRowThreads) void conv_rows_inverse_kernel(const fl
     for (int e = tid; e < 2 * kFft; e += kRowThreads) {
         const int r = e >> kLog2Fft, n = e & (kFft - 1);
         if (n < G && m0 + r < G) {
-            const float2 p0 = s[r * 2 + 0][n], p1 = s[r * 2 + 1][n];
+            const float2 p0 = s[r * 2 + 0][pad(n)], p1 = s[r * 2 + 1][pad(n)];
             node_potentials[(size_t)(m0 + r) * G + n] =
                 make_float4(p0.x * scale, p1.x * scale, p1.y * scale, p0.y * scale3);
         }
@@ -935,14 +982,14 @@ int launch_finish_z(tsne_hip_plan *p, float *normalization, hipStream_t s) {
     return 0;
 }
 
-int launch_bounds_reset(tsne_hip_plan *p, int slot, hipStream_t s) {
-    bounds_reset_kernel<<<1, 64, 0, s>>>(p->scalars, slot);
+int launch_bounds_reset(tsne_hip_plan *p, int slot, hipStream_t s, bool new_embedding) {
+    bounds_reset_kernel<<<1, 64, 0, s>>>(p->scalars, slot, new_embedding ? 1 : 0);
     TSNE_LAUNCHED(s);
     return 0;
 }
 
-int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s) {
-    if (launch_bounds_reset(p, slot, s)) return 1;
+int launch_bounds(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s, bool new_embedding) {
+    if (launch_bounds_reset(p, slot, s, new_embedding)) return 1;
     const int64_t n = 2 * (int64_t)p->num_points;
     const int blocks = (int)std::min<int64_t>(div_up(n, 256 * 4), 2048);
     bounds_kernel<<<blocks, 256, 0, s>>>(embedding, n, p->scalars, slot);
@@ -977,7 +1024,7 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     // than workgroups the surplus ones exit at once).
     const int spread_blocks = std::min(N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1, p->spread_grid);
     spread_kernel<<<spread_blocks, kSpreadThreads, 0, s>>>(p->tile_xy, p->tile_perm, p->yxy, p->chunks,
-                                                           p->num_chunks, p->scalars, slot, nb, p->lagrange,
+                                                           p->num_chunks, p->scalars, slot, slot ^ 1, nb, p->lagrange,
                                                            reinterpret_cast<float *>(p->node_charges), keep);
     TSNE_LAUNCHED(s);
     if (charges_out)
