@@ -59,6 +59,7 @@ def main():
     ap.add_argument("--points", type=int, default=None, help="override the point count of the workload")
     ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end fit through pymodule_tsne")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-approx", action="store_true", help="skip the timing of the optional approximate neighbour search")
     ap.add_argument("--no-overlap", action="store_true",
                     help="run the repulsive chain and the attractive kernel one after the other (TSNE_OVERLAP=0): "
                          "per-kernel durations in a trace then are those of kernels running alone")
@@ -114,7 +115,7 @@ def main():
     # The optional approximate search (inverted file, floor(sqrt(N)) lists as the reference's FAISS index, 100
     # lists probed per list: what TSNE_KNN=ivf runs): training and search timed, recall against the exact rows.
     approx = None
-    if d <= 126 and n >= 4096:
+    if d <= 126 and n >= 4096 and not args.no_approx:
         import math
         nlist = int(math.isqrt(n))
         cen, train_s = timed(lambda: stages.ivf_train(dXs, nlist))

@@ -195,6 +195,16 @@ int tsne_hip_repulsive(tsne_hip_plan *plan, const float *embedding, float *repul
                        float *normalization, float *node_charges, float *node_potentials,
                        float *point_potentials, void *stream);
 
+/* tsne_hip_repulsive as a step of a gradient loop evaluates it: the grouping of the points by
+ * grid tile that the previous evaluation through this function left in the plan is kept while
+ * few points have left the neighbourhood of their tile (those are spread on a slower path and
+ * counted, see tsne_hip_plan_grouping_stats), otherwise the points are grouped afresh.  Same
+ * results as tsne_hip_repulsive up to the order of floating-point additions.  No counterpart
+ * in the reference. */
+int tsne_hip_repulsive_kept(tsne_hip_plan *plan, const float *embedding, float *repulsive_forces,
+                       float *normalization, float *node_charges, float *node_potentials,
+                       float *point_potentials, void *stream);
+
 /* Gains / momentum update of all 2N coordinates; zeroes both force arrays.
  * normalization is a device scalar.  Replaces tsnecuda::ApplyForces
  * (src/kernels/apply_forces.cu:59-82). */

@@ -417,6 +417,22 @@ int tsne_hip_repulsive(tsne_hip_plan *plan, const float *embedding, float *repul
     return launch_finish_z(plan, normalization, s);
 }
 
+int tsne_hip_repulsive_kept(tsne_hip_plan *plan, const float *embedding, float *repulsive_forces,
+                            float *normalization, float *node_charges, float *node_potentials,
+                            float *point_potentials, void *stream) {
+    if (check_plan(plan, "repulsive_kept")) return 1;
+    TSNE_REQUIRE(embedding && repulsive_forces && normalization, "repulsive_kept: null pointer argument");
+    hipStream_t s = (hipStream_t)stream;
+    if (launch_bounds(plan, embedding, 0, s, false)) return 1;
+    if (launch_pack_xy(plan, embedding, s)) return 1;
+    if (launch_repulsive(plan, embedding, 0, repulsive_forces, point_potentials, node_charges, s, true)) return 1;
+    if (node_potentials)
+        TSNE_TRY(hipMemcpyAsync(node_potentials, plan->node_potentials,
+                                sizeof(float4) * (size_t)plan->n_nodes * plan->n_nodes, hipMemcpyDeviceToDevice,
+                                s));
+    return launch_finish_z(plan, normalization, s);
+}
+
 int tsne_hip_update(tsne_hip_plan *plan, float *embedding, float *attractive_forces, float *repulsive_forces,
                     float *gains, float *old_forces, float eta, const float *normalization, float momentum,
                     float exaggeration, void *stream) {

@@ -47,6 +47,19 @@ __device__ __forceinline__ float2 cmul_conj(float2 a, float2 b) {  // a * conj(b
 __device__ __forceinline__ float2 cadd(float2 a, float2 b) { return make_float2(a.x + b.x, a.y + b.y); }
 __device__ __forceinline__ float2 csub(float2 a, float2 b) { return make_float2(a.x - b.x, a.y - b.y); }
 
+// The row passes read or write the transposed spectra in 16-byte pieces (two neighbouring rows of one spectrum
+// position); the eight workgroups whose pieces share a 128-byte line should meet in one L2, or every XCD fetches
+// (or partially writes) the line for itself.  Workgroups go to the XCDs round robin by their number, so
+// workgroup b takes row block (b mod 8) * ceil(blocks / 8) + b / 8: an XCD gets a run of neighbouring rows.
+// Returns -1 for the surplus workgroups of the rounded-up launch.
+constexpr int kXcds = 8;
+__device__ __forceinline__ int xcd_row_block(int b, int blocks) {
+    const int per = (blocks + kXcds - 1) / kXcds;
+    const int logical = (b % kXcds) * per + b / kXcds;
+    return (b / kXcds < per && logical < blocks) ? logical : -1;
+}
+inline int xcd_launch_blocks(int blocks) { return kXcds * ((blocks + kXcds - 1) / kXcds); }
+
 // The transforms of length 1024 are five radix-4 levels (sub-transform lengths 1024, 256, 64, 16, 4 forwards, the
 // same backwards for the inverse), run as three passes over the LDS: levels 1024 + 256 and 64 + 16 are fused - a
 // thread holds the 16 elements that the two levels combine among themselves in registers - and level 4 is a pass
@@ -475,7 +488,8 @@ constexpr int kHalo = 1;
 constexpr int kRegionBoxes = kTileBoxes + 2 * kHalo;
 constexpr int kRegionBoxes2 = kRegionBoxes * kRegionBoxes;
 constexpr int kMaxSortAge = 32;  // steps a grouping is kept at most
-constexpr int kStrayShift = 10;  // ... and only while at most N / 2^10 points strayed in the last step (36 global atomics each)
+constexpr int kStrayShift = 10;  // ... and only while at most N / 2^10 points strayed in the last step (36 global atomics each),
+constexpr int kStrayFloor = 128; // or 128 of a small problem's
 __device__ __forceinline__ constexpr int moment_index(int i, int j) { return j <= 2 ? j * 5 + i : 15 + (j - 3) * 3 + i; }
 
 __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__restrict__ tile_xy,
@@ -496,9 +510,12 @@ __global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__
         sc->center_sum[next_slot][1] = 0.0;
     }
     const int nc = *num_chunks;
-    const int c0 = (int)((long long)blockIdx.x * nc / gridDim.x);
-    const int c1 = (int)((long long)(blockIdx.x + 1) * nc / gridDim.x);
-    if (c0 >= c1) return;
+    // Neighbouring stretches of the chunk list (tiles next to each other) go to workgroups of one XCD: the
+    // points of a region of the embedding tend to have numbers from one range, which that XCD's L2 then serves.
+    const int share = xcd_row_block(blockIdx.x, gridDim.x);  // (the grid is a multiple of the XCD count)
+    const int c0 = (int)((long long)share * nc / gridDim.x);
+    const int c1 = (int)((long long)(share + 1) * nc / gridDim.x);
+    if (share < 0 || c0 >= c1) return;
     const bool reuse = keep_grouping && sc->reuse_sort;
     const int tid = threadIdx.x;
     for (int e = tid; e < kMoments * kRegionBoxes2; e += kSpreadThreads) acc[e] = 0ull;
@@ -773,11 +790,14 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
     // The workgroups past the rows produce the kernel's row spectra (needed by the column
     // pass only): the two jobs are independent and share the launch.
     const int row_blocks = (G + ROWS - 1) / ROWS;
-    if ((int)blockIdx.x >= row_blocks) {
-        kernel_rows_block<kThreads>(blockIdx.x - row_blocks, sc, slot, n_boxes, tw, kernel_rows, s);
+    const int launched = kXcds * ((row_blocks + kXcds - 1) / kXcds);
+    if ((int)blockIdx.x >= launched) {
+        kernel_rows_block<kThreads>(blockIdx.x - launched, sc, slot, n_boxes, tw, kernel_rows, s);
         return;
     }
-    const int m0 = blockIdx.x * ROWS;
+    const int row_block = xcd_row_block(blockIdx.x, row_blocks);
+    if (row_block < 0) return;
+    const int m0 = row_block * ROWS;
     const float s3 = r2_plane_scale(sc, slot);
     for (int e = tid; e < ROWS * kFft; e += kThreads) {
         const int r = e >> kLog2Fft, n = e & (kFft - 1);
@@ -878,7 +898,9 @@ __global__ __launch_bounds__(kRowThreads) void conv_rows_inverse_kernel(const fl
     __shared__ float2 s[4][kFftPad];  // [row * 2 + pair]
     const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
     const int tid = threadIdx.x;
-    const int m0 = blockIdx.x * 2;
+    const int row_block = xcd_row_block(blockIdx.x, (G + 1) / 2);
+    if (row_block < 0) return;
+    const int m0 = row_block * 2;
     for (int e = tid; e < 2 * kFft; e += kRowThreads) {
         const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
         const float4 v =
@@ -924,7 +946,7 @@ __global__ __launch_bounds__(256) void gather_forces_kernel(const float *__restr
         sc->chain_runs += 1u;
         sc->chain_sorts += reused ? 0u : 1u;
         sc->strays_total += strays;
-        sc->reuse_sort = (keep_grouping && strays <= (unsigned int)(N >> kStrayShift) && age < kMaxSortAge) ? 1 : 0;
+        sc->reuse_sort = (keep_grouping && strays <= (unsigned int)max(N >> kStrayShift, kStrayFloor) && age < kMaxSortAge) ? 1 : 0;
     }
     const Bounds bd = load_bounds(sc_in, slot, n_boxes);
     const int G = n_boxes * kInterp;
@@ -1022,7 +1044,8 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     if (profile_mark(p, kKernelSpread, s)) return 1;
     // Resident workgroups share the chunk list (its length is only known on the device; with fewer chunks
     // than workgroups the surplus ones exit at once).
-    const int spread_blocks = std::min(N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1, p->spread_grid);
+    const int spread_blocks =
+        xcd_launch_blocks(std::min(N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1, p->spread_grid));
     spread_kernel<<<spread_blocks, kSpreadThreads, 0, s>>>(p->tile_xy, p->tile_perm, p->yxy, p->chunks,
                                                            p->num_chunks, p->scalars, slot, slot ^ 1, nb, p->lagrange,
                                                            reinterpret_cast<float *>(p->node_charges), keep);
@@ -1031,14 +1054,14 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
         TSNE_TRY(hipMemcpyAsync(charges_out, p->node_charges, sizeof(float4) * (size_t)G * G,
                                 hipMemcpyDeviceToDevice, s));
     if (profile_mark(p, kKernelConvRowsForward, s)) return 1;
-    conv_rows_forward_kernel<2><<<div_up(G, 2) + div_up(G, 4), 512, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
+    conv_rows_forward_kernel<2><<<xcd_launch_blocks(div_up(G, 2)) + div_up(G, 4), 512, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
                                                                             p->twiddles, p->row_spectra, p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
     conv_columns_kernel<<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvRowsInverse, s)) return 1;
-    conv_rows_inverse_kernel<<<div_up(G, 2), kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
+    conv_rows_inverse_kernel<<<xcd_launch_blocks(div_up(G, 2)), kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
                                                           p->node_potentials);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelGather, s)) return 1;

@@ -59,6 +59,7 @@ def lib():
         L.tsne_hip_attractive_prepare.argtypes = [_vp, _vp, _vp, _vp]
         L.tsne_hip_attractive_prepare.restype = c_int
         L.tsne_hip_repulsive.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]
+        L.tsne_hip_repulsive_kept.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]
         L.tsne_hip_update.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, c_float, _vp, c_float, c_float, _vp]
         L.tsne_hip_iterate.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, c_int, c_int, c_int, c_float, c_float,
                                        c_float, c_float, _vp, _vp]
@@ -274,7 +275,7 @@ class Plan(object):
         self._csr = (row_ptr, col_idx, values)
         _check(lib().tsne_hip_plan_set_csr_pattern(self._h, _ptr(row_ptr), _ptr(col_idx), _ptr(values)))
 
-    def repulsive(self, embedding, details=False):
+    def repulsive(self, embedding, details=False, keep_grouping=False):
         n, g = self.num_points, self.n_nodes
         rep = torch.empty(2 * n, dtype=torch.float32, device=self.device)
         z = torch.empty(1, dtype=torch.float32, device=self.device)
@@ -283,8 +284,8 @@ class Plan(object):
             w = torch.empty((g, g, 4), dtype=torch.float32, device=self.device)
             yt = torch.empty((g, g, 4), dtype=torch.float32, device=self.device)
             phi = torch.empty((n, 4), dtype=torch.float32, device=self.device)
-        _check(lib().tsne_hip_repulsive(self._h, _ptr(_f32(embedding)), _ptr(rep), _ptr(z), _ptr(w), _ptr(yt),
-                                        _ptr(phi), _stream()))
+        fn = lib().tsne_hip_repulsive_kept if keep_grouping else lib().tsne_hip_repulsive
+        _check(fn(self._h, _ptr(_f32(embedding)), _ptr(rep), _ptr(z), _ptr(w), _ptr(yt), _ptr(phi), _stream()))
         return (rep, z, w, yt, phi) if details else (rep, z)
 
     def update_(self, embedding, attr, rep, gains, old_forces, eta, normalization, momentum, exaggeration):
