@@ -27,7 +27,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 def traffic_from_profile(path):
     """HBM bytes per launch of the attractive kernel from the committed rocprofv3 summary: the per-kernel
     averages of its FETCH_SIZE and WRITE_SIZE passes, each scaled by what the same counter read for the plain
-    256 MiB device copy of the same run (262144 KiB read and written per launch)."""
+    256 MiB device copies of the same run (262144 KiB read and written per launch; the summary lists them as
+    `calibration_copy_256MiB`)."""
     if not os.path.exists(path):
         return None, None
     avg, copy_max = {}, {}
@@ -41,8 +42,8 @@ def traffic_from_profile(path):
             continue
         if f[0].startswith("attractive_blocked_kernel"):
             avg[f[-4]] = a
-        elif f[0] == "__amd_rocclr_copyBuffer":
-            copy_max[f[-4]] = m
+        elif f[0] == "calibration_copy_256MiB":
+            copy_max[f[-4]] = a
     if set(avg) != {"FETCH_SIZE", "WRITE_SIZE"} or set(copy_max) != {"FETCH_SIZE", "WRITE_SIZE"}:
         return None, None
     kib = 262144.0  # one calibration copy
