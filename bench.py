@@ -195,7 +195,7 @@ def main():
                                   "frac": flop / knn_s / 1e12 / 157.3, "tile_pairs_per_mille": knn_stats[2],
                                   "note": "fp32 matrix peak; time of the whole kNN call (sweep, re-rank, packing)"}
 
-    # One-shot stages that are HBM problems (bytes as SURVEY-style algorithmic traffic).
+    # One-shot stages that are HBM problems (algorithmic bytes: what the stage must read and write once).
     nnz = float(n) * k
     for name, secs, b in (("perplexity", perp_s, 8.0 * nnz), ("symmetrize", sym_s, 12.0 * nnz),
                           ("symmetrize_full", sym_full_s, 8.0 * nnz + 8.0 * nnz_sym + 4.0 * (n + 1))):

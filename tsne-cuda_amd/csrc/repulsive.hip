@@ -830,14 +830,14 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
 // spectrum column of each position is produced here from kernel_rows (one more
 // packed transform) so it never travels through memory.
 // ---------------------------------------------------------------------------
-// The two plane pairs go through the transforms together (40 KB of LDS): half as many stages one after
-// the other as with one pair at a time (24 KB, which would also fit beside the attractive kernel's
-// workgroup on a CU: no faster at a million points, 3-4 % slower per step from 5000 to 800000).
+// The two plane pairs go through the transforms together (41 KB of LDS): half as many passes one after
+// the other as with one pair at a time (25 KB, which would also fit beside the attractive kernel's
+// workgroup on a CU: 1 % slower at a million points, 3-4 % slower per step from 5000 to 800000).
 __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restrict__ row_spectra, int G,
                                                            const float *__restrict__ kernel_rows,
                                                            const float2 *__restrict__ twiddles,
                                                            float2 *__restrict__ col_results) {
-    // Twiddles come straight from memory.  Layout: [pair in flight][col], then the kernel columns.
+    // Layout: [pair in flight][col], then the kernel columns (every transform padded, see pad()).
     constexpr int kPairsInFlight = 2;
     constexpr int kData = 2 * kPairsInFlight;  // transforms of data per round
     __shared__ float2 s[kData + 1][kFftPad];
