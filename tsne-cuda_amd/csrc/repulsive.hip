@@ -60,43 +60,25 @@ __device__ __forceinline__ int xcd_row_block(int b, int blocks) {
 }
 inline int xcd_launch_blocks(int blocks) { return kXcds * ((blocks + kXcds - 1) / kXcds); }
 
-// The transforms of length 1024 are five radix-4 levels (sub-transform lengths 1024, 256, 64, 16, 4 forwards, the
-// same backwards for the inverse), run as three passes over the LDS: levels 1024 + 256 and 64 + 16 are fused - a
-// thread holds the 16 elements that the two levels combine among themselves in registers - and level 4 is a pass
-// of its own.  Data flow and element order are those of five in-place radix-4 passes; what the fusion saves is two
-// of the five trips through the LDS and two of the five barriers of what is a chain of dependent, latency-bound
-// steps.  The three twiddles a thread needs per level and butterfly depend on its number only (thread mod 64 is
-// the butterfly it works on in every transform it visits), so they are loaded once, ahead of the data, and stay
-// in registers.
+// The transforms of length 1024 are five in-place radix-4 passes over the LDS (sub-transform lengths 1024, 256, 64,
+// 16, 4 forwards - decimation in frequency, natural order in, base-4 digit-reversed order out - and the same
+// backwards for the inverse, decimation in time), 256 butterflies per transform and pass, a barrier after each.
 //
 // A transform occupies 1056 LDS slots: one slot of padding after every 32 elements, so that the strides the
-// levels use (64, 4 and 1 elements between the lanes of a wave, 8-byte elements) fall on different banks - with
-// a plain layout the lanes of the 16- and 4-point levels hit each bank eight deep.
+// passes use (256, 64, 16, 4 and 1 elements between a butterfly's inputs, 8-byte elements) fall on different
+// banks - with a plain layout the lanes of the 16- and 4-point passes hit each bank eight deep (forward row
+// pass 17 -> 15 us, column pass 22 -> 21 us, inverse row pass 17 -> 13.5 us at 390 rows; 5-8 % of the whole
+// fit of 5000 to 60000 points, where the chain of dependent launches is what a step costs).
+//
+// The twiddles come straight from memory (an 8 KB table that every CU keeps in its L1).
+//
+// Measured and not kept: passes 1024+256 and 64+16 fused (a thread holding 16 elements in registers, three trips
+// through the LDS instead of five): only 64 threads per transform have work in a fused pass, and the passes
+// came out 10-15 % slower than five passes that keep every thread busy.  The thread's fifteen twiddles loaded
+// once into registers ahead of the data (they are the same for every transform it visits): 1-2 us slower per
+// pass than loading them where they are used.
 constexpr int kFftPad = kFft + kFft / 32;
 __device__ __forceinline__ int pad(int i) { return i + (i >> 5); }
-
-struct StageTwiddles {
-    float2 a[2][4][3];  // fused pass 0 (lengths 1024 + 256) and 1 (64 + 16): level of length L, [element mod 4][power]
-    float2 b[2][3];     // ... level of length L / 4
-};
-__device__ __forceinline__ StageTwiddles load_twiddles(const float2 *tw, int tid) {
-    StageTwiddles t;
-    const int lane = tid & 63;
-#pragma unroll
-    for (int fs = 0; fs < 2; ++fs) {
-        const int log2L = kLog2Fft - 4 * fs;
-        const int q16 = 1 << (log2L - 4);
-        const int k = lane & (q16 - 1);
-        const int stride = kFft >> log2L;
-#pragma unroll
-        for (int jl = 0; jl < 4; ++jl)
-#pragma unroll
-            for (int pw = 0; pw < 3; ++pw) t.a[fs][jl][pw] = tw[(pw + 1) * (k + jl * q16) * stride];
-#pragma unroll
-        for (int pw = 0; pw < 3; ++pw) t.b[fs][pw] = tw[(pw + 1) * k * stride * 4];
-    }
-    return t;
-}
 
 // Radix-4 butterflies on four registers: decimation in frequency forwards (twiddles after the sums), decimation in
 // time for the inverse (conjugate twiddles first).
@@ -116,70 +98,41 @@ __device__ __forceinline__ void butterfly_inverse(float2 &x0, float2 &x1, float2
     x3 = make_float2(u1.x + u3.y, u1.y - u3.x);
 }
 
-// Fused pass FS over `nfft` transforms stored kFftPad slots apart: 64 threads per transform, 16 elements each.
-template <bool INVERSE, int FS>
-__device__ __forceinline__ void radix16_pass(float2 *s, int nfft, const StageTwiddles &tw, int tid, int nthreads) {
-    constexpr int log2L = kLog2Fft - 4 * FS;
-    constexpr int L = 1 << log2L, q16 = L >> 4;
-    for (int id = tid; id < nfft * 64; id += nthreads) {
-        const int f = id >> 6, t = id & 63;  // t == tid & 63: nthreads is a multiple of 64
-        const int k = t & (q16 - 1), b = t >> (log2L - 4);
-        float2 *base = s + f * kFftPad;
-        const int i0 = b * L + k;
-        float2 x[16];
-#pragma unroll
-        for (int j = 0; j < 16; ++j) x[j] = base[pad(i0 + j * q16)];
-        if (!INVERSE) {
-#pragma unroll
-            for (int jl = 0; jl < 4; ++jl) butterfly_forward(x[jl], x[jl + 4], x[jl + 8], x[jl + 12], tw.a[FS][jl]);
-#pragma unroll
-            for (int m = 0; m < 4; ++m) butterfly_forward(x[4 * m], x[4 * m + 1], x[4 * m + 2], x[4 * m + 3], tw.b[FS]);
-        } else {
-#pragma unroll
-            for (int m = 0; m < 4; ++m) butterfly_inverse(x[4 * m], x[4 * m + 1], x[4 * m + 2], x[4 * m + 3], tw.b[FS]);
-#pragma unroll
-            for (int jl = 0; jl < 4; ++jl) butterfly_inverse(x[jl], x[jl + 4], x[jl + 8], x[jl + 12], tw.a[FS][jl]);
-        }
-#pragma unroll
-        for (int j = 0; j < 16; ++j) base[pad(i0 + j * q16)] = x[j];
-    }
-}
-
-// The level of length 4 (no twiddles): 256 threads per transform, four neighbouring elements each.
+// One pass (sub-transform length L = 2^log2L) over `nfft` transforms stored kFftPad slots apart.
 template <bool INVERSE>
-__device__ __forceinline__ void radix4_last_pass(float2 *s, int nfft, int tid, int nthreads) {
-    const float2 one[3] = {make_float2(1.f, 0.f), make_float2(1.f, 0.f), make_float2(1.f, 0.f)};
+__device__ __forceinline__ void radix4_pass(float2 *s, int nfft, int log2L, const float2 *tw, int tid, int nthreads) {
+    const int L = 1 << log2L, q4 = L >> 2, log2q4 = log2L - 2, stride = kFft >> log2L;
     for (int id = tid; id < nfft * (kFft / 4); id += nthreads) {
         const int f = id >> 8, q = id & 255;
+        const int k = q & (q4 - 1), b = q >> log2q4;
         float2 *base = s + f * kFftPad;
-        float2 x0 = base[pad(4 * q)], x1 = base[pad(4 * q + 1)], x2 = base[pad(4 * q + 2)], x3 = base[pad(4 * q + 3)];
+        const int i0 = b * L + k;
+        const float2 w[3] = {tw[k * stride], tw[2 * k * stride], tw[3 * k * stride]};
+        float2 x0 = base[pad(i0)], x1 = base[pad(i0 + q4)], x2 = base[pad(i0 + 2 * q4)], x3 = base[pad(i0 + 3 * q4)];
         if (!INVERSE)
-            butterfly_forward(x0, x1, x2, x3, one);
+            butterfly_forward(x0, x1, x2, x3, w);
         else
-            butterfly_inverse(x0, x1, x2, x3, one);
-        base[pad(4 * q)] = x0;
-        base[pad(4 * q + 1)] = x1;
-        base[pad(4 * q + 2)] = x2;
-        base[pad(4 * q + 3)] = x3;
+            butterfly_inverse(x0, x1, x2, x3, w);
+        base[pad(i0)] = x0;
+        base[pad(i0 + q4)] = x1;
+        base[pad(i0 + 2 * q4)] = x2;
+        base[pad(i0 + 3 * q4)] = x3;
     }
 }
 
-// Forward: natural order in, base-4 digit-reversed order out; inverse: the other way round.  Both end with a barrier.
-__device__ __forceinline__ void fft_forward(float2 *s, int nfft, const StageTwiddles &tw, int tid, int nthreads) {
-    radix16_pass<false, 0>(s, nfft, tw, tid, nthreads);
-    __syncthreads();
-    radix16_pass<false, 1>(s, nfft, tw, tid, nthreads);
-    __syncthreads();
-    radix4_last_pass<false>(s, nfft, tid, nthreads);
-    __syncthreads();
+__device__ __forceinline__ void fft_forward(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+#pragma unroll
+    for (int l = kLog2Fft; l >= 2; l -= 2) {
+        radix4_pass<false>(s, nfft, l, tw, tid, nthreads);
+        __syncthreads();
+    }
 }
-__device__ __forceinline__ void fft_inverse(float2 *s, int nfft, const StageTwiddles &tw, int tid, int nthreads) {
-    radix4_last_pass<true>(s, nfft, tid, nthreads);
-    __syncthreads();
-    radix16_pass<true, 1>(s, nfft, tw, tid, nthreads);
-    __syncthreads();
-    radix16_pass<true, 0>(s, nfft, tw, tid, nthreads);
-    __syncthreads();
+__device__ __forceinline__ void fft_inverse(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+#pragma unroll
+    for (int l = 2; l <= kLog2Fft; l += 2) {
+        radix4_pass<true>(s, nfft, l, tw, tid, nthreads);
+        __syncthreads();
+    }
 }
 
 struct Bounds {
@@ -737,7 +690,7 @@ __device__ __forceinline__ float kernel_value(float lo, float h, int a, int b) {
 
 template <int THREADS>
 __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *sc, int slot, int n_boxes,
-                                                  const StageTwiddles &tw, float *__restrict__ kernel_rows,
+                                                  const float2 *__restrict__ tw, float *__restrict__ kernel_rows,
                                                   float2 (*s)[kFftPad]) {
     const int tid = threadIdx.x;
     const int G = n_boxes * kInterp;
@@ -785,7 +738,7 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
                                                                        float *__restrict__ kernel_rows) {
     constexpr int kThreads = 256 * ROWS;
     __shared__ float2 s[2 * ROWS][kFftPad];  // [row * 2 + pair]
-    const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
+    const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     // The workgroups past the rows produce the kernel's row spectra (needed by the column
     // pass only): the two jobs are independent and share the launch.
@@ -841,7 +794,7 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
     constexpr int kPairsInFlight = 2;
     constexpr int kData = 2 * kPairsInFlight;  // transforms of data per round
     __shared__ float2 s[kData + 1][kFftPad];
-    const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
+    const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int c0 = blockIdx.x * 2;
     {
@@ -896,7 +849,7 @@ __global__ __launch_bounds__(kRowThreads) void conv_rows_inverse_kernel(const fl
                                                                 const float2 *__restrict__ twiddles,
                                                                 float4 *__restrict__ node_potentials) {
     __shared__ float2 s[4][kFftPad];  // [row * 2 + pair]
-    const StageTwiddles tw = load_twiddles(twiddles, threadIdx.x);
+    const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int row_block = xcd_row_block(blockIdx.x, (G + 1) / 2);
     if (row_block < 0) return;
