@@ -331,6 +331,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
         int cus = 256;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, p->device) != hipSuccess) cus = 256;
         p->spread_grid = 2 * cus;  // 512 threads and 14 KB of LDS each: two fit beside the attractive kernel's workgroup
+        p->stream_grid = cus + cus / 2;
     }
     // yxy carries one spare pair so that two-point (float4) loads may straddle the end.
     bool ok = hipMalloc(&p->yxy, sizeof(float2) * (N + 2)) == hipSuccess &&
