@@ -130,15 +130,15 @@ int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *e
     hipStream_t side = p->side_stream;
     TSNE_TRY(hipEventRecord(p->fork_event, s));  // everything up to the previous step's update
     TSNE_TRY(hipStreamWaitEvent(side, p->fork_event, 0));
-    // Where the attractive kernel's workgroups (one per compute unit, 125 KB of LDS each) cover a good part of
-    // the device, the kernel is enqueued before the chain (in a captured graph: its node comes first), so that
-    // they are placed while the units are empty.  Enqueued after the chain's nine kernels it started 10 us
-    // later, and on every unit above the LDS block of a workgroup of the chain's first kernels: the 35 KB left
-    // on a unit were then in two pieces, neither large enough for a workgroup of the row passes (33 KB), which
-    // waited for the attractive kernel to end.  Smaller problems wait for the chain, not for the attractive
-    // kernel, and lose by the chain's later start (measured: 3 % slower at 50000 points, even at 200000,
-    // 1 % faster at 400000, 4 % at 800000).
-    const bool attractive_first = !pij && !p->csr_row_ptr && p->blocked_ready && p->n_strips * 4 >= p->num_cus;
+    // Where the attractive kernel's workgroups (one per compute unit) hold strips of a thousand rows and more
+    // (a quarter of a million points and up: as much as 125 KB of LDS each), the kernel is enqueued before the
+    // chain (in a captured graph: its node comes first), so that they are placed while the units are empty.
+    // Enqueued after the chain's nine kernels it started 10 us later, and on every unit above the LDS block of
+    // a workgroup of the chain's first kernels: the 35 KB left on a unit were then in two pieces, neither large
+    // enough for a workgroup of the row passes (33 KB), which waited for the attractive kernel to end.  Smaller
+    // problems wait for the chain, not for the attractive kernel, and lose by the chain's later start
+    // (measured: 3-10 % slower from 5000 to 60000 points, even at 200000, 1 % faster at 400000, 4 % at 800000).
+    const bool attractive_first = !pij && !p->csr_row_ptr && p->blocked_ready && p->strip_rows >= 1024;
     if (attractive_first && launch_step_attractive(p, pij, indices, s)) return 1;
     if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, side, true)) return 1;
     if (normalization && launch_finish_z(p, normalization, side)) return 1;
