@@ -64,11 +64,13 @@ inline int xcd_launch_blocks(int blocks) { return kXcds * ((blocks + kXcds - 1) 
 // 16, 4 forwards - decimation in frequency, natural order in, base-4 digit-reversed order out - and the same
 // backwards for the inverse, decimation in time), 256 butterflies per transform and pass, a barrier after each.
 //
-// A transform occupies 1056 LDS slots: one slot of padding after every 32 elements, so that the strides the
-// passes use (256, 64, 16, 4 and 1 elements between a butterfly's inputs, 8-byte elements) fall on different
-// banks - with a plain layout the lanes of the 16- and 4-point passes hit each bank eight deep (forward row
-// pass 17 -> 15 us, column pass 22 -> 21 us, inverse row pass 17 -> 13.5 us at 390 rows; 5-8 % of the whole
-// fit of 5000 to 60000 points, where the chain of dependent launches is what a step costs).
+// A transform occupies its 1024 LDS slots in a swizzled order: element i sits in slot pad(i), which exchanges
+// bits among the low five of i (bit 4 is added into bits 0 and 2, bit 5 into bits 1 and 3, bit 6 into bit 4), so
+// that the strides the passes use (256, 64, 16, 4 and 1 elements between the butterflies of neighbouring lanes,
+// 8-byte elements) fall on different banks, whether the LDS serves 16 or 32 lanes of an 8-byte access at a time.
+// With a plain layout the lanes of the 16- and 4-point passes hit each bank eight deep (forward row pass
+// 17 -> 15 us, column pass 22 -> 21 us, inverse row pass 17 -> 13.5 us at 390 rows; 5-8 % of the whole fit of
+// 5000 to 60000 points, where the chain of dependent launches is what a step costs).
 //
 // The twiddles come straight from memory (an 8 KB table that every CU keeps in its L1).
 //
@@ -77,8 +79,10 @@ inline int xcd_launch_blocks(int blocks) { return kXcds * ((blocks + kXcds - 1) 
 // came out 10-15 % slower than five passes that keep every thread busy.  The thread's fifteen twiddles loaded
 // once into registers ahead of the data (they are the same for every transform it visits): 1-2 us slower per
 // pass than loading them where they are used.
-constexpr int kFftPad = kFft + kFft / 32;
-__device__ __forceinline__ int pad(int i) { return i + (i >> 5); }
+constexpr int kFftPad = kFft;  // slots per transform
+__device__ __forceinline__ int pad(int i) {
+    return i ^ (((i >> 4) & 1) * 5) ^ (((i >> 5) & 1) * 10) ^ (((i >> 6) & 1) << 4);
+}
 
 // Radix-4 butterflies on four registers: decimation in frequency forwards (twiddles after the sums), decimation in
 // time for the inverse (conjugate twiddles first).
@@ -445,7 +449,9 @@ constexpr int kStrayShift = 10;  // ... and only while at most N / 2^10 points s
 constexpr int kStrayFloor = 128; // or 128 of a small problem's
 __device__ __forceinline__ constexpr int moment_index(int i, int j) { return j <= 2 ? j * 5 + i : 15 + (j - 3) * 3 + i; }
 
-__global__ __launch_bounds__(kSpreadThreads) void spread_kernel(const float2 *__restrict__ tile_xy,
+// (At most 128 registers, whatever the compiler would like: beside the attractive kernel's sixteen waves of 64
+// registers a compute unit has room for eight waves of 128, one workgroup of this kernel, and for none of more.)
+__global__ __launch_bounds__(kSpreadThreads, 4) void spread_kernel(const float2 *__restrict__ tile_xy,
                                                      const int *__restrict__ tile_perm,
                                                      const float2 *__restrict__ yxy, int4 *chunks,
                                                      const int *__restrict__ num_chunks, LoopScalars *sc,
