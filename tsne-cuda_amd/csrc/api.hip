@@ -134,8 +134,8 @@ int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *e
     // (a quarter of a million points and up: as much as 125 KB of LDS each), the kernel is enqueued before the
     // chain (in a captured graph: its node comes first), so that they are placed while the units are empty.
     // Enqueued after the chain's nine kernels it started 10 us later, and on every unit above the LDS block of
-    // a workgroup of the chain's first kernels: the 35 KB left on a unit were then in two pieces, neither large
-    // enough for a workgroup of the row passes (33 KB), which waited for the attractive kernel to end.  Smaller
+    // a workgroup of the chain's first kernels: the 34 KB left on a unit were then in two pieces, neither large
+    // enough for a workgroup of the row passes (32 KB), which waited for the attractive kernel to end.  Smaller
     // problems wait for the chain, not for the attractive kernel, and lose by the chain's later start
     // (measured: 3-10 % slower from 5000 to 60000 points, even at 200000, 1 % faster at 400000, 4 % at 800000).
     const bool attractive_first = !pij && !p->csr_row_ptr && p->blocked_ready && p->strip_rows >= 1024;

@@ -731,10 +731,10 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
 // charges it consumed so that the next step starts from zero without a memset.  Output is transposed:
 // row_spectra[pair][pos][m], pos = digit-reversed frequency position.
 //
-// Two rows per workgroup (512 threads, 32 KB of LDS) is what the loop uses.  One row per workgroup (256 threads,
-// 16 KB, so that two fit into the 35 KB of LDS a CU has left beside the attractive kernel's workgroup and the
-// whole launch is resident at once) measured 51 us against 61 us beside that kernel and 21 us against 17 us
-// alone, and 2 % fewer iterations per second: what slows the pass down there is not the number of rounds.
+// Two rows per workgroup (512 threads, 32 KB of LDS) is what the loop uses: one such workgroup fits into the 34 KB
+// of LDS (27 allocation units of 1280 bytes) that a workgroup of the attractive kernel leaves on a compute unit,
+// provided those are in one piece (the loop enqueues the attractive kernel first for that reason).  One row per
+// workgroup (256 threads, 16 KB) measured 21 us against 17 us alone and 2 % fewer iterations per second.
 // ---------------------------------------------------------------------------
 template <int ROWS>
 __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *__restrict__ w, int G, int n_boxes,
@@ -789,8 +789,8 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
 // spectrum column of each position is produced here from kernel_rows (one more
 // packed transform) so it never travels through memory.
 // ---------------------------------------------------------------------------
-// The two plane pairs go through the transforms together (41 KB of LDS): half as many passes one after
-// the other as with one pair at a time (25 KB, which would also fit beside the attractive kernel's
+// The two plane pairs go through the transforms together (40 KB of LDS): half as many passes one after
+// the other as with one pair at a time (24 KB, which would also fit beside the attractive kernel's
 // workgroup on a CU: 1 % slower at a million points, 3-4 % slower per step from 5000 to 800000).
 __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restrict__ row_spectra, int G,
                                                            const float *__restrict__ kernel_rows,
