@@ -290,8 +290,10 @@ __device__ __forceinline__ void count_wave(unsigned int *counter, int lane) {
 
 // RUNTIME_LIMIT: the poll limit is the argument (the override for tests); otherwise it is the constant, with
 // which the compiler lays the wait loops out better (197 against 203 us per launch at a million points).
+// At most 64 registers (the second launch bound): the kernel's sixteen waves then take half of a compute unit's
+// register file and leave room for the eight waves of 128 registers of a spreading workgroup beside them.
 template <bool RUNTIME_LIMIT>
-__global__ __launch_bounds__(kBlock) void attractive_blocked_kernel(const float *__restrict__ ent_p,
+__global__ __launch_bounds__(kBlock, 8) void attractive_blocked_kernel(const float *__restrict__ ent_p,
                                                                     const unsigned int *__restrict__ seg,
                                                                     const float2 *__restrict__ yxy,
                                                                     LoopScalars *__restrict__ scalars,
