@@ -102,12 +102,21 @@ static bool overlap_enabled() {
     return on;
 }
 
-// Overlapped form: the side stream carries chain(k) (the repulsive kernels), the caller's stream carries
-// attractive(k), update(k), attractive(k+1), ...: chain(k) waits for update(k-1) (an event recorded on the
-// caller's stream) and update(k) for chain(k), one event each way per step.  The attractive kernel of the next
-// step follows the update on its own stream without a hand-over, and every step leaves the caller's stream
-// joined with the side stream.  (With the update on the side stream behind the chain, as it was while the
-// attractive kernel was the longer of the two, a step took 2 % longer.)
+// Overlapped form: a step's repulsive chain and its attractive kernel run on two streams, the update behind the
+// chain on the chain's stream.  A dependency between two kernels of one stream costs 2-3 us, one across streams
+// about 9 us when the waiting stream gets there before the event has fired (measured between the chain's last
+// kernel and an update on the other stream) and next to nothing when it fired long before.  So the transitions
+// a step waits for are kept inside a stream:
+//  * problems whose step is its chain (up to a quarter of a million points): chain(k), update(k), chain(k+1) ...
+//    on the caller's stream, the attractive kernel on the side stream (it starts 9 us late and has the time);
+//  * larger ones, whose step is the attractive kernel and what of the chain cannot run beside it: the attractive
+//    kernel of step k+1 follows update(k) on the same stream, so chain and attractive kernel change streams every
+//    step (pairs of steps, see launch_steps); a single step keeps the chain on the side stream and the attractive
+//    kernel and the update on the caller's.
+// Every form leaves the caller's stream joined with the side stream.  (Measured without captured graphs, where the
+// streams are what the hardware queues see: fits of 5000-60000 points 15 % shorter than with the update on the
+// attractive kernel's stream, a million points 2.8 % more iterations per second.  A captured graph holds the same
+// dependencies whichever stream they were recorded on and runs as before.)
 // Attractive forces of a step: the explicit N x K pattern if given, else the plan's CSR pattern if one is set,
 // else the re-blocked pattern.
 static int launch_step_attractive(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s) {
@@ -116,11 +125,45 @@ static int launch_step_attractive(tsne_hip_plan *p, const float *pij, const int 
     return launch_attractive_blocked(p, p->attr, s);
 }
 
+static bool overlap_active(const tsne_hip_plan *p) {
+    return overlap_enabled() && !p->profiling && p->side_stream != nullptr;
+}
+
+// Where the attractive kernel's workgroups (one per compute unit) hold strips of a thousand rows and more (a
+// quarter of a million points and up: as much as 125 KB of LDS each), a step is that kernel plus what of the
+// chain cannot run beside it, and the kernel is enqueued before the chain (in a captured graph: its node comes
+// first), so that its workgroups are placed while the units are empty.  Enqueued after the chain's nine kernels
+// it started 10 us later, and on every unit above the LDS block of a workgroup of the chain's first kernels:
+// the 34 KB left on a unit were then in two pieces, neither large enough for a workgroup of the row passes
+// (32 KB), which waited for the attractive kernel to end.  Smaller problems wait for the chain, not for the
+// attractive kernel, and lose by the chain's later start (measured: 3-10 % slower from 5000 to 60000 points,
+// even at 200000, 1 % faster at 400000, 4 % at 800000).
+static bool attractive_is_critical(const tsne_hip_plan *p, const float *pij) {
+    return !pij && !p->csr_row_ptr && p->blocked_ready && p->strip_rows >= 1024;
+}
+
+// One overlapped step: chain and update on `cs`, attractive kernel on `as`; `prev` (one of the two) is the stream
+// whose work so far includes the update before.
+static int launch_step_on(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
+                          float *old_forces, float eta, float momentum, float exaggeration, int slot,
+                          float *normalization, hipStream_t cs, hipStream_t as, hipStream_t prev,
+                          bool attractive_first) {
+    TSNE_TRY(hipEventRecord(p->fork_event, prev));
+    TSNE_TRY(hipStreamWaitEvent(prev == cs ? as : cs, p->fork_event, 0));
+    if (attractive_first && launch_step_attractive(p, pij, indices, as)) return 1;
+    if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, cs, true)) return 1;
+    if (normalization && launch_finish_z(p, normalization, cs)) return 1;
+    if (!attractive_first && launch_step_attractive(p, pij, indices, as)) return 1;
+    TSNE_TRY(hipEventRecord(p->join_event, as));
+    TSNE_TRY(hipStreamWaitEvent(cs, p->join_event, 0));
+    return launch_update(p, embedding, p->attr, p->rep, gains, old_forces, eta, nullptr, momentum, exaggeration,
+                         slot ^ 1, cs);
+}
+
 int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
                 float *old_forces, float eta, float momentum, float exaggeration, int slot, float *normalization,
                 hipStream_t s) {
-    const bool overlap = overlap_enabled() && !p->profiling && p->side_stream != nullptr;
-    if (!overlap) {
+    if (!overlap_active(p)) {
         if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, s, true)) return 1;
         if (launch_step_attractive(p, pij, indices, s)) return 1;
         if (normalization && launch_finish_z(p, normalization, s)) return 1;
@@ -128,25 +171,36 @@ int launch_step(tsne_hip_plan *p, const float *pij, const int *indices, float *e
                              slot ^ 1, s);
     }
     hipStream_t side = p->side_stream;
+    if (!attractive_is_critical(p, pij))
+        return launch_step_on(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot,
+                              normalization, s, side, s, false);
     TSNE_TRY(hipEventRecord(p->fork_event, s));  // everything up to the previous step's update
     TSNE_TRY(hipStreamWaitEvent(side, p->fork_event, 0));
-    // Where the attractive kernel's workgroups (one per compute unit) hold strips of a thousand rows and more
-    // (a quarter of a million points and up: as much as 125 KB of LDS each), the kernel is enqueued before the
-    // chain (in a captured graph: its node comes first), so that they are placed while the units are empty.
-    // Enqueued after the chain's nine kernels it started 10 us later, and on every unit above the LDS block of
-    // a workgroup of the chain's first kernels: the 34 KB left on a unit were then in two pieces, neither large
-    // enough for a workgroup of the row passes (32 KB), which waited for the attractive kernel to end.  Smaller
-    // problems wait for the chain, not for the attractive kernel, and lose by the chain's later start
-    // (measured: 3-10 % slower from 5000 to 60000 points, even at 200000, 1 % faster at 400000, 4 % at 800000).
-    const bool attractive_first = !pij && !p->csr_row_ptr && p->blocked_ready && p->strip_rows >= 1024;
-    if (attractive_first && launch_step_attractive(p, pij, indices, s)) return 1;
+    if (launch_step_attractive(p, pij, indices, s)) return 1;
     if (launch_repulsive(p, embedding, slot, p->rep, nullptr, nullptr, side, true)) return 1;
     if (normalization && launch_finish_z(p, normalization, side)) return 1;
     TSNE_TRY(hipEventRecord(p->join_event, side));
-    if (!attractive_first && launch_step_attractive(p, pij, indices, s)) return 1;
     TSNE_TRY(hipStreamWaitEvent(s, p->join_event, 0));
     return launch_update(p, embedding, p->attr, p->rep, gains, old_forces, eta, nullptr, momentum, exaggeration,
                          slot ^ 1, s);
+}
+
+// Two steps; where the attractive kernel is what a step waits for, with the streams' parts exchanged between them
+// (the first step's update runs on the side stream and the second step's attractive kernel follows it there; the
+// second step's update runs on the caller's stream again).
+static int launch_two_steps(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
+                            float *old_forces, float eta, float momentum, float exaggeration, int slot,
+                            hipStream_t s) {
+    // (with more strips than compute units the attractive kernel runs in rounds and the exchange measured 2 % slower)
+    if (overlap_active(p) && attractive_is_critical(p, pij) && p->n_strips <= p->num_cus) {
+        hipStream_t side = p->side_stream;
+        return launch_step_on(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot, nullptr,
+                              side, s, s, true) ||
+               launch_step_on(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot ^ 1,
+                              nullptr, s, side, side, true);
+    }
+    return launch_step(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot, nullptr, s) ||
+           launch_step(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot ^ 1, nullptr, s);
 }
 
 // Replaying a captured graph saves launch gaps wherever the chain of nine short kernels is what a step waits for.
@@ -173,10 +227,8 @@ int launch_steps(tsne_hip_plan *p, const float *pij, const int *indices, float *
             // Capture two steps (the bounds slot is back where it started) including the side stream's part.
             hipGraph_t graph = nullptr;
             TSNE_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
-            int rc = launch_step(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot,
-                                 nullptr, s);
-            rc = rc || launch_step(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration,
-                                   slot ^ 1, nullptr, s);
+            const int rc =
+                launch_two_steps(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot, s);
             const hipError_t end = hipStreamEndCapture(s, &graph);
             if (rc) {
                 if (graph) (void)hipGraphDestroy(graph);
@@ -191,7 +243,10 @@ int launch_steps(tsne_hip_plan *p, const float *pij, const int *indices, float *
         }
         for (; count >= 2; count -= 2) TSNE_TRY(hipGraphLaunch(exec, s));
     }
-    for (; count > 0; --count) {
+    for (; count >= 2; count -= 2)  // (the bounds slot is back where it started after two steps)
+        if (launch_two_steps(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot, s))
+            return 1;
+    if (count > 0) {
         if (launch_step(p, pij, indices, embedding, gains, old_forces, eta, momentum, exaggeration, slot, nullptr, s))
             return 1;
         slot ^= 1;
