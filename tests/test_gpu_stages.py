@@ -563,10 +563,13 @@ def test_attractive_wait_that_runs_out_is_reported(stages, monkeypatch):
     plan.close()
 
 
-def test_iterate_after_preparing_a_second_pattern(stages, c0_problem):
+def test_iterate_after_preparing_a_second_pattern(stages, c0_problem, monkeypatch):
     """Steps replay captured graphs, which hold the addresses of the re-blocked
     pattern: preparing another pattern in the same plan must drop them.  The
-    second run has to follow the second pattern, like a fresh plan does."""
+    second run has to follow the second pattern, like a fresh plan does.
+    (Problems of this size run without graphs and on one stream unless told otherwise.)"""
+    monkeypatch.setenv("TSNE_GRAPH", "1")
+    monkeypatch.setenv("TSNE_OVERLAP", "1")
     c = c0_problem
     n, k = c["P"].shape
     dP, di = dev(c["P"]), dev(c["idx"])
@@ -592,10 +595,13 @@ def test_iterate_after_preparing_a_second_pattern(stages, c0_problem):
     assert rel_l2(twice, once) <= 1e-5
 
 
-def test_plan_closed_or_reprepared_while_steps_are_in_flight(stages, c0_problem):
-    """iterate_ returns while its steps (a replaying graph here) still run.  Closing the
-    plan, or preparing another pattern in it, right away - no synchronisation in
+@pytest.mark.parametrize("graph, overlap", [("1", "1"), ("0", "1"), ("0", "0")])
+def test_plan_closed_or_reprepared_while_steps_are_in_flight(stages, c0_problem, monkeypatch, graph, overlap):
+    """iterate_ returns while its steps (a replaying graph, eager steps on two streams, or on one) still run.
+    Closing the plan, or preparing another pattern in it, right away - no synchronisation in
     between - must wait for them: the embedding ends where a synchronised run ends."""
+    monkeypatch.setenv("TSNE_GRAPH", graph)
+    monkeypatch.setenv("TSNE_OVERLAP", overlap)
     c = c0_problem
     n, k = c["P"].shape
     dP, di = dev(c["P"]), dev(c["idx"])
@@ -866,9 +872,9 @@ def test_knn_few_failed_queries_are_redone_by_candidate_range(stages):
 
 
 def test_iterate_graph_replay_matches_eager(stages, c0_problem, monkeypatch):
-    """Small problems replay a captured graph of two steps.  Replays, with eager
-    work and synchronisations between them, give what the eager loop gives (to
-    the repeatability of the loop itself: its float atomics are unordered)."""
+    """Steps on one stream or two, launched one by one or as replays of a captured graph of two
+    steps, with eager work and synchronisations between the calls, give what the plain loop gives
+    (to the repeatability of the loop itself: its float atomics are unordered)."""
     c = c0_problem
     n = c["P"].shape[0]
     dP, di = dev(c["P"]), dev(c["idx"])
@@ -888,11 +894,18 @@ def test_iterate_graph_replay_matches_eager(stages, c0_problem, monkeypatch):
         plan.close()
         return out
 
+    # (problems of this size run on one stream and without graphs unless told otherwise)
     monkeypatch.setenv("TSNE_GRAPH", "0")
+    monkeypatch.setenv("TSNE_OVERLAP", "0")
     eager = run([12])
-    monkeypatch.setenv("TSNE_GRAPH", "1")
-    replayed = run([5, 4, 3])  # 2 + 2 + 1 replays of the same graph, odd remainders eager
-    assert np.isfinite(replayed).all()
-    assert rel_l2(replayed, eager) <= 1e-3
     oracle_y, _ = oracle.iterate(c["P"], c["idx"], c["y0"], 12)
-    assert rel_l2(replayed, oracle_y) <= 1e-3
+    for overlap in ("1", "0"):
+        monkeypatch.setenv("TSNE_OVERLAP", overlap)
+        monkeypatch.setenv("TSNE_GRAPH", "0")
+        stepped = run([5, 4, 3])
+        monkeypatch.setenv("TSNE_GRAPH", "1")
+        replayed = run([5, 4, 3])  # 2 + 2 + 1 replays of the same graph, odd remainders eager
+        for got in (stepped, replayed):
+            assert np.isfinite(got).all()
+            assert rel_l2(got, eager) <= 1e-3
+            assert rel_l2(got, oracle_y) <= 1e-3

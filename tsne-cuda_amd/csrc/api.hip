@@ -94,12 +94,16 @@ int check_plan(const tsne_hip_plan *p, const char *who) {
 
 namespace tsnehip {
 
-static bool overlap_enabled() {
-    static const bool on = [] {
-        const char *v = std::getenv("TSNE_OVERLAP");
-        return !(v && v[0] == '0');
-    }();
-    return on;
+// Up to this many points a step is a chain of short dependent kernels that the attractive kernel hardly
+// lengthens: one stream without events and without a captured graph is then the fastest form (fits of 5000, 60000
+// and 50000 points 5 %, 3.5 % and 2.7 % shorter than with two streams and graphs, whose events cost 7-10 us per
+// step and whose instantiation 4 ms per stretch of constant parameters; at 100000 points two streams are 4 % ahead).
+constexpr int kSingleStreamPoints = 65536;
+
+// TSNE_OVERLAP: 0 never, 1 always, unset: by the size of the problem.
+static bool overlap_enabled(const tsne_hip_plan *p) {
+    const char *v = std::getenv("TSNE_OVERLAP");  // read on every call, like TSNE_GRAPH
+    return v ? v[0] != '0' : p->num_points > kSingleStreamPoints;
 }
 
 // Overlapped form: a step's repulsive chain and its attractive kernel run on two streams, the update behind the
@@ -126,7 +130,7 @@ static int launch_step_attractive(tsne_hip_plan *p, const float *pij, const int 
 }
 
 static bool overlap_active(const tsne_hip_plan *p) {
-    return overlap_enabled() && !p->profiling && p->side_stream != nullptr;
+    return overlap_enabled(p) && !p->profiling && p->side_stream != nullptr;
 }
 
 // Where the attractive kernel's workgroups (one per compute unit) hold strips of a thousand rows and more (a
@@ -208,9 +212,10 @@ static bool graphs_enabled(const tsne_hip_plan *p) {
     const char *v = std::getenv("TSNE_GRAPH");  // read on every call: cheap, and lets one process try both
     const int mode = v ? (v[0] == '0' ? 0 : 1) : -1;
     if (p->profiling || sync_kernels_enabled() || mode == 0) return false;
-    // Measured gain per step: 15 % at 5000-60000 points, 2-3.5 % at 400000-800000, 0.3 % at a million; setting a
-    // graph up costs about 4 ms whatever the size.
-    return mode == 1 || p->num_points <= 1048576;
+    // Measured gain per step beside two streams without a graph: 2 % at 100000 points, 0-0.5 % from 200000 to a
+    // million (and none against one stream up to kSingleStreamPoints); setting a graph up costs about 4 ms
+    // whatever the size.
+    return mode == 1 || (p->num_points > kSingleStreamPoints && p->num_points <= 1048576);
 }
 
 int launch_steps(tsne_hip_plan *p, const float *pij, const int *indices, float *embedding, float *gains,
