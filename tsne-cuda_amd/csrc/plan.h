@@ -60,7 +60,7 @@ struct tsne_hip_plan {
     int4 *chunks = nullptr;        // (tile, first point, count, box offset of the first point in the tile's LDS region)
     int *num_chunks = nullptr;  // [0] chunks of the current step, [1] ticket counter of the tile count kernel
     int max_chunks = 0;
-    int spread_grid = 512;         // workgroups of the spreading kernel (two per CU)
+    int spread_grid = 256;         // workgroups of the spreading kernel (one per CU)
     int num_cus = 256;            // compute units of the device
     int stream_grid = 384;        // workgroups of the kernels that only stream arrays (update): 1.5 per compute unit
     const float *loop_embedding = nullptr;  // where tsne_hip_iterate last left off: the buffer and the step after its last
