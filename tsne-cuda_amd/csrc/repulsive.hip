@@ -795,17 +795,24 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
 // spectrum column of each position is produced here from kernel_rows (one more
 // packed transform) so it never travels through memory.
 // ---------------------------------------------------------------------------
-// The two plane pairs go through the transforms together (40 KB of LDS): half as many passes one after
-// the other as with one pair at a time (24 KB, which would also fit beside the attractive kernel's
-// workgroup on a CU: 1 % slower at a million points, 3-4 % slower per step from 5000 to 800000).
+// The two plane pairs go through the transforms together: half as many passes one after the other as with one
+// pair at a time (24 KB of LDS: 1 % slower at a million points, 3-4 % slower per step from 5000 to 800000).
+//
+// SLIM = false: the kernel's columns are transformed with the data, as a fifth transform (40 KB of LDS).
+// SLIM = true: they are transformed first, on their own, and their spectrum kept in registers (a thread multiplies
+// the same two positions of every transform), so the workgroup holds four transforms: 32 KB, the 26 allocation
+// units of LDS that fit beside a workgroup of the attractive kernel (27 free), where 40 KB do not.  The extra pass
+// has work for half the threads and costs 1.5 us alone.
+template <bool SLIM>
 __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restrict__ row_spectra, int G,
                                                            const float *__restrict__ kernel_rows,
                                                            const float2 *__restrict__ twiddles,
                                                            float2 *__restrict__ col_results) {
-    // Layout: [pair in flight][col], then the kernel columns (every transform padded, see pad()).
+    // Layout: [pair in flight][col], then (SLIM = false) the kernel columns; every transform swizzled, see pad().
     constexpr int kPairsInFlight = 2;
     constexpr int kData = 2 * kPairsInFlight;  // transforms of data per round
-    __shared__ float2 s[kData + 1][kFftPad];
+    constexpr int kKernelSlot = SLIM ? 0 : kData;
+    __shared__ float2 s[SLIM ? kData : kData + 1][kFftPad];
     const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int c0 = blockIdx.x * 2;
@@ -820,8 +827,16 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
                 v.x = kernel_rows[(size_t)v0 * kNodePad + a];
                 v.y = kernel_rows[(size_t)v1 * kNodePad + a];
             }
-            s[kData][pad(m)] = v;
+            s[kKernelSlot][pad(m)] = v;
         }
+    }
+    float2 kk_reg[2] = {make_float2(0.f, 0.f), make_float2(0.f, 0.f)};  // SLIM: the kernel's spectrum at tid, tid + 512
+    if (SLIM) {
+        __syncthreads();
+        fft_forward(&s[0][0], 1, tw, tid, 512);
+        kk_reg[0] = s[0][pad(tid)];
+        kk_reg[1] = s[0][pad(tid + 512)];
+        __syncthreads();
     }
     for (int pair0 = 0; pair0 < 2; pair0 += kPairsInFlight) {
         for (int e = tid; e < kData * kFft; e += 512) {
@@ -831,11 +846,13 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
             s[t][pad(m)] = v;
         }
         __syncthreads();
-        // (the kernel columns are transformed with the first round)
-        fft_forward(&s[0][0], pair0 == 0 ? kData + 1 : kData, tw, tid, 512);
-        for (int e = tid; e < kData * kFft; e += 512) {
-            const int t = e >> kLog2Fft, m = e & (kFft - 1);
-            const float2 kk = s[kData][pad(m)];
+        // (SLIM = false: the kernel columns are transformed with the first round)
+        fft_forward(&s[0][0], !SLIM && pair0 == 0 ? kData + 1 : kData, tw, tid, 512);
+#pragma unroll
+        for (int r = 0; r < kData * kFft / 512; ++r) {
+            const int e = tid + r * 512;
+            const int t = e >> kLog2Fft, m = e & (kFft - 1);  // (m = tid + 512 (r & 1))
+            const float2 kk = SLIM ? kk_reg[r & 1] : s[kKernelSlot][pad(m)];
             const float kv = (t & 1) ? kk.y : kk.x;
             float2 v = s[t][pad(m)];
             v.x *= kv;
@@ -1025,7 +1042,12 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
                                                                             p->twiddles, p->row_spectra, p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
-    conv_columns_kernel<<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
+    static const int slim_mode = getenv("TSNE_SLIM_COLUMNS") ? atoi(getenv("TSNE_SLIM_COLUMNS")) : -1;
+    const bool slim = slim_mode < 0 ? (p->blocked_ready && p->strip_rows >= 1024) : slim_mode == 1;
+    if (slim)
+        conv_columns_kernel<true><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
+    else
+        conv_columns_kernel<false><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvRowsInverse, s)) return 1;
     conv_rows_inverse_kernel<<<xcd_launch_blocks(div_up(G, 2)), kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
