@@ -700,15 +700,17 @@ __device__ __forceinline__ float kernel_value(float lo, float h, int a, int b) {
     return (float)(1.0 / (s * s));
 }
 
-template <int THREADS>
+// Kernel values of 4 * PAIRS rows of the grid (two rows packed into one complex transform) and their transforms.
+template <int THREADS, int PAIRS>
 __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *sc, int slot, int n_boxes,
                                                   const float2 *__restrict__ tw, float *__restrict__ kernel_rows,
                                                   float2 (*s)[kFftPad]) {
+    constexpr int kTransforms = 2 * PAIRS;
     const int tid = threadIdx.x;
     const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    const int a0 = block * 4;
-    for (int e = tid; e < 2 * kFft; e += THREADS) {
+    const int a0 = block * 2 * kTransforms;
+    for (int e = tid; e < kTransforms * kFft; e += THREADS) {
         const int f = e >> kLog2Fft, m = e & (kFft - 1);
         const int b = m < kFft / 2 ? m : kFft - m;
         const int ra = a0 + 2 * f;
@@ -720,12 +722,12 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
         s[f][pad(m)] = v;
     }
     __syncthreads();
-    fft_forward(&s[0][0], 2, tw, tid, THREADS);
-    for (int e = tid; e < 2 * kFft; e += THREADS) {
+    fft_forward(&s[0][0], kTransforms, tw, tid, THREADS);
+    for (int e = tid; e < kTransforms * kFft; e += THREADS) {
         const int f = e >> kLog2Fft, pos = e & (kFft - 1);
         const int v = rev4(pos);
-        if (v <= kFft / 2) {
-            const int ra = a0 + 2 * f;
+        const int ra = a0 + 2 * f;
+        if (v <= kFft / 2 && ra < kNodePad) {
             const float2 val = s[f][pad(pos)];
             *reinterpret_cast<float2 *>(kernel_rows + (size_t)v * kNodePad + ra) = val;
         }
@@ -757,7 +759,7 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
     const int row_blocks = (G + ROWS - 1) / ROWS;
     const int launched = kXcds * ((row_blocks + kXcds - 1) / kXcds);
     if ((int)blockIdx.x >= launched) {
-        kernel_rows_block<kThreads>(blockIdx.x - launched, sc, slot, n_boxes, tw, kernel_rows, s);
+        kernel_rows_block<kThreads, ROWS>(blockIdx.x - launched, sc, slot, n_boxes, tw, kernel_rows, s);
         return;
     }
     const int row_block = xcd_row_block(blockIdx.x, row_blocks);
@@ -1038,7 +1040,7 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
         TSNE_TRY(hipMemcpyAsync(charges_out, p->node_charges, sizeof(float4) * (size_t)G * G,
                                 hipMemcpyDeviceToDevice, s));
     if (profile_mark(p, kKernelConvRowsForward, s)) return 1;
-    conv_rows_forward_kernel<2><<<xcd_launch_blocks(div_up(G, 2)) + div_up(G, 4), 512, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
+    conv_rows_forward_kernel<2><<<xcd_launch_blocks(div_up(G, 2)) + div_up(G, 8), 512, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
                                                                             p->twiddles, p->row_spectra, p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
