@@ -65,12 +65,21 @@ constexpr int kMQ = 128;  // MFMA sweep: queries per workgroup (4 waves x 32)
 constexpr int kMfmaMaxSteps = 64;  // k-steps of 2 dimensions: up to 126 dimensions + 2 augmented
 static_assert(kMQ == kCT, "query tiles and candidate tiles share the packed layout");
 
-// v_min3_f32 without the quieting moves the library fminf adds for signalling NaNs.
+// v_min3_f32 / v_min_f32 without the quieting moves the library fminf adds for signalling NaNs.
+// The compiler's wait states between a matrix instruction and a vector instruction that reads its result do
+// not cover instructions inside inline assembly: a chain of these over an accumulator has to start from
+// matrix_result(), an ordinary instruction on one of the accumulator's registers, and depend on its value.
 __device__ __forceinline__ float min3(float a, float b, float c) {
     float r;
     asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
     return r;
 }
+__device__ __forceinline__ float min2(float a, float b) {
+    float r;
+    asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float matrix_result(float x) { return __builtin_canonicalizef(x); }
 
 __device__ __forceinline__ u64 pack_key(float d, int j) {
     return ((u64)float_to_ordered(d) << 32) | (unsigned int)j;
@@ -789,10 +798,11 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                 for (int g = 0; g < 4; ++g) {
                     const v16f &a = g < 2 ? acc0 : acc1;
                     const int o = 8 * (g & 1);
-                    float m = min3(a[o], a[o + 1], a[o + 2]);
-                    m = min3(m, a[o + 3], a[o + 4]);
-                    m = min3(m, a[o + 5], a[o + 6]);
-                    run_min[g] = fminf(m, a[o + 7]);
+                    float m = matrix_result(a[o + 7]);
+                    m = min3(m, a[o], a[o + 1]);
+                    m = min3(m, a[o + 2], a[o + 3]);
+                    m = min3(m, a[o + 4], a[o + 5]);
+                    run_min[g] = min2(m, a[o + 6]);
                 }
                 const float best = fminf(min3(run_min[0], run_min[1], run_min[2]), run_min[3]);
                 // A query meets about K' ln(N / K') passing candidates during the sweep and the 64 lanes
@@ -1085,13 +1095,13 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
             for (int cb = 0; cb < 4; cb += 2) {
                 v16f &acc0 = acc[cb], &acc1 = acc[cb + 1];
                 // Register v of lane l holds candidate row 8*(v/4) + 4*(l/32) + v%4 of the block, query column l%32.
-                float best = min3(acc0[0], acc0[1], acc0[2]);
+                float best = matrix_result(acc0[0]);
 #pragma unroll
-                for (int v = 3; v + 1 < 16; v += 2) best = min3(best, acc0[v], acc0[v + 1]);
-                best = min3(best, acc0[15], acc1[0]);
+                for (int v = 1; v + 1 < 16; v += 2) best = min3(best, acc0[v], acc0[v + 1]);
+                best = min3(best, acc0[15], matrix_result(acc1[0]));
 #pragma unroll
                 for (int v = 1; v + 1 < 16; v += 2) best = min3(best, acc1[v], acc1[v + 1]);
-                best = fminf(best, acc1[15]);
+                best = min2(best, acc1[15]);
                 if (best <= limit_d) {
                     const int jbase = c0 + cb * 32 + 4 * kh;  // element (half, v) is candidate jbase + 32 half + 8 (v / 4) + v % 4
                     // Candidates beyond N (last tile) and the query itself (its own tile) are raised to +inf.
