@@ -744,6 +744,10 @@ def test_knn_matrix_sweep_is_exact(stages, n, d, k):
     idx_v, d2_v, stats_v = stages.knn_select(dev(X), k, 1)
     assert stats_v[0] == 0
     assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
+    # up to 125 dimensions sweep 2 multiplies bf16 terms; sweep 3 keeps the products on floats
+    idx_f, d2_f, stats_f = stages.knn_select(dev(X), k, 3)
+    assert stats_f[0] == 1
+    assert torch.equal(idx_f, idx) and torch.equal(d2_f, d2)
 
 
 @pytest.mark.parametrize("scale,d", [(30.0, 12), (2.5, 6), (0.7, 4), (6.0, 160), (0.3, 140)])
@@ -759,9 +763,10 @@ def test_knn_tile_skipping_is_exact(stages, scale, d):
     dX = dev(X)
     Xs = stages.gather_rows(dX, stages.locality_order(dX))
     idx_v, d2_v, _ = stages.knn_select(Xs, k, 1)
-    idx, d2, stats = stages.knn_select(Xs, k, 2)
-    assert stats[0] == 1
-    assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
+    for sweep in (2, 3):
+        idx, d2, stats = stages.knn_select(Xs, k, sweep)
+        assert stats[0] == 1
+        assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
     Xs_h = Xs.cpu().numpy()
     for first in (0, n // 3, n - 96):
         idx_o, d2_o = oracle.knn(Xs_h, k, rows=(first, first + 96))
@@ -848,25 +853,29 @@ def test_knn_chunked_sweep_gives_up_on_unverifiable_data(stages):
         assert np.array_equal(d2_a[first:first + 48].cpu().numpy(), d2_o)
 
 
-def test_knn_matrix_sweep_verification_falls_back(stages):
-    """Points far from the origin with tiny mutual distances: the approximate
-    |c|^2 - 2 q.c distances cannot separate them, the verification must notice
-    and the vector sweep must repair every such query; duplicates tie on index."""
+@pytest.mark.parametrize("sweep", [2, 3])
+def test_knn_matrix_sweep_verification_falls_back(stages, sweep):
+    """Points far from the origin with tiny mutual distances: neither the
+    |c|^2 - 2 q.c distances on floats (sweep 3) nor the bf16 terms relative to the
+    tile centres (sweep 2) can separate them, the verification must notice and the
+    vector sweep must repair every such query; duplicates tie on index."""
     rng = np.random.default_rng(3)
     base = rng.standard_normal((1, 16)).astype(np.float32) * 300.0
     X = (base + rng.standard_normal((2000, 16)).astype(np.float32) * 1e-2).astype(np.float32)
     X[1000:1100] = X[0:100]  # exact duplicates
     idx_o, d2_o = oracle.knn(X, 25)
-    idx, d2, stats = stages.knn_select(dev(X), 25, 2)
+    idx, d2, stats = stages.knn_select(dev(X), 25, sweep)
     assert stats[0] == 1 and stats[1] > 0
     assert np.array_equal(idx.cpu().numpy(), idx_o)
     assert np.array_equal(d2.cpu().numpy(), d2_o)
 
 
-def test_knn_few_failed_queries_are_redone_by_candidate_range(stages):
+@pytest.mark.parametrize("sweep", [2, 3])
+def test_knn_few_failed_queries_are_redone_by_candidate_range(stages, sweep):
     """A clump of 400 nearly identical points: for some of its members the 300th
     neighbour and the sweep's threshold lie closer together than the matrix sweep
-    can tell apart, so they fail its verification (95 of them on this seed) while
+    can tell apart, so they fail its verification (95 of them on this seed with the
+    products on floats) while
     the other points pass.  The vector sweep takes just those queries, cut over the chip by candidate range and merged
     (K - 1 = 299 keys per range)."""
     rng = np.random.default_rng(11)
@@ -874,7 +883,7 @@ def test_knn_few_failed_queries_are_redone_by_candidate_range(stages):
     X = rng.standard_normal((n, d)).astype(np.float32)
     clump = rng.choice(n, 400, replace=False)
     X[clump] = (rng.standard_normal((1, d)) + rng.standard_normal((400, d)) * 1e-5).astype(np.float32)
-    idx, d2, stats = stages.knn_select(dev(X), k, 2)
+    idx, d2, stats = stages.knn_select(dev(X), k, sweep)
     assert stats[0] == 1 and 0 < stats[1] <= 400
     rows = np.concatenate([clump[:80], rng.choice(n, 24, replace=False)])
     for q in rows:

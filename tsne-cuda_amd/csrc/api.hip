@@ -276,7 +276,8 @@ int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neig
 int tsne_hip_knn_select(const float *points, int num_points, int num_dims, int num_neighbors, int *indices,
                         float *sq_dist, void *stream, int sweep, int *stats) {
     TSNE_REQUIRE(points && indices && sq_dist, "knn: null pointer argument");
-    TSNE_REQUIRE(sweep >= 0 && sweep <= 2, "knn: sweep must be 0 (choose), 1 (vector) or 2 (matrix), got %d", sweep);
+    TSNE_REQUIRE(sweep >= 0 && sweep <= 3, "knn: sweep must be 0 (choose), 1 (vector), 2 (matrix) or 3 (matrix on floats), got %d",
+                 sweep);
     return run_knn_mode(points, num_points, num_dims, num_neighbors, indices, sq_dist, (hipStream_t)stream, sweep,
                         stats);
 }

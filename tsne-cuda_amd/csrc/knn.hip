@@ -57,6 +57,7 @@ namespace {
 typedef unsigned long long u64;
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 constexpr int kQT = 64;   // VALU sweep: queries per workgroup
 constexpr int kCT = 128;  // candidates per tile (both sweeps)
@@ -147,6 +148,104 @@ __global__ __launch_bounds__(256) void pack_points_kernel(const float *__restric
         }
     }
     Xp[t] = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// Nearest bf16 of a finite float (ties to even), as its 16 bits, and the float such bits stand for.
+__device__ __forceinline__ unsigned int bf16_bits(float v) {
+    const unsigned int u = __float_as_uint(v);
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float bf16_value(unsigned int bits) { return __uint_as_float(bits << 16); }
+
+// Points for the bf16 sweep: relative to the centre m of their own tile's bounding ball (small numbers, so
+// that what the bf16 terms leave out is small), every coordinate split into two bf16 terms (high = nearest
+// bf16, low = nearest bf16 of the rest), in the A-operand layout of v_mfma_f32_32x32x16_bf16.  Per tile
+//   [block of 32 points (4)][term (2: high, low)][step of 16 dimensions (S16)][lane (64)] 8 x bf16
+// (lane = 32 * (dimension % 16 / 8) + point % 32, element = dimension % 8), then 64 float4 written by
+// pack_tile_centres_kernel.  Dimensions D, D + 1 and D + 2 of the high term carry
+// beta = |x - m|^2 + 2 m.(x - m) as three bf16 terms (24 bits: the float exactly), so that against the
+// query-side operand (-2 q_d, and 1 in those three dimensions) the product is |q - x|^2 - |q - m|^2.
+__global__ __launch_bounds__(256) void pack_points_bf16_kernel(const float *__restrict__ X,
+                                                               const float *__restrict__ centers_t, int N, int D,
+                                                               int S16, int T, int Npad, uint4 *__restrict__ Xb) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // one lane's 8 values per thread
+    const int64_t total = (int64_t)Npad * S16 * 4;
+    if (t >= total) return;
+    const int lane = (int)(t & 63);
+    int64_t rest = t >> 6;
+    const int s16 = (int)(rest % S16);
+    rest /= S16;
+    const int term = (int)(rest & 1);
+    const int64_t blk = rest >> 1;  // tile * 4 + block
+    const int tile = (int)(blk >> 2);
+    const int i = (int)(blk * 32 + (lane & 31));
+    const int d0 = 16 * s16 + 8 * (lane >> 5);
+    unsigned int h[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+    if (i < N) {
+        float beta = 0.0f;
+        if (term == 0 && d0 + 8 > D && d0 < D + 3) {
+            float sq = 0.0f, dot = 0.0f;
+            for (int d = 0; d < D; ++d) {
+                const float m = centers_t[(size_t)d * T + tile];
+                const float delta = X[(size_t)i * D + d] - m;
+                sq = fmaf(delta, delta, sq);
+                dot = fmaf(m, delta, dot);
+            }
+            beta = fmaf(2.0f, dot, sq);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int d = d0 + j;
+            if (d < D) {
+                const float v = X[(size_t)i * D + d] - centers_t[(size_t)d * T + tile];
+                const unsigned int hi = bf16_bits(v);
+                h[j] = term == 0 ? hi : bf16_bits(v - bf16_value(hi));
+            } else if (d < D + 3 && term == 0) {
+                float r = beta;
+                unsigned int part = bf16_bits(r);
+                for (int k = D; k < d; ++k) {
+                    r -= bf16_value(part);
+                    part = bf16_bits(r);
+                }
+                h[j] = part;
+            }
+        }
+    }
+    const int64_t in_tile = t - (int64_t)tile * (S16 * 512);
+    Xb[(int64_t)tile * (S16 * 512 + 64) + in_tile] =
+        make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+}
+
+// The 64 float4 that close a tile of the bf16 sweep's points: floats 0 .. 16 S16 - 1 the centre m (zero beyond
+// D), floats 128 and 129 the tile's error coefficients ga, gb.  A candidate distance the sweep computes for
+// a query q against this tile is off by at most |q| ga + gb:
+//  - the two bf16 terms leave out, per dimension, low x low and what they do not represent: with u = 2^-8
+//    less than 3.1 * 2^-16 |q_d delta_d|, twice that after the factor -2, and sum |q_d delta_d| <= |q| r
+//    (r: the ball's radius);
+//  - the 3 D + 3 products are accumulated in fp32 in the matrix unit's order: 4 (3 D + 6) 2^-24 (the factor
+//    four covers that order) times the sum of the terms' magnitudes, at most 2 |q| r + r^2 + 2 |m| r;
+//  - the rounding of x - m, of beta and of the final additions is below a hundredth of the above.
+__global__ __launch_bounds__(64) void pack_tile_centres_kernel(const float *__restrict__ centers_t,
+                                                               const float *__restrict__ radius, int D, int S16,
+                                                               int T, float4 *__restrict__ Xb) {
+    const int tile = blockIdx.x, l = threadIdx.x;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (l < 32) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (4 * l + c < D) v[c] = centers_t[(size_t)(4 * l + c) * T + tile];
+    } else if (l == 32) {
+        float m2 = 0.0f;
+        for (int d = 0; d < D; ++d) {
+            const float m = centers_t[(size_t)d * T + tile];
+            m2 = fmaf(m, m, m2);
+        }
+        const float r = radius[tile], mlen = sqrtf(m2) * (1.0f + 1e-6f);
+        const float split = 6.2f / 65536.0f, acc = 4.0f * (float)(3 * D + 6) * 5.9604644775390625e-08f;
+        v[0] = 1.01f * (split + 2.0f * acc) * r;
+        v[1] = 1.01f * acc * (r * r + 2.0f * mlen * r) + 1e-30f;
+    }
+    Xb[(size_t)tile * (S16 * 512 + 64) + S16 * 512 + l] = make_float4(v[0], v[1], v[2], v[3]);
 }
 
 // Sorts sortbuf[0..cap) ascending (cap a power of two), all 256 threads.
@@ -365,21 +464,10 @@ constexpr int kHomeTiles = 8;  // candidate tiles on either side of the query ti
 // (qcenter, ra): with c, r the balls, every pair of members is at least |c_a - c_t| - r_a - r_t apart
 // (triangle inequality); 1e-3 relative slack on the centre distance, the radii are upper bounds.
 // Anything that is not a number keeps the tile.
+// Eight loads in flight and two partial sums: one load at a time would cost its latency per dimension
+// (any summation order will do, the slack covers the rounding).
 __device__ __forceinline__ bool tile_may_matter(const float *qcenter, float ra, const float *__restrict__ centers_t,
                                                 const float *__restrict__ radius, int D, int T, int t, float tmax) {
-    float d2 = 0.0f;
-    for (int d = 0; d < D; ++d) {
-        const float diff = qcenter[d] - centers_t[(size_t)d * T + t];
-        d2 = fmaf(diff, diff, d2);
-    }
-    const float lb = sqrtf(d2) * (1.0f - 1e-3f) - (ra + radius[t]);
-    return !(lb > 0.0f && lb * lb > tmax);
-}
-
-// The same test for hundreds of dimensions: eight loads in flight and two partial sums (any summation
-// order will do, the slack covers the rounding).
-__device__ __forceinline__ bool tile_may_matter_wide(const float *qcenter, float ra, const float *__restrict__ centers_t,
-                                                     const float *__restrict__ radius, int D, int T, int t, float tmax) {
     float s0 = 0.0f, s1 = 0.0f;
     int d = 0;
     for (; d + 8 <= D; d += 8) {
@@ -601,6 +689,7 @@ __global__ __launch_bounds__(256) void knn_merge_slices_kernel(const u64 *__rest
 
 struct SweepArgs {
     const float4 *Xp;
+    const float *X;  // the points as given (bf16 sweep: the query side is formed from them)
     int N, D, Dnorm, want, cap;
     u64 *lists;
     int num_qtiles;
@@ -634,9 +723,15 @@ struct SweepArgs {
 };
 
 // ---------------------------------------------------------------------------
-// MFMA sweep.  KSTEPS = Daug / 2 k-steps of v_mfma_f32_32x32x2f32.
-// Dynamic LDS: two candidate tiles, copied verbatim from the packed points
-//   a[buf][cand block (4)][step group (S4)][lane (64)] float4   (4 steps per float4)
+// MFMA sweep, in two arithmetic variants.
+// BF16 = false: KSTEPS = Daug / 2 k-steps of v_mfma_f32_32x32x2f32 on the points as floats.
+// BF16 = true: KSTEPS steps of 16 dimensions of v_mfma_f32_32x32x16_bf16 on the points split into two bf16
+// terms per coordinate; high x high, high x low and low x high are accumulated (three instructions per
+// step), which leaves out terms below 3 * 2^-16 of |q_d c_d| per dimension - the re-rank's verification
+// bound accounts for them.  A step of 16 dimensions takes half the matrix-pipe time of one fp32 step of 2.
+// Dynamic LDS: one candidate tile, copied verbatim from the packed points
+//   a[cand block (4)][step group (S4)][lane (64)] float4   (4 steps per float4)            fp32
+//   a[cand block (4)][term (2)][step (KSTEPS)][lane (64)] 8 x bf16                          bf16
 // followed by one sort buffer (cap keys) per wave and the visit bitmap (one bit per tile).
 //
 // Tiles are visited in two phases.  First the query tile's own neighbourhood in the point
@@ -652,17 +747,26 @@ struct SweepArgs {
 // (cand, -1 padded) and tau = the approximate distance of the last one kept
 // (+inf when fewer than `want` candidates exist), both without the |q|^2 term.
 // ---------------------------------------------------------------------------
-template <int KSTEPS>
-__global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_kernel(const SweepArgs args) {
+// Workgroups per compute unit the register budget is set for (bf16: the query's coordinates stay in
+// registers beside the two operand terms; three workgroups would spill at 3 steps and beyond).
+constexpr int bf16_sweep_occupancy(int steps) { return steps <= 2 ? 3 : (steps <= 4 ? 2 : 1); }
+template <int KSTEPS, bool BF16>
+constexpr int sweep_occupancy() {
+    return BF16 ? bf16_sweep_occupancy(KSTEPS) : (KSTEPS <= 28 ? 3 : 1);
+}
+
+template <int KSTEPS, bool BF16>
+__global__ __launch_bounds__(256, (sweep_occupancy<KSTEPS, BF16>())) void knn_mfma_sweep_kernel(const SweepArgs args) {
     const float4 *__restrict__ Xp = args.Xp;
     const int N = args.N, D = args.D, Dnorm = args.Dnorm, want = args.want, cap = args.cap;
     const int num_qtiles = args.num_qtiles;
     u64 *__restrict__ lists = args.lists;
     int *__restrict__ cand = args.cand;
     float *__restrict__ tau = args.tau;
-    constexpr int S4 = (KSTEPS + 3) / 4;
-    constexpr int kTileFloat4 = 4 * S4 * 64;              // float4 per candidate tile
-    constexpr int kLoadsPerThread = kTileFloat4 / 256;    // == S4
+    constexpr int S4 = BF16 ? 2 * KSTEPS : (KSTEPS + 3) / 4;  // 16-byte slots per lane and candidate block
+    constexpr int kMainFloat4 = 4 * S4 * 64;              // float4 of matrix operands per candidate tile
+    constexpr int kTileFloat4 = kMainFloat4 + (BF16 ? 64 : 0);  // ... and the centre block of the bf16 layout
+    constexpr int kLoadsPerThread = kMainFloat4 / 256;    // == S4
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     float4 *a_lds = reinterpret_cast<float4 *>(lds_raw);
     u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + kTileFloat4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
@@ -682,16 +786,18 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
     // One candidate tile: global -> registers (in flight during the matrix instructions) -> LDS.
     // The staging array is a native vector type with compile-time indices: as an array of
     // HIP float4 structs it was placed in scratch memory, where every load waited for the last.
-    v4f stage[kLoadsPerThread];
+    v4f stage[kLoadsPerThread], stage_centre;
     auto fetch = [&](int tile) {
         const v4f *src = reinterpret_cast<const v4f *>(Xp) + (size_t)tile * kTileFloat4 + tid;
 #pragma unroll
         for (int r = 0; r < kLoadsPerThread; ++r) stage[r] = src[r * 256];
+        if (BF16 && tid < 64) stage_centre = src[kMainFloat4];
     };
     auto stash = [&](int buf) {
         v4f *dst = reinterpret_cast<v4f *>(a_lds) + buf * kTileFloat4 + tid;
 #pragma unroll
         for (int r = 0; r < kLoadsPerThread; ++r) dst[r * 256] = stage[r];
+        if (BF16 && tid < 64) dst[kMainFloat4] = stage_centre;
     };
     const int num_ctiles = (N + kCT - 1) / kCT;
 
@@ -740,8 +846,37 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
         };
         // B operand from the same packed layout (query tiles and candidate tiles coincide: kMQ == kCT):
         // -2 q_d for the real dimensions, 1 for the |c|^2 row, 0 elsewhere.
-        float bq[4 * S4];
-        {
+        float bq[BF16 ? 1 : 4 * S4];
+        v8bf bq_hi[BF16 ? KSTEPS : 1], bq_lo[BF16 ? KSTEPS : 1];
+        float qf[BF16 ? 8 * KSTEPS : 1];  // this lane's half of the query's coordinates
+        float q_len = 0.0f;               // |q|, rounded up
+        if constexpr (BF16) {
+            // -2 q_d in two bf16 terms; 1 in the three dimensions of the high term that carry beta.
+            const float *xq = args.X + (size_t)(q < N ? q : 0) * D;
+            if (q < N) q_len = sqrtf(args.norms[q]) * (1.0f + 1e-6f);
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s) {
+                unsigned int oh[4], ol[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    unsigned int h2[2], l2[2];
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const int d = 16 * s + 8 * kh + 2 * k + e;
+                        const float v = q < N && d < D ? xq[d] : 0.0f;
+                        qf[8 * s + 2 * k + e] = v;
+                        const float w = -2.0f * v;
+                        const unsigned int hi = bf16_bits(w);
+                        h2[e] = d < D ? hi : (d < D + 3 ? 0x3f80u : 0u);
+                        l2[e] = d < D ? bf16_bits(w - bf16_value(hi)) : 0u;
+                    }
+                    oh[k] = h2[0] | (h2[1] << 16);
+                    ol[k] = l2[0] | (l2[1] << 16);
+                }
+                bq_hi[s] = __builtin_bit_cast(v8bf, make_uint4(oh[0], oh[1], oh[2], oh[3]));
+                bq_lo[s] = __builtin_bit_cast(v8bf, make_uint4(ol[0], ol[1], ol[2], ol[3]));
+            }
+        } else {
             const float4 *src = Xp + (size_t)qt * kTileFloat4 + (size_t)wave * S4 * 64 + lane;
 #pragma unroll
             for (int s4 = 0; s4 < S4; ++s4) {
@@ -762,28 +897,68 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
             const u64 limit = thr[wave * 32 + qn];
             // ~0 is "no threshold yet": its distance field does not decode to a number.
             const float limit_d = limit == ~0ull ? INFINITY : key_distance(limit);
+            // bf16: the matrix product lacks |q - m|^2 (m: the tile's centre), and the keys carry a lower bound
+            // of the distance: the product plus `off` = |q - m|^2 (rounded down) - the tile's error bound.
+            // The products are tested against the threshold less `off`, rounded up.
+            float off = 0.0f, limit_acc = limit_d;
+            if constexpr (BF16) {
+                const float4 *cen = a_lds + buf * kTileFloat4 + kMainFloat4;
+                float f = 0.0f;
+#pragma unroll
+                for (int s = 0; s < KSTEPS; ++s) {
+                    const float4 m0 = cen[4 * s + 2 * kh], m1 = cen[4 * s + 2 * kh + 1];
+                    const float m[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float diff = qf[8 * s + j] - m[j];
+                        f = fmaf(diff, diff, f);
+                    }
+                }
+                f += __shfl_xor(f, 32);
+                const float4 g = cen[32];
+                off = f * (1.0f - (float)(D + 4) * 5.9604644775390625e-08f) - fmaf(q_len, g.x, g.y);
+                limit_acc = limit_d - off;
+                limit_acc += 2.4e-7f * (fabsf(limit_d) + fabsf(off));  // (inf stays inf)
+            }
             // Two candidate blocks at a time: two independent accumulator chains keep the matrix pipe busy.
             auto multiply = [&](int cb, v16f &acc0, v16f &acc1) {
                 acc0 = v16f{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 acc1 = acc0;
                 const float4 *a0 = a_lds + (size_t)(buf * 4 + cb) * S4 * 64 + lane;
                 const float4 *a1 = a0 + S4 * 64;
+                if constexpr (BF16) {
+                    const v4f *b0 = reinterpret_cast<const v4f *>(a0), *b1 = reinterpret_cast<const v4f *>(a1);
 #pragma unroll
-                for (int s4 = 0; s4 < S4; ++s4) {
-                    const float4 x = a0[s4 * 64], y = a1[s4 * 64];
-                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, bq[4 * s4], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.x, bq[4 * s4], acc1, 0, 0, 0);
-                    if (4 * s4 + 1 < KSTEPS) {
-                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, bq[4 * s4 + 1], acc0, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.y, bq[4 * s4 + 1], acc1, 0, 0, 0);
+                    for (int s = 0; s < KSTEPS; ++s) {
+                        const v8bf xh = __builtin_bit_cast(v8bf, b0[s * 64]);
+                        const v8bf yh = __builtin_bit_cast(v8bf, b1[s * 64]);
+                        const v8bf xl = __builtin_bit_cast(v8bf, b0[(KSTEPS + s) * 64]);
+                        const v8bf yl = __builtin_bit_cast(v8bf, b1[(KSTEPS + s) * 64]);
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xh, bq_hi[s], acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(yh, bq_hi[s], acc1, 0, 0, 0);
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xh, bq_lo[s], acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(yh, bq_lo[s], acc1, 0, 0, 0);
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xl, bq_hi[s], acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(yl, bq_hi[s], acc1, 0, 0, 0);
                     }
-                    if (4 * s4 + 2 < KSTEPS) {
-                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, bq[4 * s4 + 2], acc0, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.z, bq[4 * s4 + 2], acc1, 0, 0, 0);
-                    }
-                    if (4 * s4 + 3 < KSTEPS) {
-                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, bq[4 * s4 + 3], acc0, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.w, bq[4 * s4 + 3], acc1, 0, 0, 0);
+                } else {
+#pragma unroll
+                    for (int s4 = 0; s4 < S4; ++s4) {
+                        const float4 x = a0[s4 * 64], y = a1[s4 * 64];
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, bq[4 * s4], acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.x, bq[4 * s4], acc1, 0, 0, 0);
+                        if (4 * s4 + 1 < KSTEPS) {
+                            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, bq[4 * s4 + 1], acc0, 0, 0, 0);
+                            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.y, bq[4 * s4 + 1], acc1, 0, 0, 0);
+                        }
+                        if (4 * s4 + 2 < KSTEPS) {
+                            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, bq[4 * s4 + 2], acc0, 0, 0, 0);
+                            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.z, bq[4 * s4 + 2], acc1, 0, 0, 0);
+                        }
+                        if (4 * s4 + 3 < KSTEPS) {
+                            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, bq[4 * s4 + 3], acc0, 0, 0, 0);
+                            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(y.w, bq[4 * s4 + 3], acc1, 0, 0, 0);
+                        }
                     }
                 }
             };
@@ -810,7 +985,7 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                 // stores its keys one after the other at the end of its own region of the query's list.
                 // The test is on the distance alone; an element that ties with the threshold's distance
                 // but not its index is appended too and sorted out by the next compaction.
-                if (best <= limit_d) {
+                if (best <= limit_acc) {
                     const int jbase = c0 + cb * 32 + 4 * kh;  // element (half, v) is candidate jbase + 32 half + 8 (v / 4) + v % 4
                     // Only the last tile has candidates beyond N and only the query's own tile holds the
                     // query: those two tiles knock the excluded elements out by raising them to +inf.
@@ -822,7 +997,7 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                             if (j + 32 >= N || j + 32 == q) acc1[e] = INFINITY;
                         }
                     }
-                    const float lim = q < N ? limit_d : -INFINITY;
+                    const float lim = q < N ? limit_acc : -INFINITY;
                     u64 *const dst0 = list + ((wave * 32 + qn) * cap + kh * half + my_n);
                     u64 *dst = dst0;
 #pragma unroll
@@ -836,7 +1011,7 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                             if (dist <= lim) {
                                 int jb = jbase;
                                 asm volatile("" : "+v"(jb));  // the index is formed here, not held in 32 registers
-                                *dst++ = pack_key(dist, jb + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
+                                *dst++ = pack_key(BF16 ? dist + off : dist, jb + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
                             }
                         }
                     }
@@ -918,7 +1093,7 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                     float v = -INFINITY;
                     if (q0 + tid < N) {
                         const u64 t = thr[tid];
-                        v = t == ~0ull ? INFINITY : key_distance(t) + args.norms[q0 + tid];
+                        v = t == ~0ull ? INFINITY : key_distance(t) + (BF16 ? 0.0f : args.norms[q0 + tid]);
                         v += 1e-5f * fabsf(v) + 1e-30f;
                     }
                     v = group_max<kWave>(v);
@@ -952,6 +1127,10 @@ __global__ __launch_bounds__(256, (KSTEPS <= 28 ? 3 : 1)) void knn_mfma_sweep_ke
                     stash(buf);  // the barrier that ended the last tile freed both buffers
                     __syncthreads();
                 }
+                // Nothing this block loaded is left in flight as far as the compiler can tell: a load it
+                // takes to be possibly outstanding here makes it wait for all loads, the next tile's
+                // included, at the first register reuse after process() has issued them.
+                __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
             }
             cur = nxt;
         }
@@ -1202,7 +1381,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                 const float ra = args.radius[qt];
                 for (int t = tid; t < T; t += 256)
                     if ((t < h0 || t > h1) && t % P == part &&
-                        tile_may_matter_wide(qcenter, ra, args.centers_t, args.radius, D, T, t, tmax))
+                        tile_may_matter(qcenter, ra, args.centers_t, args.radius, D, T, t, tmax))
                         atomicOr(&bitmap[t >> 5], 1u << (t & 31));
                 __syncthreads();
                 nxt = next_tile();
@@ -1211,6 +1390,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                     stash();  // the barrier that ended the last tile freed the LDS chunk
                     __syncthreads();
                 }
+                __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), as in the kernel above
             }
             cur = nxt;
         }
@@ -1277,7 +1457,7 @@ __global__ __launch_bounds__(256) void knn_rerank_kernel(const float *__restrict
                                                          int *__restrict__ out_idx, float *__restrict__ out_d,
                                                          int *__restrict__ fail_count, int *__restrict__ fail_list,
                                                          const int *__restrict__ qtile_list, int qtile_first,
-                                                         int qtile_step, int n_slots) {
+                                                         int qtile_step, int n_slots, int lower_bounds) {
     extern __shared__ u64 keys_all[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     // Query slot w belongs to query tile qtile_list[w / kMQ], or first + (w / kMQ) step without a list
@@ -1380,19 +1560,25 @@ __global__ __launch_bounds__(256) void knn_rerank_kernel(const float *__restrict
         }
     }
     if (!live) return;
-    // Every candidate outside the list has an approximate distance >= tau (without |q|^2), so its
-    // canonical distance is >= tau + |q|^2 - g.  g bounds |approximate - canonical|: both are sums of
-    // at most D + 3 rounded terms of magnitude <= (|q| + |c|)^2, and the canonical distance carries
+    // Sweep on floats: every candidate outside the list has an approximate distance >= tau (without
+    // |q|^2), so its canonical distance is >= tau + |q|^2 - g.  g bounds |approximate - canonical|: both are
+    // sums of at most D + 3 rounded terms of magnitude <= (|q| + |c|)^2, and the canonical distance carries
     // a relative error of (D + 2) 2^-24 of itself; a factor of four covers the matrix unit's
     // accumulation order and the rounding of the stored norms.
+    // Sweep on bf16 terms (lower_bounds): the sweep's keys are lower bounds of the distances, so every
+    // candidate outside the list has a distance >= tau, and a canonical distance within (D + 2) 2^-24 of that.
     const float kth = key_distance(keys[K - 2]);
     const float t = tau[w];
     bool pass = isinf(t) && t > 0.0f;
     if (!pass) {
-        const double nq = norms[q], nmax = *max_norm;
         const double eps = 5.9604644775390625e-08;  // 2^-24
-        const double g = 4.0 * (D + 4) * eps * (nq + nmax + 2.0 * sqrt(nq * nmax)) + (D + 4) * eps * (double)kth;
-        pass = (double)kth < (double)t + nq - g;
+        if (lower_bounds) {
+            pass = (double)kth + (D + 4) * eps * ((double)kth + fabs((double)t)) < (double)t;
+        } else {
+            const double nq = norms[q], nmax = *max_norm;
+            const double g = 4.0 * (D + 4) * eps * (nq + nmax + 2.0 * sqrt(nq * nmax)) + (D + 4) * eps * (double)kth;
+            pass = (double)kth < (double)t + nq - g;
+        }
     }
     if (pass) {
         for (int e = lane; e < K; e += kWave) {
@@ -1431,23 +1617,42 @@ int next_pow2(int v) {
     return n;
 }
 
-template <int KSTEPS>
+template <int KSTEPS, bool BF16>
 int launch_mfma_sweep(const SweepArgs &args, int grid, hipStream_t s) {
-    constexpr int S4 = (KSTEPS + 3) / 4;
-    // two tiles + a sort buffer per wave + the visit bitmap
-    const size_t lds = sizeof(float4) * 4 * S4 * 64 + sizeof(u64) * 4 * args.cap + sizeof(unsigned int) * args.bitmap_words;
-    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_sweep_kernel<KSTEPS>),
+    constexpr int S4 = BF16 ? 2 * KSTEPS : (KSTEPS + 3) / 4;
+    // one tile (bf16: with its centre block) + a sort buffer per wave + the visit bitmap
+    const size_t lds = sizeof(float4) * (4 * S4 * 64 + (BF16 ? 64 : 0)) + sizeof(u64) * 4 * args.cap +
+                       sizeof(unsigned int) * args.bitmap_words;
+    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_sweep_kernel<KSTEPS, BF16>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    knn_mfma_sweep_kernel<KSTEPS><<<grid, 256, lds, s>>>(args);
+    knn_mfma_sweep_kernel<KSTEPS, BF16><<<grid, 256, lds, s>>>(args);
     TSNE_TRY(hipGetLastError());
     return 0;
 }
+
+// Steps of 16 dimensions of the bf16 sweep: up to 125 dimensions + the three |c|^2 terms.
+int dispatch_bf16_sweep(int steps, const SweepArgs &args, int grid, hipStream_t s) {
+    switch (steps) {
+        case 1: return launch_mfma_sweep<1, true>(args, grid, s);
+        case 2: return launch_mfma_sweep<2, true>(args, grid, s);
+        case 3: return launch_mfma_sweep<3, true>(args, grid, s);
+        case 4: return launch_mfma_sweep<4, true>(args, grid, s);
+        case 5: return launch_mfma_sweep<5, true>(args, grid, s);
+        case 6: return launch_mfma_sweep<6, true>(args, grid, s);
+        case 7: return launch_mfma_sweep<7, true>(args, grid, s);
+        case 8: return launch_mfma_sweep<8, true>(args, grid, s);
+        default:
+            set_error("knn: no bf16 matrix-instruction sweep for %d steps", steps);
+            return 1;
+    }
+}
+
 
 // Instantiated step counts: every count up to 32 (62 dimensions), then multiples of 4.
 int dispatch_mfma_sweep(int ksteps, const SweepArgs &args, int grid, hipStream_t s) {
 #define TSNE_MFMA_CASE(KS) \
     case KS:               \
-        return launch_mfma_sweep<KS>(args, grid, s);
+        return launch_mfma_sweep<KS, false>(args, grid, s);
     switch (ksteps) {
         TSNE_MFMA_CASE(2) TSNE_MFMA_CASE(3) TSNE_MFMA_CASE(4) TSNE_MFMA_CASE(5) TSNE_MFMA_CASE(6)
         TSNE_MFMA_CASE(7) TSNE_MFMA_CASE(8) TSNE_MFMA_CASE(9) TSNE_MFMA_CASE(10) TSNE_MFMA_CASE(11)
@@ -1518,7 +1723,8 @@ int run_valu_sweep(const float *points, const float *Xt, int N, int Npad, int D,
 
 }  // namespace
 
-// mode: 0 = choose, 1 = VALU sweep only, 2 = matrix-instruction sweep (error if the shape does not fit).
+// mode: 0 = choose, 1 = VALU sweep only, 2 = matrix-instruction sweep (error if the shape does not fit),
+// 3 = as 2 with the products on floats also where the bf16 split applies (up to 125 dimensions).
 // stats (optional, 3 ints): [0] = 1 if the matrix-instruction sweep ran, [1] = queries redone by the VALU sweep,
 // [2] = per mille of the (query tile, candidate tile) pairs the matrix sweep computed.
 int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s, int mode,
@@ -1553,12 +1759,18 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     const int n_chunks = chunked ? div_up(ksteps, kChunkSteps) : 0;
     if (chunked) ksteps = n_chunks * kChunkSteps;
     else if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
+    // Up to 125 dimensions the sweep multiplies bf16 terms (two per coordinate) of the points relative to
+    // their tile's centre.
+    const bool force_f32 = mode == 3;
+    if (mode == 3) mode = 2;
+    const bool bf16 = !chunked && !force_f32 && D + 3 <= 128;
+    const int steps16 = div_up(D + 3, 16);
     const int num_tiles = div_up(N, kCT);
     const int bitmap_words = div_up(num_tiles, 32);
     // Room for the candidates kept, as many again and one more tile where the LDS sort buffers of that
     // size fit: a list that is nearly full right after a selection would be selected again after every tile.
     const size_t tile_lds = chunked ? sizeof(float4) * kChunkFloat4 + sizeof(float) * D
-                                    : sizeof(float4) * 4 * ((ksteps + 3) / 4) * 64;
+                                    : sizeof(float4) * (bf16 ? 512 * steps16 + 64 : 4 * ((ksteps + 3) / 4) * 64);
     auto lds_with = [&](int cap) -> size_t {
         return tile_lds + sizeof(u64) * 4 * cap + sizeof(unsigned int) * bitmap_words;
     };
@@ -1600,10 +1812,11 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         return run_valu_sweep(points, Xt.as<float>(), N, Npad, D, K, nullptr, N, cus, indices, sq_dist, s);
     }
 
-    const int S4 = (ksteps + 3) / 4;
+    const int S4 = bf16 ? 2 * steps16 : (ksteps + 3) / 4;  // 16-byte slots per lane and block of the packed points
     DeviceMem Xp, Bp, norms, scal, fail_list, centers, radius;
     const int num_qtiles = div_up(N, kMQ);
-    if (!Xp.alloc(sizeof(float4) * (size_t)Npad * S4 * 2) || !norms.alloc(sizeof(float) * Npad) ||
+    const size_t tile_float4 = bf16 ? 512 * (size_t)steps16 + 64 : (size_t)kCT * S4 * 2;  // float4 per packed tile
+    if (!Xp.alloc(sizeof(float4) * tile_float4 * num_tiles) || !norms.alloc(sizeof(float) * Npad) ||
         (chunked && !Bp.alloc(sizeof(float4) * (size_t)Npad * S4 * 2)) ||
         !scal.alloc(4 * sizeof(int)) || !fail_list.alloc(sizeof(int) * N) ||
         !centers.alloc(sizeof(float) * (size_t)D * num_tiles) || !radius.alloc(sizeof(float) * num_tiles)) {
@@ -1613,9 +1826,11 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     TSNE_TRY(hipMemsetAsync(scal.p, 0, 4 * sizeof(int), s));  // [0] max |x|^2 (float bits), [1] fail count, [2..3] tiles swept (64-bit)
     norms_kernel<<<div_up(Npad, 256), 256, 0, s>>>(points, N, D, Npad, norms.as<float>(), scal.as<float>());
     TSNE_TRY(hipGetLastError());
-    pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm, S4,
-                                                                          Npad, Xp.as<float4>(), false);
-    TSNE_TRY(hipGetLastError());
+    if (!bf16) {
+        pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm,
+                                                                              S4, Npad, Xp.as<float4>(), false);
+        TSNE_TRY(hipGetLastError());
+    }
     if (chunked) {
         pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm,
                                                                               S4, Npad, Bp.as<float4>(), true);
@@ -1624,6 +1839,14 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     tile_balls_kernel<<<num_tiles, 128, sizeof(float) * D, s>>>(points, N, D, num_tiles, centers.as<float>(),
                                                                radius.as<float>());
     TSNE_TRY(hipGetLastError());
+    if (bf16) {
+        pack_points_bf16_kernel<<<div_up((int64_t)Npad * steps16 * 4, 256), 256, 0, s>>>(
+            points, centers.as<float>(), N, D, steps16, num_tiles, Npad, Xp.as<uint4>());
+        TSNE_TRY(hipGetLastError());
+        pack_tile_centres_kernel<<<num_tiles, 64, 0, s>>>(centers.as<float>(), radius.as<float>(), D, steps16,
+                                                         num_tiles, Xp.as<float4>());
+        TSNE_TRY(hipGetLastError());
+    }
 
     // Sweep + re-rank of `count` query tiles: those of tile_list (device), or first, first + step, ... without a
     // list.  Keeps `keep` candidates per query and part.  failed = queries of those tiles whose verification
@@ -1635,7 +1858,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         // of dimensions, and the tiles differ in how many candidate tiles they can skip: unless there are
         // several query tiles per workgroup slot to even that out, the chunked kernel splits every tile's
         // candidates over up to 8 workgroups.
-        const int slots = cus * (!chunked && ksteps <= 28 ? 3 : 2);
+        const int slots = cus * (bf16 ? bf16_sweep_occupancy(steps16) : (!chunked && ksteps <= 28 ? 3 : 2));
         int parts = 1;
         if (chunked)
             while (parts < 8 && count * parts < 3 * slots && parts * 2 * keep <= 2048 && parts * 2 <= num_tiles)
@@ -1652,6 +1875,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         TSNE_TRY(hipMemsetAsync(scal.as<int>() + 1, 0, 3 * sizeof(int), s));
         SweepArgs args;
         args.Xp = Xp.as<float4>();
+        args.X = points;
         args.N = N;
         args.D = D;
         args.Dnorm = Dnorm;
@@ -1685,7 +1909,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             knn_mfma_chunked_sweep_kernel<<<grid, 256, lds, s>>>(args);
             TSNE_TRY(hipGetLastError());
-        } else if (dispatch_mfma_sweep(ksteps, args, grid, s)) {
+        } else if (bf16 ? dispatch_bf16_sweep(steps16, args, grid, s) : dispatch_mfma_sweep(ksteps, args, grid, s)) {
             return 1;
         }
         if (parts > 1) {
@@ -1703,7 +1927,8 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)(sizeof(u64) * 4 * sort_n)));
         knn_rerank_kernel<<<div_up((int)n_slots, 4), 256, sizeof(u64) * 4 * sort_n, s>>>(
             points, norms.as<float>(), N, D, K, keep, sort_n, cand.as<int>(), tau.as<float>(), scal.as<float>(),
-            indices, sq_dist, scal.as<int>() + 1, fail_list.as<int>(), tile_list, first, step, (int)n_slots);
+            indices, sq_dist, scal.as<int>() + 1, fail_list.as<int>(), tile_list, first, step, (int)n_slots,
+            bf16 ? 1 : 0);
         TSNE_TRY(hipGetLastError());
         int host_scal[4] = {0, 0, 0, 0};
         TSNE_TRY(hipMemcpyAsync(host_scal, scal.p, sizeof(host_scal), hipMemcpyDeviceToHost, s));
