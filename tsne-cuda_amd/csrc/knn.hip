@@ -928,12 +928,20 @@ __global__ __launch_bounds__(256, (sweep_occupancy<KSTEPS, BF16>())) void knn_mf
                 const float4 *a1 = a0 + S4 * 64;
                 if constexpr (BF16) {
                     const v4f *b0 = reinterpret_cast<const v4f *>(a0), *b1 = reinterpret_cast<const v4f *>(a1);
+                    // The operands of step s + 1 are read from LDS while the products of step s run.
+                    v4f next[4] = {b0[0], b1[0], b0[KSTEPS * 64], b1[KSTEPS * 64]};
 #pragma unroll
                     for (int s = 0; s < KSTEPS; ++s) {
-                        const v8bf xh = __builtin_bit_cast(v8bf, b0[s * 64]);
-                        const v8bf yh = __builtin_bit_cast(v8bf, b1[s * 64]);
-                        const v8bf xl = __builtin_bit_cast(v8bf, b0[(KSTEPS + s) * 64]);
-                        const v8bf yl = __builtin_bit_cast(v8bf, b1[(KSTEPS + s) * 64]);
+                        const v8bf xh = __builtin_bit_cast(v8bf, next[0]);
+                        const v8bf yh = __builtin_bit_cast(v8bf, next[1]);
+                        const v8bf xl = __builtin_bit_cast(v8bf, next[2]);
+                        const v8bf yl = __builtin_bit_cast(v8bf, next[3]);
+                        if (s + 1 < KSTEPS) {
+                            next[0] = b0[(s + 1) * 64];
+                            next[1] = b1[(s + 1) * 64];
+                            next[2] = b0[(KSTEPS + s + 1) * 64];
+                            next[3] = b1[(KSTEPS + s + 1) * 64];
+                        }
                         acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xh, bq_hi[s], acc0, 0, 0, 0);
                         acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(yh, bq_hi[s], acc1, 0, 0, 0);
                         acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xh, bq_lo[s], acc0, 0, 0, 0);
