@@ -186,14 +186,20 @@ def main():
                "frac": b / (kernels_us[name] * 1e-6) / 1e9 / HBM_PEAK_GBS}
         for name, b in loop_bytes.items() if kernels_us.get(name)}
     if knn_stats[0] == 1:
-        # Flop the matrix sweep executed: 2 x 128 x 128 x (padded dimensions) per tile pair it did not skip.
-        ksteps = (((d + 1) & ~1) + 2) // 2
-        ksteps = -(-ksteps // 32) * 32 if ksteps > 64 else (-(-ksteps // 4) * 4 if ksteps > 32 else ksteps)
+        # Flop the matrix sweep executed per tile pair it did not skip.  Up to 125 dimensions: three products of
+        # bf16 terms over the dimensions padded to 16 (v_mfma_f32_32x32x16_bf16); beyond: float products over the
+        # padded dimensions (v_mfma_f32_32x32x2_f32).
         tiles = -(-n // 128)
-        flop = 2.0 * 128 * 128 * (2 * ksteps) * tiles * tiles * knn_stats[2] / 1000.0
+        if d + 3 <= 128:
+            per_pair, peak, pipe = 2.0 * 128 * 128 * 3 * (-(-(d + 3) // 16) * 16), 2500.0, "bf16"
+        else:
+            ksteps = (((d + 1) & ~1) + 2) // 2
+            ksteps = -(-ksteps // 32) * 32 if ksteps > 64 else (-(-ksteps // 4) * 4 if ksteps > 32 else ksteps)
+            per_pair, peak, pipe = 2.0 * 128 * 128 * (2 * ksteps), 157.3, "fp32"
+        flop = per_pair * tiles * tiles * knn_stats[2] / 1000.0
         phase_rooflines["knn"] = {"bound": "mfma", "flop": flop, "achieved": flop / knn_s / 1e12, "unit": "TFLOP/s",
-                                  "frac": flop / knn_s / 1e12 / 157.3, "tile_pairs_per_mille": knn_stats[2],
-                                  "note": "fp32 matrix peak; time of the whole kNN call (sweep, re-rank, packing)"}
+                                  "frac": flop / knn_s / 1e12 / peak, "tile_pairs_per_mille": knn_stats[2],
+                                  "note": pipe + " matrix peak; time of the whole kNN call (sweep, re-rank, packing)"}
 
     # One-shot stages that are HBM problems (algorithmic bytes: what the stage must read and write once).
     nnz = float(n) * k
