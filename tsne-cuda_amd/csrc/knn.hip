@@ -292,12 +292,18 @@ __device__ __forceinline__ void compact_query(u64 *list, int cap, int want, int 
 // (LDS operations of a wave execute in order; the wavefront fences only stop the compiler from
 // reordering them), so the other waves keep issuing matrix instructions meanwhile.
 __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        const int o = __shfl_up(v, off, kWave);
-        if (lane >= off) v += o;
-    }
-    return v;
+    // Within the rows of 16 lanes by DPP row shifts (a lane without a source adds 0), then the row totals
+    // across the rows by the two row broadcasts (lane 15 of a row to the next row: rows 1 and 3; lane 31 to
+    // rows 2 and 3).  Twelve vector instructions; six ds_bpermute round trips through LDS before.
+    (void)lane;
+    int x = v;
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, true);   // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, true);   // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, true);   // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, true);   // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false);  // row_bcast:15
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false);  // row_bcast:31
+    return x;
 }
 
 // list: this query's entries in global memory (n = *cnt of them); buf: cap keys of LDS; hist: 64 words
@@ -371,10 +377,10 @@ __device__ __forceinline__ int wave_select(u64 *list, int want, int *cnt, u64 *t
         const int c = (int)hist[lane];
         const int incl = wave_inclusive_scan(c, lane);
         const int b = __ffsll((long long)__ballot(incl >= rank)) - 1;  // some lane qualifies: the last one holds all matches
-        rank -= __shfl(incl - c, b, kWave);
+        rank -= __builtin_amdgcn_readlane(incl - c, b);  // (b is the same in every lane)
         prefix = (prefix << w) | (unsigned int)b;
         if (slack > 0 && shift > 0) {
-            const int kept = (want - rank) + __shfl(c, b, kWave);  // below the bin + the whole bin
+            const int kept = (want - rank) + __builtin_amdgcn_readlane(c, b);  // below the bin + the whole bin
             if (kept <= want + slack) {
                 // Keep everything up to the upper edge of the bin.
                 const u64 edge = (u64)lo + ((((u64)prefix + 1ull) << shift) - 1ull);
