@@ -28,6 +28,12 @@
 //    >= tau - g for a rigorous rounding bound g, and the query passes when its
 //    K-th canonical distance is below that.  Queries that do not pass are redone
 //    by the VALU sweep, so the result is exact either way.
+//    Up to 125 dimensions the products run on the bf16 matrix pipe instead
+//    (v_mfma_f32_32x32x16_bf16, two bf16 terms per coordinate, three products):
+//    the candidates are stored relative to the centre m of their own 128-point
+//    tile, which keeps what the split leaves out small, |q - m|^2 is added on
+//    the vector ALU per (query, tile), and the keys are the distances less the
+//    tile's error bound - lower bounds, so the proof above needs no g.
 //
 //  * Chunked MFMA sweep (more than 126 dimensions): the same products, but the
 //    queries no longer fit a wave's registers, so both operands stream in chunks
