@@ -737,10 +737,12 @@ struct SweepArgs {
 // ---------------------------------------------------------------------------
 // MFMA sweep, in two arithmetic variants.
 // BF16 = false: KSTEPS = Daug / 2 k-steps of v_mfma_f32_32x32x2f32 on the points as floats.
-// BF16 = true: KSTEPS steps of 16 dimensions of v_mfma_f32_32x32x16_bf16 on the points split into two bf16
-// terms per coordinate; high x high, high x low and low x high are accumulated (three instructions per
-// step), which leaves out terms below 3 * 2^-16 of |q_d c_d| per dimension - the re-rank's verification
-// bound accounts for them.  A step of 16 dimensions takes half the matrix-pipe time of one fp32 step of 2.
+// BF16 = true: KSTEPS steps of 16 dimensions of v_mfma_f32_32x32x16_bf16 on the points relative to their
+// tile's centre, split into two bf16 terms per coordinate; high x high, high x low and low x high are
+// accumulated (three instructions per step), which leaves out terms below 3.1 * 2^-16 of |q_d delta_d| per
+// dimension.  The keys stored are the products plus |q - centre|^2 less the tile's error bound (see
+// pack_tile_centres_kernel): lower bounds of the distances.  A step of 16 dimensions takes half the
+// matrix-pipe time of one fp32 step of 2.
 // Dynamic LDS: one candidate tile, copied verbatim from the packed points
 //   a[cand block (4)][step group (S4)][lane (64)] float4   (4 steps per float4)            fp32
 //   a[cand block (4)][term (2)][step (KSTEPS)][lane (64)] 8 x bf16                          bf16
