@@ -721,7 +721,13 @@ def test_iterate_with_prepared_pattern(stages, c0_problem):
 @pytest.mark.parametrize("n,d,k", [
     (3000, 50, 90),    # the benchmark's shape at small N
     (700, 7, 20),      # odd dimension count, fewer candidates than the K' margin wants
-    (1500, 126, 33),   # the largest dimension count one wave's registers hold
+    (1500, 126, 33),   # the largest dimension count one wave's registers hold (products on floats)
+    (1500, 125, 33),   # the largest on bf16 terms (8 steps of 16 dimensions, the last three carry beta)
+    (1300, 13, 25),    # bf16: one step, beta in its last three dimensions
+    (1300, 14, 25),    # bf16: beta straddles two steps
+    (1400, 61, 30),    # bf16: four full steps
+    (1400, 62, 30),    # bf16: five steps (one workgroup per compute unit)
+    (1400, 1, 10),     # one dimension
     (1500, 127, 33),   # the first that is cut into chunks (3 chunks, the norm row opens the last one)
     (2200, 190, 40),   # 3 chunks, the last one full but for the norm row's partner
     (1200, 784, 50),   # config c1's dimension count (13 chunks)
