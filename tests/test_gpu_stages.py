@@ -727,6 +727,9 @@ def test_iterate_with_prepared_pattern(stages, c0_problem):
     (1300, 14, 25),    # bf16: beta straddles two steps
     (1400, 61, 30),    # bf16: four full steps
     (1400, 62, 30),    # bf16: five steps (one workgroup per compute unit)
+    (1400, 40, 30),    # bf16: three steps
+    (1400, 90, 30),    # bf16: six steps
+    (1400, 100, 30),   # bf16: seven steps
     (1400, 1, 10),     # one dimension
     (1500, 127, 33),   # the first that is cut into chunks (3 chunks, the norm row opens the last one)
     (2200, 190, 40),   # 3 chunks, the last one full but for the norm row's partner
