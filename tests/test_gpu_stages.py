@@ -759,7 +759,7 @@ def test_knn_matrix_sweep_is_exact(stages, n, d, k):
     assert torch.equal(idx_f, idx) and torch.equal(d2_f, d2)
 
 
-@pytest.mark.parametrize("scale,d", [(30.0, 12), (2.5, 6), (0.7, 4), (6.0, 160), (0.3, 140)])
+@pytest.mark.parametrize("scale,d", [(30.0, 12), (2.5, 6), (0.7, 4), (6.0, 160), (0.3, 140), (10.0, 50), (4.0, 100)])
 def test_knn_tile_skipping_is_exact(stages, scale, d):
     """On locality-ordered points both sweeps skip candidate tiles by their
     bounding balls.  Well separated clusters (most tiles skipped), touching
