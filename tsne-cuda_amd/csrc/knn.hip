@@ -762,8 +762,11 @@ struct SweepArgs {
 // (+inf when fewer than `want` candidates exist), both without the |q|^2 term.
 // ---------------------------------------------------------------------------
 // Workgroups per compute unit the register budget is set for (bf16: the query's coordinates stay in
-// registers beside the two operand terms; three workgroups would spill at 3 steps and beyond).
-constexpr int bf16_sweep_occupancy(int steps) { return steps <= 2 ? 3 : (steps <= 4 ? 2 : 1); }
+// registers beside the two operand terms).  Measured: three workgroups with 330 bytes of spills per lane
+// ran at half the speed of two at 4 steps; two workgroups beat one at 5 to 7 steps in spite of 100 to 380
+// bytes of spills (300,000 points, 64 / 90 / 100 dimensions: 0.040 -> 0.027 s, 0.044 -> 0.033 s,
+// 0.045 -> 0.040 s); at 8 steps two tiles of 66 KB do not fit a compute unit's LDS.
+constexpr int bf16_sweep_occupancy(int steps) { return steps <= 2 ? 3 : (steps <= 7 ? 2 : 1); }
 template <int KSTEPS, bool BF16>
 constexpr int sweep_occupancy() {
     return BF16 ? bf16_sweep_occupancy(KSTEPS) : (KSTEPS <= 28 ? 3 : 1);
