@@ -254,6 +254,90 @@ __global__ __launch_bounds__(64) void pack_tile_centres_kernel(const float *__re
     Xb[(size_t)tile * (S16 * 512 + 64) + S16 * 512 + l] = make_float4(v[0], v[1], v[2], v[3]);
 }
 
+// The bf16 operands of the chunked sweep, in its layout [tile][block of 32 points (4)][chunk of 64 dimensions]
+// [slot (8)][lane (64)] 8 x bf16 with slot = 4 * term + step (step: 16 dimensions of the chunk; lane and
+// element as in pack_points_bf16_kernel).  Candidate side: the points relative to their tile's centre in two
+// terms, beta in dimensions D .. D + 2 of the high term.  Query side: -2 x in two terms, 1 in those three.
+__global__ __launch_bounds__(256) void pack_points_bf16_chunked_kernel(const float *__restrict__ X,
+                                                                       const float *__restrict__ centers_t, int N,
+                                                                       int D, int n_chunks, int T, int Npad,
+                                                                       uint4 *__restrict__ Xb, bool query_side) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // one lane's 8 values per thread
+    const int64_t total = (int64_t)Npad * n_chunks * 16;
+    if (t >= total) return;
+    const int lane = (int)(t & 63);
+    int64_t rest = t >> 6;
+    const int slot = (int)(rest & 7);
+    rest >>= 3;
+    const int chunk = (int)(rest % n_chunks);
+    const int64_t blk = rest / n_chunks;  // tile * 4 + block
+    const int tile = (int)(blk >> 2);
+    const int term = slot >> 2, step = slot & 3;
+    const int i = (int)(blk * 32 + (lane & 31));
+    const int d0 = 64 * chunk + 16 * step + 8 * (lane >> 5);
+    unsigned int h[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+    if (i < N) {
+        float beta = 0.0f;
+        if (!query_side && term == 0 && d0 + 8 > D && d0 < D + 3) {
+            float sq = 0.0f, dot = 0.0f;
+            for (int d = 0; d < D; ++d) {
+                const float m = centers_t[(size_t)d * T + tile];
+                const float delta = X[(size_t)i * D + d] - m;
+                sq = fmaf(delta, delta, sq);
+                dot = fmaf(m, delta, dot);
+            }
+            beta = fmaf(2.0f, dot, sq);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int d = d0 + j;
+            if (d < D) {
+                const float x = X[(size_t)i * D + d];
+                const float v = query_side ? -2.0f * x : x - centers_t[(size_t)d * T + tile];
+                const unsigned int hi = bf16_bits(v);
+                h[j] = term == 0 ? hi : bf16_bits(v - bf16_value(hi));
+            } else if (d < D + 3 && term == 0) {
+                if (query_side) {
+                    h[j] = 0x3f80u;
+                } else {
+                    float r = beta;
+                    unsigned int part = bf16_bits(r);
+                    for (int k = D; k < d; ++k) {
+                        r -= bf16_value(part);
+                        part = bf16_bits(r);
+                    }
+                    h[j] = part;
+                }
+            }
+        }
+    }
+    Xb[t] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+}
+
+// Tile centres for the chunked bf16 sweep: centres_p[tile][64 n_chunks] and the two error coefficients of
+// pack_tile_centres_kernel in tile_coef[2 tile], [2 tile + 1].  Beyond D the centre is zero, except -1/2 in
+// dimensions D .. D + 2: the sweep forms |q - m|^2 from the query-side operand, which holds 1 there and
+// stands for -2 q, so those three dimensions add nothing.
+__global__ __launch_bounds__(64) void pack_chunked_centres_kernel(const float *__restrict__ centers_t,
+                                                                  const float *__restrict__ radius, int D,
+                                                                  int n_chunks, int T, float *__restrict__ centres_p,
+                                                                  float *__restrict__ tile_coef) {
+    const int tile = blockIdx.x, l = threadIdx.x;
+    float m2 = 0.0f;
+    for (int d = l; d < 64 * n_chunks; d += 64) {
+        const float m = d < D ? centers_t[(size_t)d * T + tile] : 0.0f;
+        centres_p[(size_t)tile * 64 * n_chunks + d] = d >= D && d < D + 3 ? -0.5f : m;
+        m2 = fmaf(m, m, m2);
+    }
+    m2 = group_sum<kWave>(m2);
+    if (l == 0) {
+        const float r = radius[tile], mlen = sqrtf(m2) * (1.0f + 1e-5f);
+        const float split = 6.2f / 65536.0f, acc = 4.0f * (float)(3 * D + 6) * 5.9604644775390625e-08f;
+        tile_coef[2 * tile] = 1.01f * (split + 2.0f * acc) * r;
+        tile_coef[2 * tile + 1] = 1.01f * acc * (r * r + 2.0f * mlen * r) + 1e-30f;
+    }
+}
+
 // Sorts sortbuf[0..cap) ascending (cap a power of two), all 256 threads.
 __device__ __forceinline__ void bitonic_sort(u64 *sortbuf, int cap, int tid) {
     for (int k = 2; k <= cap; k <<= 1) {
@@ -702,6 +786,7 @@ __global__ __launch_bounds__(256) void knn_merge_slices_kernel(const u64 *__rest
 struct SweepArgs {
     const float4 *Xp;
     const float *X;  // the points as given (bf16 sweep: the query side is formed from them)
+    const float *centres_p, *tile_coef;  // chunked bf16 sweep: tile centres by chunk, error coefficients
     int N, D, Dnorm, want, cap;
     u64 *lists;
     int num_qtiles;
@@ -1197,6 +1282,7 @@ constexpr int kChunkSteps = 32;
 constexpr int kChunkS4 = kChunkSteps / 4;            // float4 per lane, block and chunk
 constexpr int kChunkFloat4 = 4 * kChunkS4 * 64;      // float4 per tile chunk
 
+template <bool BF16>
 __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const SweepArgs args) {
     const int N = args.N, D = args.D, want = args.want, cap = args.cap;
     const int num_qtiles = args.num_qtiles, n_chunks = args.n_chunks;
@@ -1244,6 +1330,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
             thr[tid] = ~0ull;
             cnt[tid] = 0;
         }
+        const float q_len = BF16 && q < N ? sqrtf(args.norms[q]) * (1.0f + 1e-6f) : 0.0f;  // |q|, rounded up
         // This wave's block of the query-side copy.
         const v4f *bsrc = reinterpret_cast<const v4f *>(args.Bp) + (size_t)qt * tile_stride + (size_t)wave * block_stride + lane;
         v4f bcur[kChunkS4], bnext[kChunkS4];
@@ -1259,8 +1346,18 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
             for (int b = 0; b < 4; ++b)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+            float f_part = 0.0f;  // bf16: this lane's share of |q - m|^2 (m: the tile's centre)
             for (int c = 0; c < n_chunks; ++c) {
                 const bool last = c + 1 == n_chunks;
+                v4f mc[kChunkS4];  // bf16: the centre's 32 coordinates that go with this lane's 32 of the chunk
+                if constexpr (BF16) {
+                    const v4f *msrc = reinterpret_cast<const v4f *>(args.centres_p) + (size_t)ct * (16 * n_chunks) + 16 * c + 2 * kh;
+#pragma unroll
+                    for (int step = 0; step < 4; ++step) {
+                        mc[2 * step] = msrc[4 * step];
+                        mc[2 * step + 1] = msrc[4 * step + 1];
+                    }
+                }
                 if (!last) fetch(ct, c + 1);
                 else if (next_ct >= 0) fetch(next_ct, 0);
                 {
@@ -1268,16 +1365,51 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
 #pragma unroll
                     for (int s4 = 0; s4 < kChunkS4; ++s4) bnext[s4] = bn[s4 * 64];
                 }
+                if constexpr (BF16) {
 #pragma unroll
-                for (int s4 = 0; s4 < kChunkS4; ++s4) {
-                    v4f x[4];
+                    for (int step = 0; step < 4; ++step) {
+                        v4f xh[4], xl[4];
 #pragma unroll
-                    for (int b = 0; b < 4; ++b) x[b] = a_lds[(b * kChunkS4 + s4) * 64 + lane];
-#pragma unroll
-                    for (int k = 0; k < 4; ++k)
+                        for (int b = 0; b < 4; ++b) {
+                            xh[b] = a_lds[(b * kChunkS4 + step) * 64 + lane];
+                            xl[b] = a_lds[(b * kChunkS4 + 4 + step) * 64 + lane];
+                        }
+                        const v8bf qh = __builtin_bit_cast(v8bf, bcur[step]), ql = __builtin_bit_cast(v8bf, bcur[4 + step]);
 #pragma unroll
                         for (int b = 0; b < 4; ++b)
-                            acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(x[b][k], bcur[s4][k], acc[b], 0, 0, 0);
+                            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xh[b]), qh, acc[b], 0, 0, 0);
+#pragma unroll
+                        for (int b = 0; b < 4; ++b)
+                            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xh[b]), ql, acc[b], 0, 0, 0);
+#pragma unroll
+                        for (int b = 0; b < 4; ++b)
+                            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xl[b]), qh, acc[b], 0, 0, 0);
+                        // |q - m|^2 from the query's two terms: q_d = -(high + low) / 2 to within 2^-16 |q_d|.
+                        const uint4 uh = __builtin_bit_cast(uint4, bcur[step]), ul = __builtin_bit_cast(uint4, bcur[4 + step]);
+                        const unsigned int wh[4] = {uh.x, uh.y, uh.z, uh.w}, wl[4] = {ul.x, ul.y, ul.z, ul.w};
+                        const float m[8] = {mc[2 * step][0], mc[2 * step][1], mc[2 * step][2], mc[2 * step][3],
+                                            mc[2 * step + 1][0], mc[2 * step + 1][1], mc[2 * step + 1][2], mc[2 * step + 1][3]};
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const float s0 = __uint_as_float(wh[k] << 16) + __uint_as_float(wl[k] << 16);
+                            const float s1 = __uint_as_float(wh[k] & 0xffff0000u) + __uint_as_float(wl[k] & 0xffff0000u);
+                            const float e0 = fmaf(-0.5f, s0, -m[2 * k]), e1 = fmaf(-0.5f, s1, -m[2 * k + 1]);
+                            f_part = fmaf(e0, e0, f_part);
+                            f_part = fmaf(e1, e1, f_part);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int s4 = 0; s4 < kChunkS4; ++s4) {
+                        v4f x[4];
+#pragma unroll
+                        for (int b = 0; b < 4; ++b) x[b] = a_lds[(b * kChunkS4 + s4) * 64 + lane];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+#pragma unroll
+                            for (int b = 0; b < 4; ++b)
+                                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(x[b][k], bcur[s4][k], acc[b], 0, 0, 0);
+                    }
                 }
                 if (!last) {
                     __syncthreads();  // all waves have read this chunk
@@ -1293,7 +1425,18 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
             // Never +inf: excluded elements are raised to +inf and must fail the test also while the query
             // has no threshold yet (a part can hold fewer than `want` real candidates, so nothing would
             // push them out of the list later).
-            const float lim = q < N ? fminf(limit_d, 3.4028234663852886e38f) : -INFINITY;
+            // bf16: the keys are lower bounds of the distances: product + `off`, off = |q - m|^2 rounded down
+            // (the rounding of its sum, and the 2^-16 |q| by which the query's two terms miss q) less the tile's
+            // error bound; the products are tested against the threshold less `off`, rounded up.
+            float off = 0.0f, limit_acc = limit_d;
+            if constexpr (BF16) {
+                const float f = f_part + __shfl_xor(f_part, 32);
+                off = f * (1.0f - (float)(D + 4) * 5.9604644775390625e-08f) - 2.1f / 65536.0f * q_len * sqrtf(f) -
+                      fmaf(q_len, args.tile_coef[2 * ct], args.tile_coef[2 * ct + 1]);
+                limit_acc = limit_d - off;
+                limit_acc += 2.4e-7f * (fabsf(limit_d) + fabsf(off));
+            }
+            const float lim = q < N ? fminf(limit_acc, 3.4028234663852886e38f) : -INFINITY;
             const bool edge_tile = c0 + kCT > N || (unsigned int)(q0 - c0) < (unsigned int)kCT;
 #pragma unroll
             for (int cb = 0; cb < 4; cb += 2) {
@@ -1306,7 +1449,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
 #pragma unroll
                 for (int v = 1; v + 1 < 16; v += 2) best = min3(best, acc1[v], acc1[v + 1]);
                 best = min2(best, acc1[15]);
-                if (best <= limit_d) {
+                if (best <= limit_acc) {
                     const int jbase = c0 + cb * 32 + 4 * kh;  // element (half, v) is candidate jbase + 32 half + 8 (v / 4) + v % 4
                     // Candidates beyond N (last tile) and the query itself (its own tile) are raised to +inf.
                     if (edge_tile) {
@@ -1329,7 +1472,8 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
 #pragma unroll
                         for (int e = 0; e < 32; ++e) {
                             const float dist = e < 16 ? acc0[e & 15] : acc1[e & 15];
-                            if (dist <= lim2) *dst++ = pack_key(dist, jbase + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
+                            if (dist <= lim2)
+                                *dst++ = pack_key(BF16 ? dist + off : dist, jbase + 32 * (e >> 4) + 8 * ((e & 15) >> 2) + (e & 3));
                         }
                     }
                 }
@@ -1395,7 +1539,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                     float v = -INFINITY;
                     if (q0 + tid < N) {
                         const u64 t = thr[tid];
-                        v = t == ~0ull ? INFINITY : key_distance(t) + args.norms[q0 + tid];
+                        v = t == ~0ull ? INFINITY : key_distance(t) + (BF16 ? 0.0f : args.norms[q0 + tid]);
                         v += 1e-5f * fabsf(v) + 1e-30f;
                     }
                     v = group_max<kWave>(v);
@@ -1781,14 +1925,15 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     const int Dnorm = (D + 1) & ~1;        // |x|^2 row: first even row after the real dimensions
     int ksteps = (Dnorm + 2) / 2;          // k-steps incl. the augmented pair
     const bool chunked = ksteps > kMfmaMaxSteps;  // more dimensions than one wave's registers hold
-    const int n_chunks = chunked ? div_up(ksteps, kChunkSteps) : 0;
-    if (chunked) ksteps = n_chunks * kChunkSteps;
-    else if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
-    // Up to 125 dimensions the sweep multiplies bf16 terms (two per coordinate) of the points relative to
-    // their tile's centre.
+    // Unless mode 3 asks for products of floats, the sweeps multiply bf16 terms (two per coordinate) of the
+    // points relative to their tile's centre; three more dimensions carry a per-point term.
     const bool force_f32 = mode == 3;
     if (mode == 3) mode = 2;
     const bool bf16 = !chunked && !force_f32 && D + 3 <= 128;
+    const bool bf16_chunked = chunked && !force_f32;
+    const int n_chunks = chunked ? (bf16_chunked ? div_up(D + 3, 64) : div_up(ksteps, kChunkSteps)) : 0;
+    if (chunked) ksteps = n_chunks * kChunkSteps;
+    else if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
     const int steps16 = div_up(D + 3, 16);
     const int num_tiles = div_up(N, kCT);
     const int bitmap_words = div_up(num_tiles, 32);
@@ -1851,12 +1996,12 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     TSNE_TRY(hipMemsetAsync(scal.p, 0, 4 * sizeof(int), s));  // [0] max |x|^2 (float bits), [1] fail count, [2..3] tiles swept (64-bit)
     norms_kernel<<<div_up(Npad, 256), 256, 0, s>>>(points, N, D, Npad, norms.as<float>(), scal.as<float>());
     TSNE_TRY(hipGetLastError());
-    if (!bf16) {
+    if (!bf16 && !bf16_chunked) {
         pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm,
                                                                               S4, Npad, Xp.as<float4>(), false);
         TSNE_TRY(hipGetLastError());
     }
-    if (chunked) {
+    if (chunked && !bf16_chunked) {
         pack_points_kernel<<<div_up((int64_t)Npad * S4 * 2, 256), 256, 0, s>>>(points, norms.as<float>(), N, D, Dnorm,
                                                                               S4, Npad, Bp.as<float4>(), true);
         TSNE_TRY(hipGetLastError());
@@ -1870,6 +2015,24 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         TSNE_TRY(hipGetLastError());
         pack_tile_centres_kernel<<<num_tiles, 64, 0, s>>>(centers.as<float>(), radius.as<float>(), D, steps16,
                                                          num_tiles, Xp.as<float4>());
+        TSNE_TRY(hipGetLastError());
+    }
+    DeviceMem centres_p, tile_coef;
+    if (bf16_chunked) {
+        if (!centres_p.alloc(sizeof(float) * 64 * (size_t)n_chunks * num_tiles) ||
+            !tile_coef.alloc(sizeof(float) * 2 * (size_t)num_tiles)) {
+            set_error("knn: out of device memory for the tile centres");
+            return 1;
+        }
+        const int64_t pieces = (int64_t)Npad * n_chunks * 16;
+        pack_points_bf16_chunked_kernel<<<div_up(pieces, 256), 256, 0, s>>>(points, centers.as<float>(), N, D, n_chunks,
+                                                                           num_tiles, Npad, Xp.as<uint4>(), false);
+        TSNE_TRY(hipGetLastError());
+        pack_points_bf16_chunked_kernel<<<div_up(pieces, 256), 256, 0, s>>>(points, centers.as<float>(), N, D, n_chunks,
+                                                                           num_tiles, Npad, Bp.as<uint4>(), true);
+        TSNE_TRY(hipGetLastError());
+        pack_chunked_centres_kernel<<<num_tiles, 64, 0, s>>>(centers.as<float>(), radius.as<float>(), D, n_chunks,
+                                                            num_tiles, centres_p.as<float>(), tile_coef.as<float>());
         TSNE_TRY(hipGetLastError());
     }
 
@@ -1901,6 +2064,8 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         SweepArgs args;
         args.Xp = Xp.as<float4>();
         args.X = points;
+        args.centres_p = centres_p.as<float>();
+        args.tile_coef = tile_coef.as<float>();
         args.N = N;
         args.D = D;
         args.Dnorm = Dnorm;
@@ -1930,9 +2095,15 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         args.probe_list_tiles = probes ? probes->list_tiles : nullptr;
         if (chunked) {
             const size_t lds = sweep_lds(keep);
-            TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_chunked_sweep_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            knn_mfma_chunked_sweep_kernel<<<grid, 256, lds, s>>>(args);
+            if (bf16_chunked) {
+                TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_chunked_sweep_kernel<true>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                knn_mfma_chunked_sweep_kernel<true><<<grid, 256, lds, s>>>(args);
+            } else {
+                TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(knn_mfma_chunked_sweep_kernel<false>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                knn_mfma_chunked_sweep_kernel<false><<<grid, 256, lds, s>>>(args);
+            }
             TSNE_TRY(hipGetLastError());
         } else if (bf16 ? dispatch_bf16_sweep(steps16, args, grid, s) : dispatch_mfma_sweep(ksteps, args, grid, s)) {
             return 1;
@@ -1953,7 +2124,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         knn_rerank_kernel<<<div_up((int)n_slots, 4), 256, sizeof(u64) * 4 * sort_n, s>>>(
             points, norms.as<float>(), N, D, K, keep, sort_n, cand.as<int>(), tau.as<float>(), scal.as<float>(),
             indices, sq_dist, scal.as<int>() + 1, fail_list.as<int>(), tile_list, first, step, (int)n_slots,
-            bf16 ? 1 : 0);
+            bf16 || bf16_chunked ? 1 : 0);
         TSNE_TRY(hipGetLastError());
         int host_scal[4] = {0, 0, 0, 0};
         TSNE_TRY(hipMemcpyAsync(host_scal, scal.p, sizeof(host_scal), hipMemcpyDeviceToHost, s));
@@ -1994,11 +2165,11 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
         stats[1] = failed;
         stats[2] = (int)((1000.0 * (double)swept) / ((double)num_tiles * (double)num_tiles) + 0.5);
     }
-    // Up to a few query tiles' worth of failures go straight to the vector sweep, which spreads a short list of
-    // queries over the chip by candidate range.  Beyond that the chunked sweep takes the tiles of the queries
-    // that failed once more with twice the margin (a vector sweep of many query tiles over all points in hundreds
-    // of dimensions takes as long as the whole matrix sweep); what fails again, and every failure of the
-    // register-resident sweep, goes to the vector sweep.
+    // Few failures, or failures scattered thinly over the query tiles, go straight to the vector sweep, which
+    // spreads a list of queries over the chip by candidate range.  Where a quarter or more of the queries of the
+    // tiles concerned failed, the chunked sweep takes those tiles once more with twice the margin (a vector sweep
+    // of that many queries over all points in hundreds of dimensions takes longer than the matrix sweep of their
+    // tiles); what fails again, and every failure of the register-resident sweep, goes to the vector sweep.
     if (failed > 4 * kQT && chunked && failed * 10 <= N) {
         const int wider = std::min(N - 1, 2 * want);
         if (wider != want && sweep_fits(wider)) {
@@ -2007,14 +2178,17 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
             for (int q : queries) tiles.push_back(q / kMQ);
             std::sort(tiles.begin(), tiles.end());
             tiles.erase(std::unique(tiles.begin(), tiles.end()), tiles.end());
-            DeviceMem tile_list;
-            if (!tile_list.alloc(sizeof(int) * tiles.size())) {
-                set_error("knn: out of device memory for the retry list");
-                return 1;
+            if ((size_t)failed * 4 >= tiles.size() * kMQ) {
+                DeviceMem tile_list;
+                if (!tile_list.alloc(sizeof(int) * tiles.size())) {
+                    set_error("knn: out of device memory for the retry list");
+                    return 1;
+                }
+                TSNE_TRY(hipMemcpy(tile_list.p, tiles.data(), sizeof(int) * tiles.size(), hipMemcpyHostToDevice));
+                unsigned long long swept_again = 0;
+                if (sweep_and_rerank(wider, tile_list.as<int>(), 0, 1, (int)tiles.size(), failed, swept_again))
+                    return 1;
             }
-            TSNE_TRY(hipMemcpy(tile_list.p, tiles.data(), sizeof(int) * tiles.size(), hipMemcpyHostToDevice));
-            unsigned long long swept_again = 0;
-            if (sweep_and_rerank(wider, tile_list.as<int>(), 0, 1, (int)tiles.size(), failed, swept_again)) return 1;
         }
     }
     if (failed > 0) {
