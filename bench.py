@@ -186,16 +186,15 @@ def main():
                "frac": b / (kernels_us[name] * 1e-6) / 1e9 / HBM_PEAK_GBS}
         for name, b in loop_bytes.items() if kernels_us.get(name)}
     if knn_stats[0] == 1:
-        # Flop the matrix sweep executed per tile pair it did not skip.  Up to 125 dimensions: three products of
-        # bf16 terms over the dimensions padded to 16 (v_mfma_f32_32x32x16_bf16); beyond: float products over the
-        # padded dimensions (v_mfma_f32_32x32x2_f32).
+        # Flop the matrix sweep executed per tile pair it did not skip: three products of bf16 terms
+        # (v_mfma_f32_32x32x16_bf16) over the dimensions + 3, padded to 16 (up to 125 dimensions) or to 64 (chunked
+        # sweep, beyond 126); at exactly 126 dimensions float products over 128 (v_mfma_f32_32x32x2_f32).
         tiles = -(-n // 128)
-        if d + 3 <= 128:
-            per_pair, peak, pipe = 2.0 * 128 * 128 * 3 * (-(-(d + 3) // 16) * 16), 2500.0, "bf16"
+        if d == 126:
+            per_pair, peak, pipe = 2.0 * 128 * 128 * 128, 157.3, "fp32"
         else:
-            ksteps = (((d + 1) & ~1) + 2) // 2
-            ksteps = -(-ksteps // 32) * 32 if ksteps > 64 else (-(-ksteps // 4) * 4 if ksteps > 32 else ksteps)
-            per_pair, peak, pipe = 2.0 * 128 * 128 * (2 * ksteps), 157.3, "fp32"
+            pad = 16 if d + 3 <= 128 else 64
+            per_pair, peak, pipe = 2.0 * 128 * 128 * 3 * (-(-(d + 3) // pad) * pad), 2500.0, "bf16"
         flop = per_pair * tiles * tiles * knn_stats[2] / 1000.0
         phase_rooflines["knn"] = {"bound": "mfma", "flop": flop, "achieved": flop / knn_s / 1e12, "unit": "TFLOP/s",
                                   "frac": flop / knn_s / 1e12 / peak, "tile_pairs_per_mille": knn_stats[2],

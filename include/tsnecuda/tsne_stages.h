@@ -48,7 +48,7 @@ int tsne_hip_knn(const float *points, int num_points, int num_dims, int num_neig
  * shape (what tsne_hip_knn does), 1 = vector-ALU sweep, 2 = matrix-instruction
  * (MFMA) candidate sweep followed by an exact re-rank and verification (up to
  * 126 dimensions the queries stay in registers; beyond, both operands stream in
- * chunks of 64 dimensions; up to 125 dimensions the candidate distances are
+ * chunks of 64 dimensions; except at 126 dimensions the candidate distances are
  * products of bf16 terms, two per coordinate, on the bf16 matrix pipe), 3 = as 2
  * with the candidate distances as products of floats throughout.  Results are
  * identical whichever sweep runs.  stats

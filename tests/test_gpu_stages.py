@@ -753,7 +753,7 @@ def test_knn_matrix_sweep_is_exact(stages, n, d, k):
     idx_v, d2_v, stats_v = stages.knn_select(dev(X), k, 1)
     assert stats_v[0] == 0
     assert torch.equal(idx_v, idx) and torch.equal(d2_v, d2)
-    # up to 125 dimensions sweep 2 multiplies bf16 terms; sweep 3 keeps the products on floats
+    # sweep 2 multiplies bf16 terms (except at 126 dimensions); sweep 3 keeps the products on floats
     idx_f, d2_f, stats_f = stages.knn_select(dev(X), k, 3)
     assert stats_f[0] == 1
     assert torch.equal(idx_f, idx) and torch.equal(d2_f, d2)

@@ -28,18 +28,19 @@
 //    >= tau - g for a rigorous rounding bound g, and the query passes when its
 //    K-th canonical distance is below that.  Queries that do not pass are redone
 //    by the VALU sweep, so the result is exact either way.
-//    Up to 125 dimensions the products run on the bf16 matrix pipe instead
+//    Except at 126 dimensions the products run on the bf16 matrix pipe instead
 //    (v_mfma_f32_32x32x16_bf16, two bf16 terms per coordinate, three products):
 //    the candidates are stored relative to the centre m of their own 128-point
 //    tile, which keeps what the split leaves out small, |q - m|^2 is added on
 //    the vector ALU per (query, tile), and the keys are the distances less the
 //    tile's error bound - lower bounds, so the proof above needs no g.
 //
-//  * Chunked MFMA sweep (more than 126 dimensions): the same products, but the
-//    queries no longer fit a wave's registers, so both operands stream in chunks
-//    of 64 dimensions (candidates through LDS, queries straight into registers
-//    from a pre-scaled packed copy) while the 32 x 128 results of a wave
-//    accumulate in registers.  With hundreds of dimensions a query's neighbour
+//  * Chunked MFMA sweep (more than 126 dimensions): the same products (bf16
+//    terms by default), but the queries no longer fit a wave's registers, so
+//    both operands stream in chunks of 64 dimensions (candidates through LDS,
+//    queries straight into registers from a pre-scaled packed copy) while the
+//    32 x 128 results of a wave accumulate in registers; |q - m|^2 is formed
+//    chunk by chunk from the query-side operand and the centre's chunk.  With hundreds of dimensions a query's neighbour
 //    distances lie close together and the rounding bound g grows, so the margin
 //    K' - K is first tried on a sample of query tiles and doubled until the
 //    sample verifies (or the vector sweep is taken instead); the query tiles of
@@ -1893,7 +1894,7 @@ int run_valu_sweep(const float *points, const float *Xt, int N, int Npad, int D,
 }  // namespace
 
 // mode: 0 = choose, 1 = VALU sweep only, 2 = matrix-instruction sweep (error if the shape does not fit),
-// 3 = as 2 with the products on floats also where the bf16 split applies (up to 125 dimensions).
+// 3 = as 2 with the products on floats where 2 multiplies bf16 terms (every dimension count but 126).
 // stats (optional, 3 ints): [0] = 1 if the matrix-instruction sweep ran, [1] = queries redone by the VALU sweep,
 // [2] = per mille of the (query tile, candidate tile) pairs the matrix sweep computed.
 int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *sq_dist, hipStream_t s, int mode,

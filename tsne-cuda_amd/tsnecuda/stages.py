@@ -108,7 +108,7 @@ def knn(points, num_neighbors):
 
 def knn_select(points, num_neighbors, sweep):
     """knn() with an explicit sweep (1 = vector ALU, 2 = matrix instructions,
-    3 = matrix instructions on floats also where the bf16 terms apply).
+    3 = matrix instructions with the products on floats instead of bf16 terms).
     Returns (indices, sq_dist, stats) with stats = (matrix sweep ran, queries redone,
     per mille of tile pairs computed)."""
     points = _f32(points)
