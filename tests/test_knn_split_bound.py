@@ -42,8 +42,10 @@ def fp32_sum_random_order(terms, rng):
     return acc
 
 
-def keys_for_tile(Q, C, rng):
-    """Keys the sweep would store for queries Q against one candidate tile C (both float32, rows = points)."""
+def keys_for_tile(Q, C, rng, from_terms=False):
+    """Keys the sweep would store for queries Q against one candidate tile C (both float32, rows = points).
+    from_terms: the chunked sweep's way (more than 126 dimensions): |q - m|^2 from the query's two bf16
+    terms, -(high + low) / 2 for q, with 2.1 * 2^-16 |q| |q - m| taken off the key for what they miss."""
     D = C.shape[1]
     m = (C.sum(0, dtype=np.float32) / np.float32(len(C))).astype(np.float32)      # tile_balls_kernel's centre
     delta = (C - m).astype(np.float32)
@@ -71,11 +73,14 @@ def keys_for_tile(Q, C, rng):
                                 b2[:, None].astype(np.float64)], axis=1)
         product = fp32_sum_random_order(terms, rng)
         f = np.float32(0)
+        q_used = (np.float32(-0.5) * (wh + wl).astype(np.float32)).astype(np.float32) if from_terms else q
         for d in range(D):
-            diff = np.float32(q[d] - m[d])
+            diff = np.float32(q_used[d] - m[d])
             f = np.float32(np.float64(diff) * diff + f)
         q_len = np.float32(np.sqrt(np.float32((q.astype(np.float64) ** 2).sum())) * (1 + 1e-6))
         off = np.float32(f * np.float32(1.0 - (D + 4) * EPS)) - np.float32(q_len * ga + gb)
+        if from_terms:
+            off = np.float32(off - np.float32(2.1 / 65536.0) * q_len * np.float32(np.sqrt(f)))
         keys[i] = (product + np.float32(off)).astype(np.float32)
     return keys, float(ga), float(gb)
 
@@ -105,6 +110,20 @@ def test_keys_are_lower_bounds(name, d, center, sigma):
     # what the bound gives away stays of the order of |q| ga + gb
     q_len = np.sqrt((Q.astype(np.float64) ** 2).sum(1))[:, None]
     assert (exact - keys <= 2.5 * (q_len * ga + gb) + 1e-3 * exact + 1e-30).all(), name
+
+
+@pytest.mark.parametrize("d,center,sigma", [(200, 3.0, 1.0), (784, 3.0, 1.0), (130, 200.0, 0.05)])
+def test_keys_are_lower_bounds_with_the_query_from_its_terms(d, center, sigma):
+    rng = np.random.default_rng(d)
+    mu = rng.standard_normal(d) * center
+    C = (mu + rng.standard_normal((128, d)) * sigma).astype(np.float32)
+    Q = np.concatenate([(mu + rng.standard_normal((4, d)) * sigma), (rng.standard_normal((2, d)) * center),
+                        C[:2]]).astype(np.float32)
+    keys, ga, gb = keys_for_tile(Q, C, rng, from_terms=True)
+    exact = true_sq_dist(Q, C)
+    assert (keys.astype(np.float64) <= exact).all()
+    q_len = np.sqrt((Q.astype(np.float64) ** 2).sum(1))[:, None]
+    assert (exact - keys <= 2.5 * (q_len * ga + gb) + 2e-3 * exact + 1e-30).all()
 
 
 def test_mixed_scale_tile():
