@@ -1276,6 +1276,11 @@ __global__ __launch_bounds__(256, (sweep_occupancy<KSTEPS, BF16>())) void knn_mf
 // all four candidate blocks accumulate over the chunks in 64 registers.  The next chunk of the tile
 // (or the first of the next tile) and of the queries travel through registers meanwhile.  Visiting
 // order, tile skipping, filter, lists and output are those of the kernel above.
+// BF16 = true: the same 32 KB hold a chunk as [block (4)][term (2)][step of 16 dimensions (4)][lane (64)]
+// 8 x bf16 of the points relative to their tile's centre, the query side two terms of -2 q likewise, and the
+// products are those of the kernel above (three v_mfma_f32_32x32x16_bf16 per step); |q - centre|^2 is summed
+// over the chunks from the query side's two terms and the centre's chunk (pack_chunked_centres_kernel), and
+// the keys are lower bounds of the distances as there.
 // Dynamic LDS: one tile chunk, one sort buffer (cap keys) per wave, the visit bitmap, D floats
 // (centre of the query tile's ball).
 // ---------------------------------------------------------------------------
