@@ -37,7 +37,7 @@
 //
 //  * Chunked MFMA sweep (more than 126 dimensions): the same products (bf16
 //    terms by default), but the queries no longer fit a wave's registers, so
-//    both operands stream in chunks of 64 dimensions (candidates through LDS,
+//    both operands stream in chunks of 64 dimensions (32 on bf16 terms; candidates through LDS,
 //    queries straight into registers from a pre-scaled packed copy) while the
 //    32 x 128 results of a wave accumulate in registers; |q - m|^2 is formed
 //    chunk by chunk from the query-side operand and the centre's chunk.  With hundreds of dimensions a query's neighbour
@@ -255,8 +255,8 @@ __global__ __launch_bounds__(64) void pack_tile_centres_kernel(const float *__re
     Xb[(size_t)tile * (S16 * 512 + 64) + S16 * 512 + l] = make_float4(v[0], v[1], v[2], v[3]);
 }
 
-// The bf16 operands of the chunked sweep, in its layout [tile][block of 32 points (4)][chunk of 64 dimensions]
-// [slot (8)][lane (64)] 8 x bf16 with slot = 4 * term + step (step: 16 dimensions of the chunk; lane and
+// The bf16 operands of the chunked sweep, in its layout [tile][block of 32 points (4)][chunk of 32 dimensions]
+// [slot (4)][lane (64)] 8 x bf16 with slot = 2 * term + step (step: 16 dimensions of the chunk; lane and
 // element as in pack_points_bf16_kernel).  Candidate side: the points relative to their tile's centre in two
 // terms, beta in dimensions D .. D + 2 of the high term.  Query side: -2 x in two terms, 1 in those three.
 __global__ __launch_bounds__(256) void pack_points_bf16_chunked_kernel(const float *__restrict__ X,
@@ -264,18 +264,18 @@ __global__ __launch_bounds__(256) void pack_points_bf16_chunked_kernel(const flo
                                                                        int D, int n_chunks, int T, int Npad,
                                                                        uint4 *__restrict__ Xb, bool query_side) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // one lane's 8 values per thread
-    const int64_t total = (int64_t)Npad * n_chunks * 16;
+    const int64_t total = (int64_t)Npad * n_chunks * 8;
     if (t >= total) return;
     const int lane = (int)(t & 63);
     int64_t rest = t >> 6;
-    const int slot = (int)(rest & 7);
-    rest >>= 3;
+    const int slot = (int)(rest & 3);
+    rest >>= 2;
     const int chunk = (int)(rest % n_chunks);
     const int64_t blk = rest / n_chunks;  // tile * 4 + block
     const int tile = (int)(blk >> 2);
-    const int term = slot >> 2, step = slot & 3;
+    const int term = slot >> 1, step = slot & 1;
     const int i = (int)(blk * 32 + (lane & 31));
-    const int d0 = 64 * chunk + 16 * step + 8 * (lane >> 5);
+    const int d0 = 32 * chunk + 16 * step + 8 * (lane >> 5);
     unsigned int h[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
     if (i < N) {
         float beta = 0.0f;
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(256) void pack_points_bf16_chunked_kernel(const flo
     Xb[t] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
 }
 
-// Tile centres for the chunked bf16 sweep: centres_p[tile][64 n_chunks] and the two error coefficients of
+// Tile centres for the chunked bf16 sweep: centres_p[tile][32 n_chunks] and the two error coefficients of
 // pack_tile_centres_kernel in tile_coef[2 tile], [2 tile + 1].  Beyond D the centre is zero, except -1/2 in
 // dimensions D .. D + 2: the sweep forms |q - m|^2 from the query-side operand, which holds 1 there and
 // stands for -2 q, so those three dimensions add nothing.
@@ -325,9 +325,9 @@ __global__ __launch_bounds__(64) void pack_chunked_centres_kernel(const float *_
                                                                   float *__restrict__ tile_coef) {
     const int tile = blockIdx.x, l = threadIdx.x;
     float m2 = 0.0f;
-    for (int d = l; d < 64 * n_chunks; d += 64) {
+    for (int d = l; d < 32 * n_chunks; d += 64) {
         const float m = d < D ? centers_t[(size_t)d * T + tile] : 0.0f;
-        centres_p[(size_t)tile * 64 * n_chunks + d] = d >= D && d < D + 3 ? -0.5f : m;
+        centres_p[(size_t)tile * 32 * n_chunks + d] = d >= D && d < D + 3 ? -0.5f : m;
         m2 = fmaf(m, m, m2);
     }
     m2 = group_sum<kWave>(m2);
@@ -1276,7 +1276,7 @@ __global__ __launch_bounds__(256, (sweep_occupancy<KSTEPS, BF16>())) void knn_mf
 // all four candidate blocks accumulate over the chunks in 64 registers.  The next chunk of the tile
 // (or the first of the next tile) and of the queries travel through registers meanwhile.  Visiting
 // order, tile skipping, filter, lists and output are those of the kernel above.
-// BF16 = true: the same 32 KB hold a chunk as [block (4)][term (2)][step of 16 dimensions (4)][lane (64)]
+// BF16 = true: a chunk is 32 dimensions, 16 KB as [block (4)][term (2)][step of 16 dimensions (2)][lane (64)]
 // 8 x bf16 of the points relative to their tile's centre, the query side two terms of -2 q likewise, and the
 // products are those of the kernel above (three v_mfma_f32_32x32x16_bf16 per step); |q - centre|^2 is summed
 // over the chunks from the query side's two terms and the centre's chunk (pack_chunked_centres_kernel), and
@@ -1295,12 +1295,18 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
     u64 *__restrict__ lists = args.lists;
     int *__restrict__ cand = args.cand;
     float *__restrict__ tau = args.tau;
-    const size_t tile_stride = (size_t)n_chunks * kChunkFloat4;  // float4 per packed tile
-    const size_t block_stride = (size_t)n_chunks * kChunkS4 * 64;  // float4 per 32-point block of a tile
+    // Slots of 16 bytes per lane, block and chunk: 8 groups of four k-steps (64 dimensions) on floats; on bf16
+    // terms 2 terms x 2 steps of 16 dimensions (32 dimensions: with 64 the chunk loop's registers did not fit
+    // and the compiler spilled the prefetched chunks the moment they were loaded).
+    constexpr int kSlots = BF16 ? 4 : kChunkS4;
+    constexpr int kSteps16 = 2;                     // bf16: steps of 16 dimensions per chunk
+    constexpr int kChunkF4 = 4 * kSlots * 64;       // float4 per tile chunk
+    const size_t tile_stride = (size_t)n_chunks * kChunkF4;  // float4 per packed tile
+    const size_t block_stride = (size_t)n_chunks * kSlots * 64;  // float4 per 32-point block of a tile
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     v4f *a_lds = reinterpret_cast<v4f *>(lds_raw);
-    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + kChunkFloat4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
-    unsigned int *bitmap = reinterpret_cast<unsigned int *>(reinterpret_cast<u64 *>(a_lds + kChunkFloat4) + 4 * (size_t)cap);
+    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + kChunkF4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
+    unsigned int *bitmap = reinterpret_cast<unsigned int *>(reinterpret_cast<u64 *>(a_lds + kChunkF4) + 4 * (size_t)cap);
     float *qcenter = reinterpret_cast<float *>(bitmap + args.bitmap_words);
     __shared__ u64 thr[kMQ];
     __shared__ int cnt[kMQ];
@@ -1314,15 +1320,17 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
 
     // Chunk c of a candidate tile: global -> registers -> LDS.  Element e = 256 r + tid of the chunk is
     // float4 (e % 512) of block e / 512 = r / 2.
-    v4f stage[kChunkS4];
+    v4f stage[kSlots];
     auto fetch = [&](int tile, int c) {
-        const v4f *src = reinterpret_cast<const v4f *>(args.Xp) + (size_t)tile * tile_stride + (size_t)c * (kChunkS4 * 64) + tid;
+        const v4f *src = reinterpret_cast<const v4f *>(args.Xp) + (size_t)tile * tile_stride + (size_t)c * (kSlots * 64) + tid;
+        // element 256 r + tid of the chunk: block (256 r + tid) / (64 kSlots), float4 (256 r + tid) % (64 kSlots) of it
 #pragma unroll
-        for (int r = 0; r < kChunkS4; ++r) stage[r] = src[(size_t)(r >> 1) * block_stride + (r & 1) * 256];
+        for (int r = 0; r < kSlots; ++r)
+            stage[r] = src[(size_t)((256 * r) / (64 * kSlots)) * block_stride + (256 * r) % (64 * kSlots)];
     };
     auto stash = [&]() {
 #pragma unroll
-        for (int r = 0; r < kChunkS4; ++r) a_lds[r * 256 + tid] = stage[r];
+        for (int r = 0; r < kSlots; ++r) a_lds[r * 256 + tid] = stage[r];
     };
     const int num_ctiles = (N + kCT - 1) / kCT;
 
@@ -1339,9 +1347,9 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
         const float q_len = BF16 && q < N ? sqrtf(args.norms[q]) * (1.0f + 1e-6f) : 0.0f;  // |q|, rounded up
         // This wave's block of the query-side copy.
         const v4f *bsrc = reinterpret_cast<const v4f *>(args.Bp) + (size_t)qt * tile_stride + (size_t)wave * block_stride + lane;
-        v4f bcur[kChunkS4], bnext[kChunkS4];
+        v4f bcur[kSlots], bnext[kSlots];
 #pragma unroll
-        for (int s4 = 0; s4 < kChunkS4; ++s4) bcur[s4] = bsrc[s4 * 64];
+        for (int s4 = 0; s4 < kSlots; ++s4) bcur[s4] = bsrc[s4 * 64];
 
         // One tile: its first chunk is in LDS and the queries' first chunk in bcur on entry; the same holds
         // for next_ct on exit.
@@ -1355,11 +1363,11 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
             float f_part = 0.0f;  // bf16: this lane's share of |q - m|^2 (m: the tile's centre)
             for (int c = 0; c < n_chunks; ++c) {
                 const bool last = c + 1 == n_chunks;
-                v4f mc[kChunkS4];  // bf16: the centre's 32 coordinates that go with this lane's 32 of the chunk
+                v4f mc[2 * kSteps16];  // bf16: the centre's 16 coordinates that go with this lane's 16 of the chunk
                 if constexpr (BF16) {
-                    const v4f *msrc = reinterpret_cast<const v4f *>(args.centres_p) + (size_t)ct * (16 * n_chunks) + 16 * c + 2 * kh;
+                    const v4f *msrc = reinterpret_cast<const v4f *>(args.centres_p) + (size_t)ct * (8 * n_chunks) + 8 * c + 2 * kh;
 #pragma unroll
-                    for (int step = 0; step < 4; ++step) {
+                    for (int step = 0; step < kSteps16; ++step) {
                         mc[2 * step] = msrc[4 * step];
                         mc[2 * step + 1] = msrc[4 * step + 1];
                     }
@@ -1367,20 +1375,20 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                 if (!last) fetch(ct, c + 1);
                 else if (next_ct >= 0) fetch(next_ct, 0);
                 {
-                    const v4f *bn = bsrc + (size_t)(last ? 0 : c + 1) * (kChunkS4 * 64);
+                    const v4f *bn = bsrc + (size_t)(last ? 0 : c + 1) * (kSlots * 64);
 #pragma unroll
-                    for (int s4 = 0; s4 < kChunkS4; ++s4) bnext[s4] = bn[s4 * 64];
+                    for (int s4 = 0; s4 < kSlots; ++s4) bnext[s4] = bn[s4 * 64];
                 }
                 if constexpr (BF16) {
 #pragma unroll
-                    for (int step = 0; step < 4; ++step) {
+                    for (int step = 0; step < kSteps16; ++step) {
                         v4f xh[4], xl[4];
 #pragma unroll
                         for (int b = 0; b < 4; ++b) {
-                            xh[b] = a_lds[(b * kChunkS4 + step) * 64 + lane];
-                            xl[b] = a_lds[(b * kChunkS4 + 4 + step) * 64 + lane];
+                            xh[b] = a_lds[(b * kSlots + step) * 64 + lane];
+                            xl[b] = a_lds[(b * kSlots + kSteps16 + step) * 64 + lane];
                         }
-                        const v8bf qh = __builtin_bit_cast(v8bf, bcur[step]), ql = __builtin_bit_cast(v8bf, bcur[4 + step]);
+                        const v8bf qh = __builtin_bit_cast(v8bf, bcur[step]), ql = __builtin_bit_cast(v8bf, bcur[kSteps16 + step]);
 #pragma unroll
                         for (int b = 0; b < 4; ++b)
                             acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xh[b]), qh, acc[b], 0, 0, 0);
@@ -1391,7 +1399,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                         for (int b = 0; b < 4; ++b)
                             acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, xl[b]), qh, acc[b], 0, 0, 0);
                         // |q - m|^2 from the query's two terms: q_d = -(high + low) / 2 to within 2^-16 |q_d|.
-                        const uint4 uh = __builtin_bit_cast(uint4, bcur[step]), ul = __builtin_bit_cast(uint4, bcur[4 + step]);
+                        const uint4 uh = __builtin_bit_cast(uint4, bcur[step]), ul = __builtin_bit_cast(uint4, bcur[kSteps16 + step]);
                         const unsigned int wh[4] = {uh.x, uh.y, uh.z, uh.w}, wl[4] = {ul.x, ul.y, ul.z, ul.w};
                         const float m[8] = {mc[2 * step][0], mc[2 * step][1], mc[2 * step][2], mc[2 * step][3],
                                             mc[2 * step + 1][0], mc[2 * step + 1][1], mc[2 * step + 1][2], mc[2 * step + 1][3]};
@@ -1422,7 +1430,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                     stash();
                     __syncthreads();
 #pragma unroll
-                    for (int s4 = 0; s4 < kChunkS4; ++s4) bcur[s4] = bnext[s4];
+                    for (int s4 = 0; s4 < kSlots; ++s4) bcur[s4] = bnext[s4];
                 }
             }
             const u64 limit = thr[wave * 32 + qn];
@@ -1500,7 +1508,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                 __syncthreads();
             }
 #pragma unroll
-            for (int s4 = 0; s4 < kChunkS4; ++s4) bcur[s4] = bnext[s4];
+            for (int s4 = 0; s4 < kSlots; ++s4) bcur[s4] = bnext[s4];
         };
 
         // Phase 1: the query tile's neighbourhood; phase 2: the tiles the bitmap keeps.
@@ -1937,15 +1945,15 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     if (mode == 3) mode = 2;
     const bool bf16 = !chunked && !force_f32 && D + 3 <= 128;
     const bool bf16_chunked = chunked && !force_f32;
-    const int n_chunks = chunked ? (bf16_chunked ? div_up(D + 3, 64) : div_up(ksteps, kChunkSteps)) : 0;
-    if (chunked) ksteps = n_chunks * kChunkSteps;
+    const int n_chunks = chunked ? (bf16_chunked ? div_up(D + 3, 32) : div_up(ksteps, kChunkSteps)) : 0;
+    if (chunked) ksteps = n_chunks * (bf16_chunked ? kChunkSteps / 2 : kChunkSteps);  // (slots of 16 bytes per lane x 4)
     else if (ksteps > 32) ksteps = (ksteps + 3) & ~3;
     const int steps16 = div_up(D + 3, 16);
     const int num_tiles = div_up(N, kCT);
     const int bitmap_words = div_up(num_tiles, 32);
     // Room for the candidates kept, as many again and one more tile where the LDS sort buffers of that
     // size fit: a list that is nearly full right after a selection would be selected again after every tile.
-    const size_t tile_lds = chunked ? sizeof(float4) * kChunkFloat4 + sizeof(float) * D
+    const size_t tile_lds = chunked ? sizeof(float4) * (bf16_chunked ? kChunkFloat4 / 2 : kChunkFloat4) + sizeof(float) * D
                                     : sizeof(float4) * (bf16 ? 512 * steps16 + 64 : 4 * ((ksteps + 3) / 4) * 64);
     auto lds_with = [&](int cap) -> size_t {
         return tile_lds + sizeof(u64) * 4 * cap + sizeof(unsigned int) * bitmap_words;
@@ -2025,12 +2033,12 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     }
     DeviceMem centres_p, tile_coef;
     if (bf16_chunked) {
-        if (!centres_p.alloc(sizeof(float) * 64 * (size_t)n_chunks * num_tiles) ||
+        if (!centres_p.alloc(sizeof(float) * 32 * (size_t)n_chunks * num_tiles) ||
             !tile_coef.alloc(sizeof(float) * 2 * (size_t)num_tiles)) {
             set_error("knn: out of device memory for the tile centres");
             return 1;
         }
-        const int64_t pieces = (int64_t)Npad * n_chunks * 16;
+        const int64_t pieces = (int64_t)Npad * n_chunks * 8;
         pack_points_bf16_chunked_kernel<<<div_up(pieces, 256), 256, 0, s>>>(points, centers.as<float>(), N, D, n_chunks,
                                                                            num_tiles, Npad, Xp.as<uint4>(), false);
         TSNE_TRY(hipGetLastError());
