@@ -1276,7 +1276,7 @@ __global__ __launch_bounds__(256, (sweep_occupancy<KSTEPS, BF16>())) void knn_mf
 // all four candidate blocks accumulate over the chunks in 64 registers.  The next chunk of the tile
 // (or the first of the next tile) and of the queries travel through registers meanwhile.  Visiting
 // order, tile skipping, filter, lists and output are those of the kernel above.
-// BF16 = true: a chunk is 32 dimensions, 16 KB as [block (4)][term (2)][step of 16 dimensions (2)][lane (64)]
+// BF16 = true: a chunk is 32 dimensions, 16 KB (two LDS buffers) as [block (4)][term (2)][step of 16 dimensions (2)][lane (64)]
 // 8 x bf16 of the points relative to their tile's centre, the query side two terms of -2 q likewise, and the
 // products are those of the kernel above (three v_mfma_f32_32x32x16_bf16 per step); |q - centre|^2 is summed
 // over the chunks from the query side's two terms and the centre's chunk (pack_chunked_centres_kernel), and
@@ -1301,12 +1301,16 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
     constexpr int kSlots = BF16 ? 4 : kChunkS4;
     constexpr int kSteps16 = 2;                     // bf16: steps of 16 dimensions per chunk
     constexpr int kChunkF4 = 4 * kSlots * 64;       // float4 per tile chunk
+    // bf16: two LDS buffers of 16 KB, so that the next chunk goes to LDS while the other waves may still read the
+    // current one, and one workgroup barrier per chunk does (floats: one buffer of 32 KB, two barriers).
+    constexpr int kBufs = BF16 ? 2 : 1;
+    int buf = 0;  // the buffer that holds the chunk being computed
     const size_t tile_stride = (size_t)n_chunks * kChunkF4;  // float4 per packed tile
     const size_t block_stride = (size_t)n_chunks * kSlots * 64;  // float4 per 32-point block of a tile
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     v4f *a_lds = reinterpret_cast<v4f *>(lds_raw);
-    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + kChunkF4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
-    unsigned int *bitmap = reinterpret_cast<unsigned int *>(reinterpret_cast<u64 *>(a_lds + kChunkF4) + 4 * (size_t)cap);
+    u64 *sortbuf = reinterpret_cast<u64 *>(a_lds + kBufs * kChunkF4) + (size_t)(threadIdx.x >> 6) * cap;  // per wave
+    unsigned int *bitmap = reinterpret_cast<unsigned int *>(reinterpret_cast<u64 *>(a_lds + kBufs * kChunkF4) + 4 * (size_t)cap);
     float *qcenter = reinterpret_cast<float *>(bitmap + args.bitmap_words);
     __shared__ u64 thr[kMQ];
     __shared__ int cnt[kMQ];
@@ -1328,9 +1332,9 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
         for (int r = 0; r < kSlots; ++r)
             stage[r] = src[(size_t)((256 * r) / (64 * kSlots)) * block_stride + (256 * r) % (64 * kSlots)];
     };
-    auto stash = [&]() {
+    auto stash = [&](int b) {
 #pragma unroll
-        for (int r = 0; r < kSlots; ++r) a_lds[r * 256 + tid] = stage[r];
+        for (int r = 0; r < kSlots; ++r) a_lds[b * kChunkF4 + r * 256 + tid] = stage[r];
     };
     const int num_ctiles = (N + kCT - 1) / kCT;
 
@@ -1385,8 +1389,8 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                         v4f xh[4], xl[4];
 #pragma unroll
                         for (int b = 0; b < 4; ++b) {
-                            xh[b] = a_lds[(b * kSlots + step) * 64 + lane];
-                            xl[b] = a_lds[(b * kSlots + kSteps16 + step) * 64 + lane];
+                            xh[b] = a_lds[buf * kChunkF4 + (b * kSlots + step) * 64 + lane];
+                            xl[b] = a_lds[buf * kChunkF4 + (b * kSlots + kSteps16 + step) * 64 + lane];
                         }
                         const v8bf qh = __builtin_bit_cast(v8bf, bcur[step]), ql = __builtin_bit_cast(v8bf, bcur[kSteps16 + step]);
 #pragma unroll
@@ -1426,9 +1430,15 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                     }
                 }
                 if (!last) {
-                    __syncthreads();  // all waves have read this chunk
-                    stash();
-                    __syncthreads();
+                    if constexpr (BF16) {
+                        stash(buf ^ 1);  // (last read a chunk ago, before the barrier that ended that chunk)
+                        __syncthreads();
+                        buf ^= 1;
+                    } else {
+                        __syncthreads();  // all waves have read this chunk
+                        stash(0);
+                        __syncthreads();
+                    }
 #pragma unroll
                     for (int s4 = 0; s4 < kSlots; ++s4) bcur[s4] = bnext[s4];
                 }
@@ -1502,10 +1512,16 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                                 args.select_slack);
                 }
             }
-            __syncthreads();  // all waves are done with the tile's last chunk
-            if (next_ct >= 0) {
-                stash();
-                __syncthreads();
+            if constexpr (BF16) {
+                if (next_ct >= 0) stash(buf ^ 1);
+                __syncthreads();  // the next tile's first chunk is in LDS; all waves are done with this tile's last
+                if (next_ct >= 0) buf ^= 1;
+            } else {
+                __syncthreads();  // all waves are done with the tile's last chunk
+                if (next_ct >= 0) {
+                    stash(0);
+                    __syncthreads();
+                }
             }
 #pragma unroll
             for (int s4 = 0; s4 < kSlots; ++s4) bcur[s4] = bnext[s4];
@@ -1530,7 +1546,8 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
         if (cur > h1) cur = -1;  // fewer tiles than parts: nothing for this part, its lists stay empty
         if (cur >= 0) fetch(cur, 0);
         __syncthreads();  // the previous query tile's last reads of the LDS chunk
-        if (cur >= 0) stash();
+        buf = 0;
+        if (cur >= 0) stash(0);
         __syncthreads();
         bool home = true;
         unsigned int swept = 0;
@@ -1570,7 +1587,7 @@ __global__ __launch_bounds__(256, 2) void knn_mfma_chunked_sweep_kernel(const Sw
                 nxt = next_tile();
                 if (nxt >= 0) {
                     fetch(nxt, 0);
-                    stash();  // the barrier that ended the last tile freed the LDS chunk
+                    stash(buf);  // the barrier that ended the last tile freed the LDS chunks
                     __syncthreads();
                 }
                 __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), as in the kernel above
@@ -1953,7 +1970,7 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     const int bitmap_words = div_up(num_tiles, 32);
     // Room for the candidates kept, as many again and one more tile where the LDS sort buffers of that
     // size fit: a list that is nearly full right after a selection would be selected again after every tile.
-    const size_t tile_lds = chunked ? sizeof(float4) * (bf16_chunked ? kChunkFloat4 / 2 : kChunkFloat4) + sizeof(float) * D
+    const size_t tile_lds = chunked ? sizeof(float4) * kChunkFloat4 + sizeof(float) * D  // (bf16: two chunks of half the size)
                                     : sizeof(float4) * (bf16 ? 512 * steps16 + 64 : 4 * ((ksteps + 3) / 4) * 64);
     auto lds_with = [&](int cap) -> size_t {
         return tile_lds + sizeof(u64) * 4 * cap + sizeof(unsigned int) * bitmap_words;
