@@ -7,8 +7,9 @@ neighbour search (each against all ten million candidates), the normalisation in
 full, sampled rows of the perplexity search and of the symmetrisation, and the
 forces and three fused steps in full.
 
-(The file sorts late on purpose: it is the longest test, and pytest -x stops at
-the first failure.)
+(The GPU test files are numbered in the order pytest collects them: stage parity,
+then the full-size configs, then whole fits, then the surface around the fit; a run
+with -x that stops early has then covered the stages first.)
 """
 import time
 

@@ -239,7 +239,11 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     if (verbose) std::cout << "done.\nInitializing low dim points... " << std::flush;
     std::vector<float> h_emb((size_t)2 * N);
     {
-        std::default_random_engine generator(opt.random_seed);
+        // Options' constructors seed from the clock (src/include/options.h:108-109).  TSNE_RANDOM_SEED, this
+        // library's extension, replaces that seed so that a run through the Python surface or the command-line
+        // program, neither of which can set Options::random_seed, can be repeated.
+        const char *seed_env = std::getenv("TSNE_RANDOM_SEED");
+        std::default_random_engine generator(seed_env && *seed_env ? std::atoi(seed_env) : opt.random_seed);
         std::normal_distribution<float> normal(0.0, 1.0);
         // The reference first draws an unused noise vector; consuming the same
         // draws keeps the generator in step for the random initialisations (the
