@@ -362,7 +362,7 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     (void)hipFree(p->wg_tile_base);
     (void)hipFree(p->chunks);
     (void)hipFree(p->num_chunks);
-    (void)hipFree(p->node_charges);
+    (void)hipFree(p->box_moments);
     (void)hipFree(p->node_potentials);
     (void)hipFree(p->row_spectra);
     (void)hipFree(p->col_results);
@@ -397,6 +397,25 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
     const size_t G2 = (size_t)(kMaxBoxes * kInterp) * (kMaxBoxes * kInterp);
     const size_t spec = (size_t)2 * kFft * kNodePad;
     const size_t N = (size_t)num_points;
+    const size_t moment_bytes = sizeof(unsigned long long) * kMoments * kMaxBoxes * kMaxBoxes;
+    {
+        // Fixed-point scales.  Moments are sums of values in [0, 1], at most N of them in a box, and at most 4096
+        // between two flushes of a workgroup's LDS region, where 2^50 is the most the conversion allows.
+        int log2n = 0;
+        while (((size_t)1 << log2n) < N) ++log2n;
+        p->moment_scale = std::ldexp(1.0, std::min(50, 62 - log2n));
+        // z_i is an interpolated sum of N kernel values in (0, 1]; the interpolation weights sum to one with
+        // magnitudes up to 3.6, so |sum_i z_i| < 4 N^2.
+        p->z_scale = std::ldexp(1.0, std::min(40, 61 - 2 * log2n));
+        // L_m(t) = (t - s_k)(t - s_l) / denom_m in monomials.
+        for (int m = 0; m < kInterp; ++m) {
+            const double sk = p->lagrange.spacing[(m + 1) % kInterp], sl = p->lagrange.spacing[(m + 2) % kInterp];
+            const double d = p->lagrange.denom[m];
+            p->monomials.c[m][0] = sk * sl / d;
+            p->monomials.c[m][1] = -(sk + sl) / d;
+            p->monomials.c[m][2] = 1.0 / d;
+        }
+    }
     p->max_chunks = (int)(N / kChunkPoints) + kMaxTiles + 1;
     {
         int cus = 256;
@@ -417,7 +436,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
               hipMalloc(&p->wg_tile_base, sizeof(int) * (size_t)kSortBlocks * kMaxTiles) == hipSuccess &&
               hipMalloc(&p->chunks, sizeof(int4) * p->max_chunks) == hipSuccess &&
               hipMalloc(&p->num_chunks, 2 * sizeof(int)) == hipSuccess &&
-              hipMalloc(&p->node_charges, sizeof(float4) * G2) == hipSuccess &&
+              hipMalloc(&p->box_moments, moment_bytes) == hipSuccess &&
               hipMalloc(&p->node_potentials, sizeof(float4) * G2) == hipSuccess &&
               hipMalloc(&p->row_spectra, sizeof(float2) * spec) == hipSuccess &&
               hipMalloc(&p->col_results, sizeof(float2) * spec) == hipSuccess &&
@@ -434,7 +453,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
         }
         ok = hipMemcpy(p->twiddles, tw.data(), sizeof(float2) * kFft, hipMemcpyHostToDevice) == hipSuccess &&
              hipMemset(p->yxy, 0, sizeof(float2) * (N + 2)) == hipSuccess &&
-             hipMemset(p->node_charges, 0, sizeof(float4) * G2) == hipSuccess &&
+             hipMemset(p->box_moments, 0, moment_bytes) == hipSuccess &&
              hipMemset(p->tile_count, 0, sizeof(int) * kMaxTiles) == hipSuccess &&
              hipMemset(p->num_chunks, 0, 2 * sizeof(int)) == hipSuccess &&
              hipMemset(p->row_spectra, 0, sizeof(float2) * spec) == hipSuccess &&
@@ -651,8 +670,8 @@ int tsne_hip_plan_set_boxes(tsne_hip_plan *plan, int n_boxes_per_dim) {
     TSNE_REQUIRE(n_boxes_per_dim >= 2 && n_boxes_per_dim <= kMaxBoxes,
                  "plan_set_boxes: n_boxes_per_dim must be in [2, %d] (got %d)", kMaxBoxes, n_boxes_per_dim);
     if (n_boxes_per_dim == plan->n_boxes) return 0;
-    // Nothing of the old grid survives a step: the charges are cleared by the pass that consumes them, every
-    // other grid buffer is written before it is read, and all of them are sized for the largest grid.
+    // Nothing of the old grid survives a step: the box moments are cleared inside the chain that consumed them,
+    // every other grid buffer is written before it is read, and all of them are sized for the largest grid.
     // Captured steps carry the grid size as kernel arguments and launch shapes.
     TSNE_TRY(hipSetDevice(plan->device));
     TSNE_TRY(hipDeviceSynchronize());

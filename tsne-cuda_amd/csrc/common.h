@@ -87,8 +87,10 @@ struct LoopScalars {
     float sumsq;              // scratch for the gradient-norm reduction
     float vmax;               // largest probability of the re-blocked pattern (fixed-point scale)
     // sum_i z_i of the current step in kZParts partial sums (Z = their sum - N): a thousand workgroups each
-    // end with one atomic add, and atomics on a single address are performed one after the other.
-    float z_part[16];
+    // end with one atomic add, and atomics on a single address are performed one after the other.  The sums are
+    // 64-bit fixed point (the plan's z_scale), so that they do not depend on the order in which the workgroups
+    // arrive.
+    long long z_part[16];
     // Workgroups of the re-blocked attractive kernel in which a wave gave up waiting for an LDS counter (their
     // rows come out as NaN).  Never non-zero unless the kernel's roles lose step; the host checks it after a loop.
     unsigned int wait_timeouts;

@@ -26,6 +26,15 @@ struct LagrangeConsts {
     float denom[kInterp];
 };
 
+// Box moments per box: sum over the box's points of u^i v^j, (u, v) the in-box coordinates, for (i <= 4, j <= 2)
+// or (i <= 2, j <= 4).
+constexpr int kMoments = 21;
+// Monomial coefficients of the three Lagrange basis polynomials of a box, L_m(t) = c[m][0] + c[m][1] t + c[m][2] t^2,
+// in double from the fp32 node positions and denominators.
+struct LagrangeMonomials {
+    double c[kInterp][3];
+};
+
 // Kernels of one gradient step, in launch order (profiling slots).
 enum LoopKernel {
     kKernelTileCount = 0,
@@ -66,7 +75,13 @@ struct tsne_hip_plan {
     const float *loop_embedding = nullptr;  // where tsne_hip_iterate last left off: the buffer and the step after its last
     int loop_next_step = -1;
     bool keep_grouping = true;     // loops may carry the grouping by tile from step to step (TSNE_KEEP_GROUPING=0: never)
-    float4 *node_charges = nullptr;     // n_nodes^2, one float4 (4 terms) per node
+    // Box moments of the charge spreading, 64-bit fixed point (scale moment_scale): [x box][moment][y box].  All
+    // zero between steps: the spread kernel adds to them, the forward row pass reads them, the column pass
+    // clears them.  Sized for the largest grid.
+    unsigned long long *box_moments = nullptr;
+    double moment_scale = 0.0;          // 2^s with N 2^s < 2^62: a box can hold every point
+    double z_scale = 0.0;               // fixed-point scale of the partial sums of z (4 N^2 z_scale < 2^63)
+    tsnehip::LagrangeMonomials monomials;
     float4 *node_potentials = nullptr;  // n_nodes^2
     float2 *row_spectra = nullptr;      // 2 plane pairs x kFft x kNodePad (transposed)
     float2 *col_results = nullptr;      // same shape

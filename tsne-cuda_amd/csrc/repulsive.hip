@@ -233,8 +233,11 @@ __global__ __launch_bounds__(256) void bounds_kernel(const float *__restrict__ v
 // kTileBoxes (5 x 5) boxes with a counting sort (count, scan, scatter:
 // positions only, the P matrix keeps its order); then a workgroup takes up to
 // 1024 points of one tile, accumulates their moments per box in a private LDS
-// tile with (integer) LDS atomics, and adds the node sums that follow from the
-// moments to the grid with one global atomic each.
+// tile with (integer) LDS atomics, and adds the box moments to the grid's with
+// one 64-bit integer atomic each.  The forward row pass forms the node sums
+// from the moments.  Every sum between a point and the node charges is an
+// integer sum, so the charges do not depend on how the points were grouped or
+// on the order in which workgroups arrive: two runs give the same bits.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ int box_of(float v, const Bounds &bd, int n_boxes) {
 #pragma clang fp contract(off)
@@ -395,11 +398,15 @@ __global__ __launch_bounds__(1024) void tile_scatter_kernel(const float *__restr
 
 constexpr int kSpreadThreads = 512;  // two points of a 1024-point chunk per thread
 
-// 64-bit fixed-point add of v * scale (|v * scale| < 2^51) to an LDS word.
-__device__ __forceinline__ void add_fixed(unsigned long long *dst, float v, double scale) {
+// v * scale rounded to a 64-bit integer (|v * scale| < 2^51).
+__device__ __forceinline__ unsigned long long to_fixed_bits(float v, double scale) {
     const double magic = 6755399441055744.0;  // 1.5 * 2^52: adding it rounds a double to an integer
     const double r = fma((double)v, scale, magic);
-    atomicAdd(dst, (unsigned long long)(__double_as_longlong(r) - __double_as_longlong(magic)));
+    return (unsigned long long)(__double_as_longlong(r) - __double_as_longlong(magic));
+}
+// 64-bit fixed-point add of v * scale to an LDS (or global) word.
+__device__ __forceinline__ void add_fixed(unsigned long long *dst, float v, double scale) {
+    atomicAdd(dst, to_fixed_bits(v, scale));
 }
 
 // LDS float atomic adds cost ~190 clocks per wave instruction on gfx950 while
@@ -410,7 +417,7 @@ __device__ __forceinline__ void add_fixed(unsigned long long *dst, float v, doub
 // A workgroup takes a contiguous range of the chunk list (the chunks are in tile
 // order): while it spreads one chunk the points of the next are already on their
 // way, consecutive chunks of one tile share the LDS tile, and the tile goes to
-// global memory (float atomics: neighbouring workgroups may hold parts of the same
+// global memory (integer atomics: neighbouring workgroups may hold parts of the same
 // tile) when the tile changes, after kChunksPerFlush chunks (the fixed-point sums
 // have room for 8192 contributions of at most 1) and at the end of the range.
 constexpr int kChunksPerFlush = 4;
@@ -438,15 +445,16 @@ __device__ __forceinline__ float box_lower(int b, const Bounds &bd) {
 // in-box coordinates, is a polynomial in (u, v): the three Lagrange weights are quadratics in their
 // coordinate and x = x_box + w u, y = y_box + w v (w the box width).  So the 36 node sums of a box follow
 // from the 21 moments sum u^i v^j with (i <= 4, j <= 2) or (i <= 2, j <= 4), and a point costs 21 LDS
-// atomics, not 36; the moments lie in [0, 1], so one fixed-point scale (2^50) serves them all and
-// up to 4096 of them sum below 2^62.  The node sums are formed from the moments in fp64 when the tile is
-// flushed, which is exact to fp64 rounding where the per-point products were rounded to fp32.
-constexpr int kMoments = 21;
+// atomics, not 36; the moments lie in [0, 1], so one fixed-point scale (at most 2^50, and small enough
+// for a box that holds every point) serves them all and up to 4096 of them sum below 2^62.  The node sums are
+// formed from the moments of the whole box in fp64 by the forward row pass, which is exact to fp64 rounding
+// where the per-point products were rounded to fp32.
 // The moments of a tile are kept for a region of the tile's 5 x 5 boxes plus a rim of kHalo boxes: when the
 // grouping by tile is carried over from an earlier step, the points of a tile have moved a little, and the region
 // is placed where the tile's points are now (the box of the chunk's first point minus the offset that point had
-// when the grouping was made).  Points that have left even the rim ("strays") add their 36 node contributions
-// with global atomics and are counted; too many of them and the next step groups the points afresh.
+// when the grouping was made).  Points that have left even the rim ("strays") add their 21 moments to the grid's
+// with global atomics - the same integers that the LDS region would have received - and are counted; too many of
+// them and the next step groups the points afresh.
 constexpr int kHalo = 1;
 constexpr int kRegionBoxes = kTileBoxes + 2 * kHalo;
 constexpr int kRegionBoxes2 = kRegionBoxes * kRegionBoxes;
@@ -461,13 +469,13 @@ __global__ __launch_bounds__(kSpreadThreads, 4) void spread_kernel(const float2 
                                                      const int *__restrict__ tile_perm,
                                                      const float2 *__restrict__ yxy, int4 *chunks,
                                                      const int *__restrict__ num_chunks, LoopScalars *sc,
-                                                     int slot, int next_slot, int n_boxes, LagrangeConsts lc,
-                                                     float *__restrict__ w, int keep_grouping) {
+                                                     int slot, int next_slot, int n_boxes, double to_fixed,
+                                                     unsigned long long *__restrict__ moments, int keep_grouping) {
     __shared__ unsigned long long acc[kMoments * kRegionBoxes2];  // one plane per moment
     __shared__ int origin[2];
     // The step's resets: the partial sums of z (the gather kernel at the chain's end adds to them) and the
     // bounds slot the coming update will fill.
-    if (blockIdx.x == 0 && threadIdx.x < kZParts) sc->z_part[threadIdx.x] = 0.0f;
+    if (blockIdx.x == 0 && threadIdx.x < kZParts) sc->z_part[threadIdx.x] = 0ll;
     if (blockIdx.x == 0 && threadIdx.x == 0 && next_slot >= 0) {
         sc->min_enc[next_slot] = 0xffffffffu;
         sc->max_enc[next_slot] = 0u;
@@ -485,18 +493,7 @@ __global__ __launch_bounds__(kSpreadThreads, 4) void spread_kernel(const float2 
     const int tid = threadIdx.x;
     for (int e = tid; e < kMoments * kRegionBoxes2; e += kSpreadThreads) acc[e] = 0ull;
     const int tiles_per_dim = (n_boxes + kTileBoxes - 1) / kTileBoxes;
-    const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    const double to_fixed = 1125899906842624.0, from_fixed = 1.0 / 1125899906842624.0;  // 2^50
-    // Monomial coefficients of the Lagrange weights: L_m(t) = (t - s_k)(t - s_l) / denom_m.
-    double coef[kInterp][3];
-#pragma unroll
-    for (int m = 0; m < kInterp; ++m) {
-        const double sk = lc.spacing[(m + 1) % kInterp], sl = lc.spacing[(m + 2) % kInterp], d = lc.denom[m];
-        coef[m][0] = sk * sl / d;
-        coef[m][1] = -(sk + sl) / d;
-        coef[m][2] = 1.0 / d;
-    }
     // Unconditional, clamped loads: a chunk holds at least one point.  With a grouping carried over, the
     // positions are the current ones of the points the grouping lists (the interleaved copy the update keeps):
     // a chunk's list of points is fetched two chunks ahead, its positions one chunk ahead, so that neither load
@@ -586,12 +583,12 @@ __global__ __launch_bounds__(kSpreadThreads, 4) void spread_kernel(const float2 
                 pu[1] = pcu[u];
                 pv[1] = pcv[u];
                 const int lx = bx - ox0, ly = by - oy0;
-                if ((unsigned int)lx < (unsigned int)kRegionBoxes && (unsigned int)ly < (unsigned int)kRegionBoxes) {
 #pragma unroll
-                    for (int k = 2; k < 5; ++k) {
-                        pu[k] = pu[k - 1] * pu[1];
-                        pv[k] = pv[k - 1] * pv[1];
-                    }
+                for (int k = 2; k < 5; ++k) {
+                    pu[k] = pu[k - 1] * pu[1];
+                    pv[k] = pv[k - 1] * pv[1];
+                }
+                if ((unsigned int)lx < (unsigned int)kRegionBoxes && (unsigned int)ly < (unsigned int)kRegionBoxes) {
                     unsigned long long *dst = acc + lx * kRegionBoxes + ly;
 #pragma unroll
                     for (int j = 0; j < 5; ++j)
@@ -600,26 +597,15 @@ __global__ __launch_bounds__(kSpreadThreads, 4) void spread_kernel(const float2 
                             if (j <= 2 || i <= 2)
                                 add_fixed(dst + moment_index(i, j) * kRegionBoxes2, pu[i] * pv[j], to_fixed);
                 } else {
-                    // A stray: its nine nodes directly (src/kernels/nbodyfft.cu:107-139).
+                    // A stray: the same 21 integers, straight to the grid's moments.
                     stray = true;
-                    const float x = pt[u].x, y = pt[u].y;
-                    float Lx[kInterp], Ly[kInterp];
+                    unsigned long long *dst = moments + (size_t)bx * kMoments * n_boxes + by;
 #pragma unroll
-                    for (int m = 0; m < kInterp; ++m) {
-                        Lx[m] = (float)(coef[m][0] + (coef[m][1] + coef[m][2] * pu[1]) * pu[1]);
-                        Ly[m] = (float)(coef[m][0] + (coef[m][1] + coef[m][2] * pv[1]) * pv[1]);
-                    }
+                    for (int j = 0; j < 5; ++j)
 #pragma unroll
-                    for (int a = 0; a < kInterp; ++a)
-#pragma unroll
-                        for (int b = 0; b < kInterp; ++b) {
-                            const float lw = Lx[a] * Ly[b];
-                            float *out = w + ((size_t)(bx * kInterp + a) * G + (by * kInterp + b)) * kTerms;
-                            atomicAdd(out + 0, lw);
-                            atomicAdd(out + 1, lw * x);
-                            atomicAdd(out + 2, lw * y);
-                            atomicAdd(out + 3, lw * (x * x + y * y));
-                        }
+                        for (int i = 0; i < 5; ++i)
+                            if (j <= 2 || i <= 2)
+                                add_fixed(dst + (size_t)moment_index(i, j) * n_boxes, pu[i] * pv[j], to_fixed);
                 }
             }
             strays += stray ? 1u : 0u;
@@ -627,40 +613,18 @@ __global__ __launch_bounds__(kSpreadThreads, 4) void spread_kernel(const float2 
         ++in_tile;
         if (last || next_ch.x != cur_tile || in_tile == kChunksPerFlush) {
             __syncthreads();
-            // One thread per (box, node of the box): five sums over the nine monomial pairs, then the four terms.
-            for (int e = tid; e < kRegionBoxes2 * kInterp * kInterp; e += kSpreadThreads) {
-                const int box = e / (kInterp * kInterp), a = (e / kInterp) % kInterp, b = e % kInterp;
-                const unsigned long long *src = acc + box;
-                if (src[0] == 0ull) continue;  // moment (0, 0) is the number of points in the box
+            // The region's moments to the grid's, and the region back to zero.  Neighbouring lanes take neighbouring
+            // boxes of one moment (no two lanes on one LDS bank, runs of seven neighbouring words in memory).
+            for (int e = tid; e < kMoments * kRegionBoxes2; e += kSpreadThreads) {
+                const unsigned long long v = acc[e];
+                if (v == 0ull) continue;
+                acc[e] = 0ull;
+                const int m = e / kRegionBoxes2, box = e % kRegionBoxes2;
                 const int bxg = ox0 + box / kRegionBoxes, byg = oy0 + box % kRegionBoxes;
-                const int gx = bxg * kInterp + a, gy = byg * kInterp + b;
-                if (gx < 0 || gy < 0 || gx >= G || gy >= G) continue;  // (boxes with points lie inside the grid)
-                double M[kMoments];
-#pragma unroll
-                for (int m = 0; m < kMoments; ++m) M[m] = (double)(long long)src[m * kRegionBoxes2] * from_fixed;
-                double s00 = 0.0, s10 = 0.0, s01 = 0.0, s20 = 0.0, s02 = 0.0;
-#pragma unroll
-                for (int i = 0; i < 3; ++i)
-#pragma unroll
-                    for (int j = 0; j < 3; ++j) {
-                        const double cc = coef[a][i] * coef[b][j];
-                        s00 += cc * M[moment_index(i, j)];
-                        s10 += cc * M[moment_index(i + 1, j)];
-                        s01 += cc * M[moment_index(i, j + 1)];
-                        s20 += cc * M[moment_index(i + 2, j)];
-                        s02 += cc * M[moment_index(i, j + 2)];
-                    }
-                const double bw = bd.box_width;
-                const double xl = box_lower(bxg, bd), yl = box_lower(byg, bd);
-                float *out = w + ((size_t)gx * G + gy) * kTerms;
-                atomicAdd(out + 0, (float)s00);
-                atomicAdd(out + 1, (float)(xl * s00 + bw * s10));
-                atomicAdd(out + 2, (float)(yl * s00 + bw * s01));
-                atomicAdd(out + 3, (float)((xl * xl + yl * yl) * s00 + 2.0 * bw * (xl * s10 + yl * s01) +
-                                           bw * bw * (s20 + s02)));
+                // (boxes with points lie inside the grid)
+                if ((unsigned int)bxg < (unsigned int)n_boxes && (unsigned int)byg < (unsigned int)n_boxes)
+                    atomicAdd(moments + ((size_t)bxg * kMoments + m) * n_boxes + byg, v);
             }
-            __syncthreads();
-            for (int e = tid; e < kMoments * kRegionBoxes2; e += kSpreadThreads) acc[e] = 0ull;
             // (the barrier of the next run's start, or the kernel's end, follows)
             cur_tile = next_ch.x;
             in_tile = 0;
@@ -735,8 +699,11 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
 }
 
 // ---------------------------------------------------------------------------
-// Row pass: transforms ROWS grid rows (x nodes m0 ...), both plane pairs, along the y-node axis; clears the
-// charges it consumed so that the next step starts from zero without a memset.  Output is transposed:
+// Row pass: transforms ROWS grid rows (x nodes m0 ...), both plane pairs, along the y-node axis.  The charges
+// of a node, w[node][t] = sum over the points of its box of L_a(u) L_b(v) q_t, are formed here from the box's
+// moments: with L_a(u) = sum_i ca_i u^i, L_b(v) = sum_j cb_j v^j, x = x_box + w u and y = y_box + w v (w the box
+// width), the four terms are combinations of the five sums s_kl = sum_ij ca_i cb_j M(i + k, j + l),
+// (k, l) = (0,0), (1,0), (0,1), (2,0), (0,2), taken in fp64.  Output is transposed:
 // row_spectra[pair][pos][m], pos = digit-reversed frequency position.
 //
 // Two rows per workgroup (512 threads, 32 KB of LDS) is what the loop uses: one such workgroup fits into the 34 KB
@@ -745,8 +712,10 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
 // workgroup (256 threads, 16 KB) measured 21 us against 17 us alone and 2 % fewer iterations per second.
 // ---------------------------------------------------------------------------
 template <int ROWS>
-__global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *__restrict__ w, int G, int n_boxes,
-                                                                       const LoopScalars *sc, int slot,
+__global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(const unsigned long long *__restrict__ moments,
+                                                                       double from_fixed, LagrangeMonomials mono,
+                                                                       float4 *__restrict__ charges_out, int G,
+                                                                       int n_boxes, const LoopScalars *sc, int slot,
                                                                        const float2 *__restrict__ twiddles,
                                                                        float2 *__restrict__ row_spectra,
                                                                        float *__restrict__ kernel_rows) {
@@ -766,13 +735,44 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(float4 *_
     if (row_block < 0) return;
     const int m0 = row_block * ROWS;
     const float s3 = r2_plane_scale(sc, slot);
+    const Bounds bd = load_bounds(sc, slot, n_boxes);
     for (int e = tid; e < ROWS * kFft; e += kThreads) {
         const int r = e >> kLog2Fft, n = e & (kFft - 1);
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (n < G && m0 + r < G) {
-            float4 *src = w + (size_t)(m0 + r) * G + n;
-            v = *src;
-            *src = make_float4(0.f, 0.f, 0.f, 0.f);
+            const int gx = m0 + r;
+            const int bx = gx / kInterp, a = gx % kInterp, by = n / kInterp, b = n % kInterp;
+            const unsigned long long *src = moments + (size_t)bx * kMoments * n_boxes + by;
+            if (src[0] != 0ull) {  // moment (0, 0) counts the points of the box
+                double M[kMoments];
+#pragma unroll
+                for (int m = 0; m < kMoments; ++m) M[m] = (double)(long long)src[(size_t)m * n_boxes] * from_fixed;
+                double ca[3], cb[3];
+#pragma unroll
+                for (int i = 0; i < 3; ++i) {
+                    ca[i] = a == 0 ? mono.c[0][i] : (a == 1 ? mono.c[1][i] : mono.c[2][i]);
+                    cb[i] = b == 0 ? mono.c[0][i] : (b == 1 ? mono.c[1][i] : mono.c[2][i]);
+                }
+                double s00 = 0.0, s10 = 0.0, s01 = 0.0, s20 = 0.0, s02 = 0.0;
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+#pragma unroll
+                    for (int j = 0; j < 3; ++j) {
+                        const double cc = ca[i] * cb[j];
+                        s00 += cc * M[moment_index(i, j)];
+                        s10 += cc * M[moment_index(i + 1, j)];
+                        s01 += cc * M[moment_index(i, j + 1)];
+                        s20 += cc * M[moment_index(i + 2, j)];
+                        s02 += cc * M[moment_index(i, j + 2)];
+                    }
+                const double bw = bd.box_width;
+                const double xl = box_lower(bx, bd), yl = box_lower(by, bd);
+                v.x = (float)s00;
+                v.y = (float)(xl * s00 + bw * s10);
+                v.z = (float)(yl * s00 + bw * s01);
+                v.w = (float)((xl * xl + yl * yl) * s00 + 2.0 * bw * (xl * s10 + yl * s01) + bw * bw * (s20 + s02));
+            }
+            if (charges_out) charges_out[(size_t)gx * G + n] = v;
         }
         s[r * 2 + 0][pad(n)] = make_float2(v.x, v.w * s3);  // planes 1 and r^2 / m^2
         s[r * 2 + 1][pad(n)] = make_float2(v.y, v.z);       // planes x and y
@@ -809,7 +809,11 @@ template <bool SLIM>
 __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restrict__ row_spectra, int G,
                                                            const float *__restrict__ kernel_rows,
                                                            const float2 *__restrict__ twiddles,
-                                                           float2 *__restrict__ col_results) {
+                                                           float2 *__restrict__ col_results,
+                                                           unsigned long long *__restrict__ moments,
+                                                           int moment_words) {
+    // The forward row pass has consumed the box moments: back to zero for the next step's spread.
+    for (int e = blockIdx.x * 512 + threadIdx.x; e < moment_words; e += gridDim.x * 512) moments[e] = 0ull;
     // Layout: [pair in flight][col], then (SLIM = false) the kernel columns; every transform swizzled, see pad().
     constexpr int kPairsInFlight = 2;
     constexpr int kData = 2 * kPairsInFlight;  // transforms of data per round
@@ -917,7 +921,7 @@ __global__ __launch_bounds__(256) void gather_forces_kernel(const float *__restr
                                                             LagrangeConsts lc,
                                                             const float4 *__restrict__ node_potentials,
                                                             float *__restrict__ rep, float *__restrict__ phi_out,
-                                                            LoopScalars *sc, int keep_grouping) {
+                                                            LoopScalars *sc, int keep_grouping, double z_scale) {
     __shared__ float partial[256 / kWave];
     // Last kernel of the chain: whether the next step keeps this step's grouping of the points by tile.  (The
     // spread kernel has finished counting; the chain's kernels of this step have all read the flag.)
@@ -968,22 +972,24 @@ __global__ __launch_bounds__(256) void gather_forces_kernel(const float *__restr
         float t = 0.0f;
 #pragma unroll
         for (int k = 0; k < 256 / kWave; ++k) t += partial[k];
-        atomicAdd(&sc->z_part[blockIdx.x % kZParts], t);
+        // (a workgroup's own sum is taken in a fixed order; the sums over workgroups are integer sums)
+        atomicAdd(reinterpret_cast<unsigned long long *>(&sc->z_part[blockIdx.x % kZParts]),
+                  (unsigned long long)__double2ll_rn((double)t * z_scale));
     }
 }
 
-__global__ void finish_z_kernel(const LoopScalars *sc, int N, float *out) {
+__global__ void finish_z_kernel(const LoopScalars *sc, int N, double z_inv_scale, float *out) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
-        float z = 0.0f;
+        long long z = 0ll;
         for (int k = 0; k < kZParts; ++k) z += sc->z_part[k];
-        *out = z - (float)N;  // src/kernels/rep_forces.cu:54
+        *out = (float)((double)z * z_inv_scale) - (float)N;  // src/kernels/rep_forces.cu:54
     }
 }
 
 }  // namespace
 
 int launch_finish_z(tsne_hip_plan *p, float *normalization, hipStream_t s) {
-    finish_z_kernel<<<1, 64, 0, s>>>(p->scalars, p->num_points, normalization);
+    finish_z_kernel<<<1, 64, 0, s>>>(p->scalars, p->num_points, 1.0 / p->z_scale, normalization);
     TSNE_LAUNCHED(s);
     return 0;
 }
@@ -1033,23 +1039,23 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     const int spread_blocks =
         xcd_launch_blocks(std::min(N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1, p->spread_grid));
     spread_kernel<<<spread_blocks, kSpreadThreads, 0, s>>>(p->tile_xy, p->tile_perm, p->yxy, p->chunks,
-                                                           p->num_chunks, p->scalars, slot, slot ^ 1, nb, p->lagrange,
-                                                           reinterpret_cast<float *>(p->node_charges), keep);
+                                                           p->num_chunks, p->scalars, slot, slot ^ 1, nb,
+                                                           p->moment_scale, p->box_moments, keep);
     TSNE_LAUNCHED(s);
-    if (charges_out)
-        TSNE_TRY(hipMemcpyAsync(charges_out, p->node_charges, sizeof(float4) * (size_t)G * G,
-                                hipMemcpyDeviceToDevice, s));
     if (profile_mark(p, kKernelConvRowsForward, s)) return 1;
-    conv_rows_forward_kernel<2><<<xcd_launch_blocks(div_up(G, 2)) + div_up(G, 8), 512, 0, s>>>(p->node_charges, G, nb, p->scalars, slot,
-                                                                            p->twiddles, p->row_spectra, p->kernel_rows);
+    conv_rows_forward_kernel<2><<<xcd_launch_blocks(div_up(G, 2)) + div_up(G, 8), 512, 0, s>>>(
+        p->box_moments, 1.0 / p->moment_scale, p->monomials, reinterpret_cast<float4 *>(charges_out), G, nb, p->scalars,
+        slot, p->twiddles, p->row_spectra, p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
     static const int slim_mode = getenv("TSNE_SLIM_COLUMNS") ? atoi(getenv("TSNE_SLIM_COLUMNS")) : -1;
     const bool slim = slim_mode < 0 ? (p->blocked_ready && p->strip_rows >= 1024) : slim_mode == 1;
     if (slim)
-        conv_columns_kernel<true><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
+        conv_columns_kernel<true><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results,
+                                                           p->box_moments, kMoments * nb * nb);
     else
-        conv_columns_kernel<false><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results);
+        conv_columns_kernel<false><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results,
+                                                            p->box_moments, kMoments * nb * nb);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvRowsInverse, s)) return 1;
     conv_rows_inverse_kernel<<<xcd_launch_blocks(div_up(G, 2)), kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
@@ -1057,7 +1063,8 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelGather, s)) return 1;
     gather_forces_kernel<<<std::min(div_up(N, 256), 1024), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
-                                                        p->node_potentials, rep, point_potentials, p->scalars, keep);
+                                                        p->node_potentials, rep, point_potentials, p->scalars, keep,
+                                                        p->z_scale);
     TSNE_LAUNCHED(s);
     return 0;
 }

@@ -85,17 +85,25 @@ __global__ void centre_reset_kernel(LoopScalars *sc, int slot) {
     if (threadIdx.x == 0 && blockIdx.x == 0) sc->center_sum[slot][0] = sc->center_sum[slot][1] = 0.0;
 }
 
+// Z of the step: the caller's scalar, or (z_ptr null) the loop's own - the fixed-point partial sums of z_i,
+// an integer sum, less N (src/kernels/rep_forces.cu:54).
+__device__ __forceinline__ float load_normalization(const float *z_ptr, const LoopScalars *sc, double z_inv_scale,
+                                                    int N) {
+    if (z_ptr) return *z_ptr;
+    long long z = 0ll;
+    for (int k = 0; k < kZParts; ++k) z += sc->z_part[k];
+    return (float)((double)z * z_inv_scale) - (float)N;
+}
+
 template <bool FUSED>
 __global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, float *__restrict__ attr,
                                                      float *__restrict__ rep, float *__restrict__ gains,
                                                      float *__restrict__ old, int N, float eta,
-                                                     const float *__restrict__ z_ptr, int z_count, float z_offset,
+                                                     const float *__restrict__ z_ptr, double z_inv_scale,
                                                      float momentum,
                                                      float exaggeration, float2 *__restrict__ yxy, LoopScalars *sc,
                                                      int next_slot, int recenter) {
-    float z_total = 0.0f;
-    for (int k = 0; k < z_count; ++k) z_total += z_ptr[k];  // same order in every thread
-    const float normalization = z_total - z_offset;
+    const float normalization = load_normalization(z_ptr, sc, z_inv_scale, N);
     float lo = INFINITY, hi = -INFINITY;
     const Centre c = load_centre<FUSED>(sc, next_slot, N, recenter);
     float sx = 0.0f, sy = 0.0f;
@@ -152,14 +160,11 @@ template <bool FUSED>
 __global__ __launch_bounds__(256) void update_vec4_kernel(float *__restrict__ emb, float *__restrict__ attr,
                                                           float *__restrict__ rep, float *__restrict__ gains,
                                                           float *__restrict__ old, int N, float eta,
-                                                          const float *__restrict__ z_ptr, int z_count,
-                                                          float z_offset,
+                                                          const float *__restrict__ z_ptr, double z_inv_scale,
                                                           float momentum, float exaggeration,
                                                           float2 *__restrict__ yxy, LoopScalars *sc, int next_slot,
                                                           int recenter) {
-    float z_total = 0.0f;
-    for (int k = 0; k < z_count; ++k) z_total += z_ptr[k];  // same order in every thread
-    const float normalization = z_total - z_offset;
+    const float normalization = load_normalization(z_ptr, sc, z_inv_scale, N);
     float lo = INFINITY, hi = -INFINITY;
     const Centre c = load_centre<FUSED>(sc, next_slot, N, recenter);
     float sx = 0.0f, sy = 0.0f;
@@ -258,9 +263,8 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
                   float eta, const float *normalization, float momentum, float exaggeration, int next_slot,
                   hipStream_t s) {
     const int N = p->num_points;
-    const float *z_ptr = normalization ? normalization : p->scalars->z_part;
-    const int z_count = normalization ? 1 : kZParts;
-    const float z_offset = normalization ? 0.0f : (float)N;
+    const float *z_ptr = normalization;
+    const double z_inv = 1.0 / p->z_scale;
     if (profile_mark(p, kKernelUpdate, s)) return 1;
     auto aligned16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     if (N % 4 == 0 && aligned16(embedding) && aligned16(attr) && aligned16(rep) && aligned16(gains) &&
@@ -270,23 +274,23 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
         // 512 25 us, one item per thread (977 workgroups) 39 us.
         const int blocks = std::min(div_up(N / 4, 256), p->stream_grid);
         if (next_slot >= 0) {
-            update_vec4_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count,
-                                                            z_offset, momentum, exaggeration, p->yxy, p->scalars,
+            update_vec4_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
+                                                            momentum, exaggeration, p->yxy, p->scalars,
                                                             next_slot, p->recenter ? 1 : 0);
         } else {
-            update_vec4_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count,
-                                                             z_offset, momentum, exaggeration, nullptr, nullptr, 0, 0);
+            update_vec4_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
+                                                             momentum, exaggeration, nullptr, p->scalars, 0, 0);
         }
         TSNE_LAUNCHED(s);
         return 0;
     }
     const int blocks = std::min(div_up(N, 256), 4 * p->stream_grid);  // 4-byte accesses: the same window
     if (next_slot >= 0) {
-        update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count, z_offset,
+        update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
                                                    momentum, exaggeration, p->yxy, p->scalars, next_slot, p->recenter ? 1 : 0);
     } else {
-        update_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_count, z_offset,
-                                                    momentum, exaggeration, nullptr, nullptr, 0, 0);
+        update_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
+                                                    momentum, exaggeration, nullptr, p->scalars, 0, 0);
     }
     TSNE_LAUNCHED(s);
     return 0;
