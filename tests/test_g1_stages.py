@@ -333,6 +333,11 @@ def test_iterate_with_recentring(stages, c0_problem, prepared):
     assert abs(float(z.item()) - z_o) <= 1e-4 * abs(z_o)
     extent = float(y.max() - y.min())
     assert abs(y[:n].mean()) <= 1e-2 * extent and abs(y[n:].mean()) <= 1e-2 * extent
+    # the centre is a sum over workgroups taken in a fixed order: a second run ends on the same bits
+    dy2 = dev(y0)
+    gains2, old2 = torch.ones_like(dy2), torch.zeros_like(dy2)
+    plan.iterate_(None if prepared else dP, None if prepared else di, dy2, gains2, old2, 0, 6)
+    assert same_bits(dy2.cpu().numpy(), y)
     # the same start without the option keeps its offset (and follows the oracle's plain loop)
     plan.set_recenter(False)
     dy = dev(y0)

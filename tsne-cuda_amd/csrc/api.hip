@@ -363,6 +363,7 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     (void)hipFree(p->chunks);
     (void)hipFree(p->num_chunks);
     (void)hipFree(p->box_moments);
+    (void)hipFree(p->centre_parts);
     (void)hipFree(p->node_potentials);
     (void)hipFree(p->row_spectra);
     (void)hipFree(p->col_results);
@@ -437,6 +438,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
               hipMalloc(&p->chunks, sizeof(int4) * p->max_chunks) == hipSuccess &&
               hipMalloc(&p->num_chunks, 2 * sizeof(int)) == hipSuccess &&
               hipMalloc(&p->box_moments, moment_bytes) == hipSuccess &&
+              hipMalloc(&p->centre_parts, sizeof(double2) * 2 * kMaxCentreParts) == hipSuccess &&
               hipMalloc(&p->node_potentials, sizeof(float4) * G2) == hipSuccess &&
               hipMalloc(&p->row_spectra, sizeof(float2) * spec) == hipSuccess &&
               hipMalloc(&p->col_results, sizeof(float2) * spec) == hipSuccess &&
@@ -454,6 +456,7 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
         ok = hipMemcpy(p->twiddles, tw.data(), sizeof(float2) * kFft, hipMemcpyHostToDevice) == hipSuccess &&
              hipMemset(p->yxy, 0, sizeof(float2) * (N + 2)) == hipSuccess &&
              hipMemset(p->box_moments, 0, moment_bytes) == hipSuccess &&
+             hipMemset(p->centre_parts, 0, sizeof(double2) * 2 * kMaxCentreParts) == hipSuccess &&
              hipMemset(p->tile_count, 0, sizeof(int) * kMaxTiles) == hipSuccess &&
              hipMemset(p->num_chunks, 0, 2 * sizeof(int)) == hipSuccess &&
              hipMemset(p->row_spectra, 0, sizeof(float2) * spec) == hipSuccess &&

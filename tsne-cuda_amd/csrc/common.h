@@ -103,11 +103,13 @@ struct LoopScalars {
     int reuse_sort;
     // Running totals since the plan was made: chain evaluations, those that grouped the points afresh, strays.
     unsigned int chain_runs, chain_sorts, strays_total;
-    // Optional re-centring (off unless the plan asks for it): per bounds slot, the sums of the x and of the y
-    // coordinates of the embedding that slot's bounds describe.
-    double center_sum[2][2];
+    // Optional re-centring (off unless the plan asks for it): per bounds slot, how many workgroups left their
+    // sums of the x and of the y coordinates of the embedding that slot's bounds describe (in the plan's
+    // centre_parts; the reader adds them in a fixed order).
+    int center_count[2];
 };
 constexpr int kZParts = 16;
+constexpr int kMaxCentreParts = 2048;  // most workgroups of a kernel that leaves coordinate sums
 
 }  // namespace tsnehip
 

@@ -105,6 +105,7 @@ struct tsne_hip_plan {
     const int *csr_row_ptr = nullptr, *csr_col_idx = nullptr;
     const float *csr_values = nullptr;
     bool recenter = false;          // the loop's updates re-centre the embedding (tsne_hip_plan_set_recenter)
+    double2 *centre_parts = nullptr;  // 2 bounds slots x kMaxCentreParts: coordinate sums per workgroup
 
     // The repulsive chain and the attractive kernel of a step are independent: the fused loop runs
     // the chain on this side stream (default priority) and joins before the update.

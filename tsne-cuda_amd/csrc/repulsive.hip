@@ -479,8 +479,6 @@ __global__ __launch_bounds__(kSpreadThreads, 4) void spread_kernel(const float2 
     if (blockIdx.x == 0 && threadIdx.x == 0 && next_slot >= 0) {
         sc->min_enc[next_slot] = 0xffffffffu;
         sc->max_enc[next_slot] = 0u;
-        sc->center_sum[next_slot][0] = 0.0;
-        sc->center_sum[next_slot][1] = 0.0;
     }
     const int nc = *num_chunks;
     // Neighbouring stretches of the chunk list (tiles next to each other) go to workgroups of one XCD: the

@@ -41,48 +41,74 @@ __device__ __forceinline__ float step_coordinate(float &gain, float &u, float at
 
 // Re-centring (optional, no counterpart in the reference, whose loop never re-centres:
 // src/kernels/apply_forces.cu:11-57): the update subtracts from every new position the centre of the embedding
-// as it stood before the step (its coordinate sums were accumulated by the update before, or by
-// centre_sums_kernel at the start of a loop) and accumulates the sums of what it writes.  All forces are
-// translation invariant, so the trajectory is that of exact re-centring after every step, one step late.
-// Without the option the centre reads as (+0, +0) and x - 0 is x, bit for bit.
+// as it stood before the step (its coordinate sums were left by the update before, or by centre_sums_kernel at
+// the start of a loop) and leaves the sums of what it writes.  All forces are translation invariant, so the
+// trajectory is that of exact re-centring after every step, one step late.  Without the option the centre reads
+// as (+0, +0) and x - 0 is x, bit for bit.
+// Every workgroup leaves its own pair of sums; the reader adds the pairs in the order of the workgroups, so the
+// centre does not depend on the order in which they finished.
 struct Centre {
     float x, y;
 };
 template <bool FUSED>
-__device__ __forceinline__ Centre load_centre(const LoopScalars *sc, int next_slot, int N, int recenter) {
+__device__ __forceinline__ Centre load_centre(const LoopScalars *sc, const double2 *parts, int next_slot, int N,
+                                              int recenter) {
     Centre c{0.0f, 0.0f};
     if (FUSED && recenter) {
-        c.x = (float)(sc->center_sum[next_slot ^ 1][0] / (double)N);
-        c.y = (float)(sc->center_sum[next_slot ^ 1][1] / (double)N);
+        __shared__ double2 tree[256];
+        const int slot = next_slot ^ 1;
+        const int count = sc->center_count[slot];
+        double2 acc = make_double2(0.0, 0.0);
+        for (int k = threadIdx.x; k < count; k += 256) {
+            const double2 v = parts[(size_t)slot * kMaxCentreParts + k];
+            acc.x += v.x;
+            acc.y += v.y;
+        }
+        tree[threadIdx.x] = acc;
+        __syncthreads();
+        for (int half = 128; half >= 1; half >>= 1) {
+            if ((int)threadIdx.x < half) {
+                tree[threadIdx.x].x += tree[threadIdx.x + half].x;
+                tree[threadIdx.x].y += tree[threadIdx.x + half].y;
+            }
+            __syncthreads();
+        }
+        c.x = (float)(tree[0].x / (double)N);
+        c.y = (float)(tree[0].y / (double)N);
     }
     return c;
 }
-// A thread's sums of the x and y coordinates it wrote into the next slot's sums: one pair of atomics per wave.
-__device__ __forceinline__ void publish_centre(LoopScalars *sc, int next_slot, float sx, float sy) {
+// A workgroup's sums of the x and y coordinates it wrote, into its place among the next slot's parts
+// (256 threads; every thread of the workgroup calls this).
+__device__ __forceinline__ void publish_centre(LoopScalars *sc, double2 *parts, int next_slot, float sx, float sy) {
+    __shared__ double2 wave_sum[256 / kWave];
     double dx = (double)sx, dy = (double)sy;
 #pragma unroll
     for (int m = kWave / 2; m > 0; m >>= 1) {
         dx += __shfl_xor(dx, m, kWave);
         dy += __shfl_xor(dy, m, kWave);
     }
-    if ((threadIdx.x & (kWave - 1)) == 0) {
-        atomicAdd(&sc->center_sum[next_slot][0], dx);
-        atomicAdd(&sc->center_sum[next_slot][1], dy);
+    if ((threadIdx.x & (kWave - 1)) == 0) wave_sum[threadIdx.x / kWave] = make_double2(dx, dy);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double2 t = wave_sum[0];
+        for (int k = 1; k < 256 / kWave; ++k) {
+            t.x += wave_sum[k].x;
+            t.y += wave_sum[k].y;
+        }
+        parts[(size_t)next_slot * kMaxCentreParts + blockIdx.x] = t;
+        if (blockIdx.x == 0) sc->center_count[next_slot] = (int)gridDim.x;
     }
 }
 
 __global__ __launch_bounds__(256) void centre_sums_kernel(const float *__restrict__ emb, int N, LoopScalars *sc,
-                                                          int slot) {
+                                                          double2 *parts, int slot) {
     float sx = 0.0f, sy = 0.0f;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
         sx += emb[i];
         sy += emb[N + i];
     }
-    publish_centre(sc, slot, sx, sy);
-}
-
-__global__ void centre_reset_kernel(LoopScalars *sc, int slot) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) sc->center_sum[slot][0] = sc->center_sum[slot][1] = 0.0;
+    publish_centre(sc, parts, slot, sx, sy);
 }
 
 // Z of the step: the caller's scalar, or (z_ptr null) the loop's own - the fixed-point partial sums of z_i,
@@ -102,10 +128,10 @@ __global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, fl
                                                      const float *__restrict__ z_ptr, double z_inv_scale,
                                                      float momentum,
                                                      float exaggeration, float2 *__restrict__ yxy, LoopScalars *sc,
-                                                     int next_slot, int recenter) {
+                                                     double2 *centre_parts, int next_slot, int recenter) {
     const float normalization = load_normalization(z_ptr, sc, z_inv_scale, N);
     float lo = INFINITY, hi = -INFINITY;
-    const Centre c = load_centre<FUSED>(sc, next_slot, N, recenter);
+    const Centre c = load_centre<FUSED>(sc, centre_parts, next_slot, N, recenter);
     float sx = 0.0f, sy = 0.0f;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
         float gx = gains[i], gy = gains[N + i];
@@ -150,7 +176,7 @@ __global__ __launch_bounds__(256) void update_kernel(float *__restrict__ emb, fl
             }
             publish_bounds(sc, next_slot, lo, hi);
         }
-        if (recenter) publish_centre(sc, next_slot, sx, sy);
+        if (recenter) publish_centre(sc, centre_parts, next_slot, sx, sy);
     }
 }
 
@@ -162,11 +188,11 @@ __global__ __launch_bounds__(256) void update_vec4_kernel(float *__restrict__ em
                                                           float *__restrict__ old, int N, float eta,
                                                           const float *__restrict__ z_ptr, double z_inv_scale,
                                                           float momentum, float exaggeration,
-                                                          float2 *__restrict__ yxy, LoopScalars *sc, int next_slot,
-                                                          int recenter) {
+                                                          float2 *__restrict__ yxy, LoopScalars *sc,
+                                                          double2 *centre_parts, int next_slot, int recenter) {
     const float normalization = load_normalization(z_ptr, sc, z_inv_scale, N);
     float lo = INFINITY, hi = -INFINITY;
-    const Centre c = load_centre<FUSED>(sc, next_slot, N, recenter);
+    const Centre c = load_centre<FUSED>(sc, centre_parts, next_slot, N, recenter);
     float sx = 0.0f, sy = 0.0f;
     const int n4 = N / 4;
     float4 *emb4 = reinterpret_cast<float4 *>(emb), *attr4 = reinterpret_cast<float4 *>(attr);
@@ -230,7 +256,7 @@ __global__ __launch_bounds__(256) void update_vec4_kernel(float *__restrict__ em
             }
             publish_bounds(sc, next_slot, lo, hi);
         }
-        if (recenter) publish_centre(sc, next_slot, sx, sy);
+        if (recenter) publish_centre(sc, centre_parts, next_slot, sx, sy);
     }
 }
 
@@ -272,25 +298,26 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
         // Eighteen arrays are streamed at once; the fewer workgroups walk them with a grid stride, the narrower
         // the window of each array that is open at any time.  Measured at 1 M points: 256-384 workgroups 19 us,
         // 512 25 us, one item per thread (977 workgroups) 39 us.
-        const int blocks = std::min(div_up(N / 4, 256), p->stream_grid);
+        const int blocks = std::min(std::min(div_up(N / 4, 256), p->stream_grid), kMaxCentreParts);
         if (next_slot >= 0) {
             update_vec4_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
                                                             momentum, exaggeration, p->yxy, p->scalars,
-                                                            next_slot, p->recenter ? 1 : 0);
+                                                            p->centre_parts, next_slot, p->recenter ? 1 : 0);
         } else {
             update_vec4_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
-                                                             momentum, exaggeration, nullptr, p->scalars, 0, 0);
+                                                             momentum, exaggeration, nullptr, p->scalars, nullptr, 0, 0);
         }
         TSNE_LAUNCHED(s);
         return 0;
     }
-    const int blocks = std::min(div_up(N, 256), 4 * p->stream_grid);  // 4-byte accesses: the same window
+    const int blocks = std::min(std::min(div_up(N, 256), 4 * p->stream_grid), kMaxCentreParts);  // 4-byte accesses: the same window
     if (next_slot >= 0) {
         update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
-                                                   momentum, exaggeration, p->yxy, p->scalars, next_slot, p->recenter ? 1 : 0);
+                                                   momentum, exaggeration, p->yxy, p->scalars, p->centre_parts, next_slot,
+                                                   p->recenter ? 1 : 0);
     } else {
         update_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
-                                                    momentum, exaggeration, nullptr, p->scalars, 0, 0);
+                                                    momentum, exaggeration, nullptr, p->scalars, nullptr, 0, 0);
     }
     TSNE_LAUNCHED(s);
     return 0;
@@ -298,10 +325,8 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
 
 // Coordinate sums of `embedding` into the centre sums of `slot` (start of a re-centred loop).
 int launch_centre_sums(tsne_hip_plan *p, const float *embedding, int slot, hipStream_t s) {
-    centre_reset_kernel<<<1, 64, 0, s>>>(p->scalars, slot);
-    TSNE_LAUNCHED(s);
     const int blocks = std::min(div_up(p->num_points, 256 * 4), 1024);
-    centre_sums_kernel<<<std::max(blocks, 1), 256, 0, s>>>(embedding, p->num_points, p->scalars, slot);
+    centre_sums_kernel<<<std::max(blocks, 1), 256, 0, s>>>(embedding, p->num_points, p->scalars, p->centre_parts, slot);
     TSNE_LAUNCHED(s);
     return 0;
 }
