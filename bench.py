@@ -51,6 +51,17 @@ def traffic_from_profile(path):
     return total, "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes over this command, profiles/" + os.path.basename(path)
 
 
+def profile_commit(path):
+    """The commit the counter summary says it was taken at (a line `commit: <hash>` in the file), so that a
+    summary older than the kernel it describes is visible in the bench line."""
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.lower().startswith("commit:"):
+            return line.split(":", 1)[1].strip()
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -162,6 +173,26 @@ def main():
     plan.iterate_(None, None, y, gains, old, done, done + prof_steps, eta=eta)
     prof = plan.profile_end()
     kernels_us = {name: 1e3 * ms / max(cnt, 1) for name, (ms, cnt) in prof.items()}
+    done += prof_steps
+    # ... and the dominant kernel's duration as the product runs it: beside the repulsive chain on the other
+    # stream (a pair of HIP events around that kernel alone, on the stream it is launched on).
+    overlapped_ms = None
+    if not args.no_overlap:
+        plan.profile_attractive_begin()
+        plan.iterate_(None, None, y, gains, old, done, done + prof_steps, eta=eta)
+        total_ms, launches = plan.profile_attractive_end()
+        done += prof_steps
+        overlapped_ms = total_ms / launches if launches else None
+    # ---- a stretch late in the fit: past the end of the early exaggeration (step 250), where the embedding has
+    # spread out and the grouping of the points by grid tile lasts longer than in the first hundred steps ----
+    late_from = max(done, 300)
+    plan.iterate_(None, None, y, gains, old, done, late_from, eta=eta)
+    late_runs, done = [], late_from
+    for _ in range(max(1, args.repeats)):
+        z, run_s = timed(lambda: plan.iterate_(None, None, y, gains, old, done, done + args.steps, eta=eta))
+        late_runs.append(run_s)
+        done += args.steps
+    late_s = sorted(late_runs)[len(late_runs) // 2]
     attr_ms = kernels_us["attractive_kernel"] * 1e-3  # profiling slot of whichever attractive kernel ran
     attr_bytes = 8.0 * n * k + 16.0 * n  # P and index streams; read positions, write forces
     achieved = attr_bytes / (attr_ms * 1e-3) / 1e9
@@ -187,13 +218,13 @@ def main():
         for name, b in loop_bytes.items() if kernels_us.get(name)}
     if knn_stats[0] == 1:
         # Flop the matrix sweep executed per tile pair it did not skip: three products of bf16 terms
-        # (v_mfma_f32_32x32x16_bf16) over the dimensions + 3, padded to 16 (up to 125 dimensions) or to 64 (chunked
+        # (v_mfma_f32_32x32x16_bf16) over the dimensions + 3, padded to 16 (up to 125 dimensions) or to 32 (chunked
         # sweep, beyond 126); at exactly 126 dimensions float products over 128 (v_mfma_f32_32x32x2_f32).
         tiles = -(-n // 128)
         if d == 126:
             per_pair, peak, pipe = 2.0 * 128 * 128 * 128, 157.3, "fp32"
         else:
-            pad = 16 if d + 3 <= 128 else 64
+            pad = 16 if d + 3 <= 128 else 32
             per_pair, peak, pipe = 2.0 * 128 * 128 * 3 * (-(-(d + 3) // pad) * pad), 2500.0, "bf16"
         flop = per_pair * tiles * tiles * knn_stats[2] / 1000.0
         phase_rooflines["knn"] = {"bound": "mfma", "flop": flop, "achieved": flop / knn_s / 1e12, "unit": "TFLOP/s",
@@ -261,9 +292,11 @@ def main():
     # HBM bytes per launch of the dominant kernel: not measurable from inside this process (it takes two
     # rocprofv3 counter passes), so it is read from the committed summary of those passes over this same
     # command; the counters belong to that exact workload, so other sizes - or a missing summary - report null.
-    traffic, traffic_source = None, None
+    traffic, traffic_source, traffic_commit = None, None, None
     if args.workload == "c3" and n == 1000000 and k == 90:
-        traffic, traffic_source = traffic_from_profile(os.path.join(ROOT, "profiles", "bench_c3_1M_hbm_counters.txt"))
+        prof_path = os.path.join(ROOT, "profiles", "bench_c3_1M_hbm_counters.txt")
+        traffic, traffic_source = traffic_from_profile(prof_path)
+        traffic_commit = profile_commit(prof_path)
 
     # ---- the smaller configurations end to end, and c0 in full on the CPU ----
     small = None
@@ -307,6 +340,10 @@ def main():
         "config": {"workload": "%s: %d x %d fp32, perplexity %g, K=%d, lr %g; step = one gradient iteration"
                                % (args.workload, n, d, fit["perplexity"], k, eta)},
         "loop_seconds_runs": loop_runs,
+        "late_ms_per_step": late_s * 1e3 / args.steps,
+        "late_iters_per_sec": args.steps / late_s,
+        "late_stretch": "steps %d-%d of the same fit (exaggeration 1, momentum 0.8), median of %d stretches of %d"
+                        % (late_from, done, len(late_runs), args.steps),
         "fit_seconds": fit_s,
         "fit_seconds_runs": fit_runs,
         "smaller_configs": small,
@@ -317,7 +354,10 @@ def main():
                      "gradient_loop_%d_steps" % args.steps: loop_s, "data_generation_host": gen_s},
         "roofline": {"bound": "hbm", "kernel": "attractive_blocked_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "traffic_source": traffic_source, "bytes_per_launch": attr_bytes, "ms_per_launch": attr_ms},
+                     "traffic_source": traffic_source, "traffic_profile_commit": traffic_commit,
+                     "bytes_per_launch": attr_bytes, "ms_per_launch": attr_ms,
+                     "overlapped_ms_per_launch": overlapped_ms,
+                     "overlapped_frac": (attr_bytes / (overlapped_ms * 1e-3) / 1e9 / HBM_PEAK_GBS) if overlapped_ms else None},
         "kernels_us": kernels_us,
         "phase_rooflines": phase_rooflines,
         "knn_approximate": approx,

@@ -301,6 +301,12 @@ int tsne_hip_profile_kernel_count(void);
 const char *tsne_hip_profile_kernel_name(int id);
 int tsne_hip_profile_begin(tsne_hip_plan *plan);
 int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches);
+/* The same for the attractive kernel alone while the loop runs as it does unprofiled (its kernels on two
+ * streams, the repulsive chain beside the attractive kernel): a pair of events around that one kernel on the
+ * stream it is launched on; *total_ms / *launches give its duration beside the chain (no reference counterpart:
+ * the reference runs its phases one after the other). */
+int tsne_hip_profile_attractive_begin(tsne_hip_plan *plan);
+int tsne_hip_profile_attractive_end(tsne_hip_plan *plan, double *total_ms, int *launches);
 
 #ifdef __cplusplus
 }

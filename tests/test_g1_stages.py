@@ -92,6 +92,32 @@ def test_perplexity(stages, c0_problem):
     assert np.array_equal(p.view(np.uint32), c["p"].view(np.uint32))
 
 
+@pytest.mark.parametrize("data,k,perp", [
+    ("c0", 90, 1.5), ("c0", 90, 2.0), ("c0", 90, 5.0), ("c0", 6, 1.2), ("c0", 3, 1.3),
+    ("d300", 1023, 30.0), ("d300", 300, 5.0), ("d300", 90, 2.0), ("d300", 1100, 50.0),
+])
+def test_perplexity_far_below_the_neighbour_count(stages, c0_problem, data, k, perp):
+    """Perplexities of 1.2 to 5 on 90 neighbours, and 300-dimensional data whose normalised distances are
+    nearly equal within a row: the search then needs precisions at which exp(-beta d) underflows (subnormal
+    probabilities, rows whose sum is zero for some of the betas tried, rows that use all 200 evaluations).
+    Every row still follows the oracle's path: the same final beta and the same probabilities, bit for bit."""
+    from tsnecuda import synthetic
+    if data == "c0":
+        X = c0_problem["X"]
+    else:
+        X = synthetic.gaussian_clusters(6000, d=300, clusters=4, center_scale=5.0, seed=7)
+    idx, d2 = stages.knn(dev(X), k)
+    dn = stages.max_normalize_(d2)
+    p, beta = stages.perplexity(dn, perp, 1e-4, return_betas=True)
+    p, beta = p.cpu().numpy(), beta.cpu().numpy()
+    p_o, beta_o, iters = oracle.perplexity(dn.cpu().numpy(), perp, 1e-4, return_search=True)
+    print("perplexity %s k=%d perp=%g: most evaluations %d, rows at the cap %d, subnormal probabilities %d"
+          % (data, k, perp, iters.max(), int((iters == 200).sum()), int(((p_o > 0) & (p_o < 1.1754944e-38)).sum())))
+    assert np.isfinite(p).all()
+    assert float((beta != beta_o).mean()) == 0.0
+    assert np.array_equal(p.view(np.uint32), p_o.view(np.uint32))
+
+
 def test_symmetrize(stages, c0_problem):
     c = c0_problem
     P = stages.symmetrize(dev(c["p"]), dev(c["idx"])).cpu().numpy()
@@ -518,6 +544,18 @@ def test_errors_are_reported(stages):
         stages.knn(dev(np.zeros((5, 2), np.float32)), 9)
     with pytest.raises(RuntimeError, match="n_boxes_per_dim"):
         stages.Plan(100, 5, n_boxes_per_dim=1000)
+    # neighbour numbers that name no point are refused by the stages that build addresses from them
+    idx = np.tile(np.arange(4, dtype=np.int32), (300, 1))
+    p = np.full((300, 4), 0.25, np.float32)
+    for bad in (300, -1):
+        idx_bad = idx.copy()
+        idx_bad[17, 2] = bad
+        with pytest.raises(RuntimeError, match="outside"):
+            stages.symmetrize_full(dev(p), dev(idx_bad))
+        plan = stages.Plan(300, 4)
+        with pytest.raises(RuntimeError, match="outside"):
+            plan.prepare_attractive(dev(p), dev(idx_bad))
+        plan.close()
 
 
 @pytest.mark.parametrize("n,k", [(5000, 90), (20000, 30), (9000, 7), (300, 300), (150000, 12)])

@@ -213,6 +213,21 @@ def test_fit_with_approximate_neighbours(monkeypatch, capfd):
     assert t_approx >= t_exact - 0.03
 
 
+def test_approximate_neighbours_fall_back_for_very_many_neighbours(monkeypatch, capfd):
+    """The inverted-file search restricts the register-resident matrix sweep; 1400 neighbours in 100 dimensions
+    are more than its candidate lists hold, and the fit then searches exactly (and says so) instead of ending."""
+    from tsnecuda import TSNE, synthetic
+    X = synthetic.gaussian_clusters(6000, d=100, clusters=3, seed=8)
+    Y0 = synthetic_start(X.shape[0])
+    kw = dict(perplexity=50.0, num_neighbors=1400, n_iter=4, perplexity_epsilon=1e-4)
+    exact = TSNE(**kw).fit_transform(X, y=Y0)
+    monkeypatch.setenv("TSNE_KNN", "ivf")
+    emb = TSNE(verbose=1, **kw).fit_transform(X, y=Y0)
+    out = capfd.readouterr().out
+    assert "(inverted file: not for 1400 neighbours, exact search instead)" in out
+    assert np.array_equal(emb, exact)
+
+
 def test_fit_with_adaptive_grid(monkeypatch, capfd):
     """TSNE_ADAPTIVE_BOXES=1: every 50 steps the grid follows the spread of the embedding.  From a start that
     is 160 units wide the first check moves from 130 to 170 boxes; the interpolation error of the repulsive

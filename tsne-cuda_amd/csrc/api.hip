@@ -123,10 +123,27 @@ static bool overlap_enabled(const tsne_hip_plan *p) {
 // dependencies whichever stream they were recorded on and runs as before.)
 // Attractive forces of a step: the explicit N x K pattern if given, else the plan's CSR pattern if one is set,
 // else the re-blocked pattern.
+static int attractive_mark(tsne_hip_plan *p, hipStream_t s) {
+    if (!p->profiling_attractive) return 0;
+    if (p->attractive_events_used == p->attractive_events.size()) {
+        hipEvent_t e;
+        TSNE_TRY(hipEventCreate(&e));
+        p->attractive_events.push_back(e);
+    }
+    TSNE_TRY(hipEventRecord(p->attractive_events[p->attractive_events_used++], s));
+    return 0;
+}
+
 static int launch_step_attractive(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s) {
-    if (pij) return launch_attractive(p, pij, indices, p->attr, s);
-    if (p->csr_row_ptr) return launch_attractive_csr(p, p->csr_row_ptr, p->csr_col_idx, p->csr_values, p->attr, s);
-    return launch_attractive_blocked(p, p->attr, s);
+    if (attractive_mark(p, s)) return 1;
+    int rc;
+    if (pij)
+        rc = launch_attractive(p, pij, indices, p->attr, s);
+    else if (p->csr_row_ptr)
+        rc = launch_attractive_csr(p, p->csr_row_ptr, p->csr_col_idx, p->csr_values, p->attr, s);
+    else
+        rc = launch_attractive_blocked(p, p->attr, s);
+    return rc || attractive_mark(p, s);
 }
 
 static bool overlap_active(const tsne_hip_plan *p) {
@@ -211,7 +228,7 @@ static int launch_two_steps(tsne_hip_plan *p, const float *pij, const int *indic
 static bool graphs_enabled(const tsne_hip_plan *p) {
     const char *v = std::getenv("TSNE_GRAPH");  // read on every call: cheap, and lets one process try both
     const int mode = v ? (v[0] == '0' ? 0 : 1) : -1;
-    if (p->profiling || sync_kernels_enabled() || mode == 0) return false;
+    if (p->profiling || p->profiling_attractive || sync_kernels_enabled() || mode == 0) return false;
     // Measured gain per step beside two streams without a graph: 2 % at 100000 points, 0-0.5 % from 200000 to a
     // million (and none against one stream up to kSingleStreamPoints); setting a graph up costs about 4 ms
     // whatever the size.
@@ -344,6 +361,7 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     if (p->side_stream) (void)hipStreamSynchronize(p->side_stream);
     (void)hipDeviceSynchronize();
     for (hipEvent_t e : p->events) (void)hipEventDestroy(e);
+    for (hipEvent_t e : p->attractive_events) (void)hipEventDestroy(e);
     if (p->fork_event) (void)hipEventDestroy(p->fork_event);
     if (p->join_event) (void)hipEventDestroy(p->join_event);
     for (auto &g : p->step_graphs) (void)hipGraphExecDestroy(g.exec);
@@ -621,6 +639,32 @@ int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches) {
         launches[id] += 1;
     }
     plan->events_used = 0;
+    return 0;
+}
+
+int tsne_hip_profile_attractive_begin(tsne_hip_plan *plan) {
+    if (check_plan(plan, "profile_attractive_begin")) return 1;
+    plan->profiling_attractive = true;
+    plan->attractive_events_used = 0;
+    return 0;
+}
+
+int tsne_hip_profile_attractive_end(tsne_hip_plan *plan, double *total_ms, int *launches) {
+    if (check_plan(plan, "profile_attractive_end")) return 1;
+    TSNE_REQUIRE(total_ms && launches, "profile_attractive_end: null output");
+    plan->profiling_attractive = false;
+    *total_ms = 0.0;
+    *launches = 0;
+    const size_t used = plan->attractive_events_used;
+    plan->attractive_events_used = 0;
+    if (used < 2) return 0;
+    TSNE_TRY(hipEventSynchronize(plan->attractive_events[used - 1]));
+    for (size_t e = 0; e + 1 < used; e += 2) {
+        float ms = 0.0f;
+        TSNE_TRY(hipEventElapsedTime(&ms, plan->attractive_events[e], plan->attractive_events[e + 1]));
+        *total_ms += ms;
+        *launches += 1;
+    }
     return 0;
 }
 

@@ -33,6 +33,7 @@
 #include <vector>
 
 #include "plan.h"
+#include "stages.h"
 
 namespace tsnehip {
 
@@ -590,6 +591,8 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
         set_error("attractive_prepare: num_neighbors = %d is too large for the blocked format", K);
         return kShapeNotSupported;
     }
+    // Columns address LDS bitmaps and partition tables below: all of them must name a point.
+    if (validate_indices(indices, (int64_t)N * K, N, "attractive_prepare", s)) return 1;
     // Equal strips, or - when they all run at once - strips of equal predicted cost.
     std::vector<int> row0;
     if (div_up(N, kStripMax) <= cus && N > cus * kMicroRows && std::getenv("TSNE_EQUAL_STRIPS") == nullptr) {

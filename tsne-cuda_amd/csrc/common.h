@@ -36,6 +36,10 @@ bool sync_kernels_enabled();
         if (::tsnehip::sync_kernels_enabled()) TSNE_TRY(hipStreamSynchronize(stream));              \
     } while (0)
 
+// Return code of the launchers that have a fallback: the shape is beyond what this form of the kernel holds
+// (as opposed to 1, a failure).
+constexpr int kShapeNotSupported = 2;
+
 inline int div_up(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
 constexpr int kWave = 64;

@@ -179,17 +179,23 @@ void RunTsne(Options &opt, GpuOptions &gpu_opt) {
     const char *knn_env = std::getenv("TSNE_KNN");
     const bool approximate = (opt.approximate_neighbors || (knn_env && std::string(knn_env) == "ivf")) && D <= 126 &&
                              N >= 4096;
+    bool searched = false;
     if (approximate) {
         int nprobe = env_int("TSNE_KNN_NPROBE", opt.knn_nprobe);
         if (nprobe <= 0) nprobe = 100;
         int nlist = 0, knn_stats[3] = {0, 0, 0};
-        TSNE_OR_DIE(tsnehip::run_knn_approximate(d_points.as<float>(), N, D, K, nprobe, d_idx.as<int>(),
-                                                 d_dist.as<float>(), &nlist, knn_stats, stream),
-                    "approximate kNN");
-        if (verbose)
+        const int rc = tsnehip::run_knn_approximate(d_points.as<float>(), N, D, K, nprobe, d_idx.as<int>(),
+                                                    d_dist.as<float>(), &nlist, knn_stats, stream);
+        // (neighbour counts whose candidate lists the restricted sweep cannot hold keep the exact search)
+        if (rc != 0 && rc != tsnehip::kShapeNotSupported) TSNE_OR_DIE(rc, "approximate kNN");
+        searched = rc == 0;
+        if (verbose && searched)
             std::cout << "(inverted file: " << nlist << " lists, " << std::min(nprobe, nlist) << " probed per list, "
                       << knn_stats[2] << " per mille of the tile pairs compared) " << std::flush;
-    } else {
+        if (verbose && !searched)
+            std::cout << "(inverted file: not for " << K << " neighbours, exact search instead) " << std::flush;
+    }
+    if (!searched) {
         TSNE_OR_DIE(tsnehip::run_knn(d_points.as<float>(), N, D, K, d_idx.as<int>(), d_dist.as<float>(), stream),
                     "kNN");
     }

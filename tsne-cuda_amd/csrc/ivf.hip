@@ -368,9 +368,9 @@ int run_knn_ivf_caller_order(const float *points, int N, int D, int K, const flo
         set_error("knn_ivf: out of device memory");
         return 1;
     }
-    if (run_knn_ivf(points, N, D, K, centroids, nlist, nprobe, order.as<int>(), idx_new.as<int>(),
-                    d_new.as<float>(), stats, s))
-        return 1;
+    if (const int rc = run_knn_ivf(points, N, D, K, centroids, nlist, nprobe, order.as<int>(), idx_new.as<int>(),
+                                   d_new.as<float>(), stats, s))
+        return rc;  // (kShapeNotSupported: the restricted sweep cannot hold this many neighbours)
     unpermute_kernel<<<(int)std::min<int64_t>(div_up((int64_t)nnz, 256), 65536), 256, 0, s>>>(
         idx_new.as<int>(), d_new.as<float>(), order.as<int>(), N, K, indices, sq_dist);
     TSNE_TRY(hipGetLastError());

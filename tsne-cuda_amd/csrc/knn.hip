@@ -1987,12 +1987,12 @@ int run_knn_mode(const float *points, int N, int D, int K, int *indices, float *
     bool use_mfma = mode == 2 || (mode == 0 && mfma_fits && N >= 8192);
     if (mode == 2 && !mfma_fits) {
         set_error("knn: the matrix-instruction sweep does not fit %d dimensions / %d neighbours", D, K);
-        return 1;
+        return kShapeNotSupported;
     }
     if (probes && (!use_mfma || chunked)) {
         set_error("knn: the approximate search runs on the register-resident matrix sweep only (at most 126 "
                   "dimensions; got %d dimensions, %d neighbours)", D, K);
-        return 1;
+        return kShapeNotSupported;
     }
 
     const int Npad = div_up(N, kCT) * kCT;

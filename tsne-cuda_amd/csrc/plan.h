@@ -134,6 +134,11 @@ struct tsne_hip_plan {
     std::vector<hipEvent_t> events;
     std::vector<int> event_kernel;  // kernel id per recorded event, -1 = end marker
     size_t events_used = 0;
+    // The other mode: the loop runs as it does unprofiled (two streams), and only the attractive kernel is
+    // bracketed by a pair of events on the stream it is launched on (its duration beside the repulsive chain).
+    bool profiling_attractive = false;
+    std::vector<hipEvent_t> attractive_events;
+    size_t attractive_events_used = 0;
 };
 
 namespace tsnehip {
@@ -174,7 +179,6 @@ int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, fl
 // Returns 0, kShapeNotSupported when the blocked format cannot hold the problem (more than 8192 column
 // partitions, num_neighbors >= 4096, or a strip of more than 2^31 entries; the row-ordered kernel then
 // serves), or 1 for any other failure (allocation, launch).
-constexpr int kShapeNotSupported = 2;
 int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s);
 void release_blocked(tsne_hip_plan *p);
 int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s);

@@ -44,6 +44,8 @@ int launch_max_normalize(float *values, int64_t n, float *scratch, hipStream_t s
 int launch_perplexity(const float *sq_dist, int N, int K, float perplexity, float eps, float *pij, float *betas,
                       hipStream_t s);
 int launch_symmetrize(const float *p, const int *idx, int N, int K, float *P, hipStream_t s);
+// 0 if all n neighbour indices lie in [0, N), else 1 with the error set (named after `who`); synchronises the stream.
+int validate_indices(const int *idx, int64_t n, int N, const char *who, hipStream_t s);
 // (A + A^T) / 2N in CSR form with the union pattern (symmetrize_full.hip): device radix sort of the (row,
 // column, value) triples of A and A^T, then a segmented reduce.  row_ptr: N + 1 ints; col_idx / values: room
 // for 2 * N * K entries.  Allocates its work buffers and synchronises the stream; *nnz_out (host) = entries.

@@ -9,6 +9,9 @@
 // every index row is fetched with coalesced loads and the match is found with a
 // ballot.
 #include "plan.h"
+#include "stages.h"
+
+#include <algorithm>
 
 namespace tsnehip {
 
@@ -41,7 +44,38 @@ __global__ __launch_bounds__(256) void symmetrize_kernel(const float *__restrict
     }
 }
 
+__global__ __launch_bounds__(256) void index_range_kernel(const int *__restrict__ idx, int64_t n, int N,
+                                                          int *__restrict__ flag) {
+    bool bad = false;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x)
+        bad = bad || (unsigned int)idx[e] >= (unsigned int)N;
+    if (__any(bad) && (threadIdx.x & (kWave - 1)) == 0) atomicOr(flag, 1);
+}
+
 }  // namespace
+
+// The stages that turn neighbour numbers into addresses of their own (sort keys, LDS bitmaps, row pointers)
+// first make sure that every one of them names a point: 0 if all n indices lie in [0, N), else 1 with the error
+// set.  Synchronises the stream.
+int validate_indices(const int *idx, int64_t n, int N, const char *who, hipStream_t s) {
+    int *flag = nullptr;
+    TSNE_TRY(hipMalloc(&flag, sizeof(int)));
+    int host = 0;
+    hipError_t e = hipMemsetAsync(flag, 0, sizeof(int), s);
+    if (e == hipSuccess) {
+        index_range_kernel<<<(int)std::min<int64_t>(div_up(n, 256 * 8), 2048), 256, 0, s>>>(idx, n, N, flag);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(&host, flag, sizeof(int), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    (void)hipFree(flag);
+    TSNE_TRY(e);
+    if (host) {
+        set_error("%s: a neighbour index lies outside [0, %d)", who, N);
+        return 1;
+    }
+    return 0;
+}
 
 int launch_symmetrize(const float *p, const int *idx, int N, int K, float *P, hipStream_t s) {
     if (K <= 16) {

@@ -442,10 +442,14 @@ int radix_sort_pairs(u64 *keys, float *vals, u64 *keys_alt, float *vals_alt, int
 int symmetrize_full(const float *p, const int *idx, int N, int K, int *row_ptr, int *col_idx, float *values,
                     int64_t *nnz_out, hipStream_t s) {
     const int64_t nnz = (int64_t)N * K, n = 2 * nnz;
-    if (n >= ((int64_t)1 << 32)) {
-        set_error("symmetrize_full: %lld triples exceed the 32-bit positions of the sort", (long long)n);
+    // (positions, row pointers and the entry count are 32-bit signed)
+    if (n >= ((int64_t)1 << 31)) {
+        set_error("symmetrize_full: %lld triples exceed the 31-bit positions of the sort and the row pointers",
+                  (long long)n);
         return 1;
     }
+    // A column outside [0, N) would spill into the row bits of its sort key.
+    if (validate_indices(idx, nnz, N, "symmetrize_full", s)) return 1;
     const int col_bits = bits_for(N);
     const int n_tiles = div_up(n, kSortTile), scan_tiles = div_up(n, kScanTile);
     Buffer keys, vals, keys_alt, vals_alt, hist, tile_sums;

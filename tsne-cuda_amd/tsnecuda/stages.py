@@ -70,7 +70,10 @@ def lib():
         L.tsne_hip_profile_kernel_name.restype = ctypes.c_char_p
         L.tsne_hip_profile_begin.argtypes = [_vp]
         L.tsne_hip_profile_end.argtypes = [_vp, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_int)]
-        for name in ("profile_begin", "profile_end", "profile_kernel_count"):
+        L.tsne_hip_profile_attractive_begin.argtypes = [_vp]
+        L.tsne_hip_profile_attractive_end.argtypes = [_vp, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_int)]
+        for name in ("profile_begin", "profile_end", "profile_kernel_count", "profile_attractive_begin",
+                     "profile_attractive_end"):
             getattr(L, "tsne_hip_" + name).restype = c_int
         for name in ("locality_order", "gather_rows", "knn", "max_normalize", "perplexity", "symmetrize", "plan_create", "attractive",
                      "repulsive", "update", "iterate", "sum_squares"):
@@ -314,6 +317,16 @@ class Plan(object):
         cnt = (ctypes.c_int * n)()
         _check(lib().tsne_hip_profile_end(self._h, ms, cnt))
         return {lib().tsne_hip_profile_kernel_name(i).decode(): (ms[i], cnt[i]) for i in range(n)}
+
+    def profile_attractive_begin(self):
+        _check(lib().tsne_hip_profile_attractive_begin(self._h))
+
+    def profile_attractive_end(self):
+        """(total ms, launches) of the attractive kernel in the iterate_ calls since profile_attractive_begin,
+        with the loop's kernels on two streams as in an unprofiled run."""
+        ms, cnt = ctypes.c_double(), ctypes.c_int()
+        _check(lib().tsne_hip_profile_attractive_end(self._h, ctypes.byref(ms), ctypes.byref(cnt)))
+        return ms.value, cnt.value
 
     def repulsive_error(self, embedding, sample_count):
         """(relative L2 error of the interpolated repulsive forces, relative error of the
