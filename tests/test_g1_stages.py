@@ -558,13 +558,17 @@ def test_errors_are_reported(stages):
         plan.close()
 
 
-@pytest.mark.parametrize("n,k", [(5000, 90), (20000, 30), (9000, 7), (300, 300), (150000, 12)])
-def test_attractive_blocked_pattern(stages, n, k):
+@pytest.mark.parametrize("n,k", [(5000, 90), (20000, 30), (9000, 7), (300, 300), (150000, 12), (1100000, 5)])
+def test_attractive_blocked_pattern(stages, monkeypatch, n, k):
     """The re-blocked (row strip x column partition) copy of the pattern gives
     the same forces as the oracle; 20000 and 9000 points span several column
     partitions, 300 x 300 is a dense pattern in a single bucket, 150000 x 12
     gives every strip several work items with dozens of partition runs in
-    each (74 partitions, ~95 entries per run)."""
+    each (74 partitions, ~95 entries per run), 1100000 x 5 spans three column
+    windows of the direct form and has more strips than the device compute units.
+    Both forms of the step kernel (partitions staged in LDS; neighbours gathered
+    from memory) and the one the library picks by itself: the sums are integer
+    sums of the same terms, so all three give the same bits."""
     rng = np.random.default_rng(n + k)
     if n <= 20000:
         idx = np.stack([rng.permutation(n)[:k] for _ in range(n)]).astype(np.int32)
@@ -575,14 +579,22 @@ def test_attractive_blocked_pattern(stages, n, k):
     P[:, 0] = 0.0
     y = (rng.standard_normal(2 * n) * 8.0).astype(np.float32)
     want = oracle.attractive(P, idx, y)
-    plan = stages.Plan(n, k)
-    plan.prepare_attractive(dev(P), dev(idx))
-    got = plan.attractive(None, None, dev(y)).cpu().numpy()
-    assert rel_l2(got, want) <= 1e-4
-    # integer accumulation: the result does not depend on the order of the additions
-    again = plan.attractive(None, None, dev(y)).cpu().numpy()
-    assert np.array_equal(got, again)
-    plan.close()
+    results = {}
+    for form in ("staged", "direct", None):
+        if form:
+            monkeypatch.setenv("TSNE_ATTRACTIVE_FORM", form)
+        else:
+            monkeypatch.delenv("TSNE_ATTRACTIVE_FORM")
+        plan = stages.Plan(n, k)
+        plan.prepare_attractive(dev(P), dev(idx))
+        got = plan.attractive(None, None, dev(y)).cpu().numpy()
+        assert rel_l2(got, want) <= 1e-4, form
+        # integer accumulation: the result does not depend on the order of the additions
+        again = plan.attractive(None, None, dev(y)).cpu().numpy()
+        assert np.array_equal(got, again)
+        plan.close()
+        results[form] = got
+    assert np.array_equal(results["staged"], results["direct"]) and np.array_equal(results["staged"], results[None])
 
 
 def test_attractive_wait_that_runs_out_is_reported(stages, monkeypatch):
@@ -596,6 +608,7 @@ def test_attractive_wait_that_runs_out_is_reported(stages, monkeypatch):
     P = (rng.random((n, k)) * 1e-5).astype(np.float32)
     y = (rng.standard_normal(2 * n) * 8.0).astype(np.float32)
     monkeypatch.setenv("TSNE_ATTRACTIVE_SPIN_LIMIT", "0")
+    monkeypatch.setenv("TSNE_ATTRACTIVE_FORM", "staged")  # (the form with the two roles)
     plan = stages.Plan(n, k)
     plan.prepare_attractive(dev(P), dev(idx))
     got = plan.attractive(None, None, dev(y)).cpu().numpy()

@@ -53,6 +53,23 @@ constexpr int kStreamWaves = kStreamThreads / kWave;
 constexpr int kLoadThreads = kBlock - kStreamThreads;  // ... waves 12-15 stage the partitions
 constexpr int kLoadWaves = kLoadThreads / kWave;
 constexpr unsigned int kItemEntries = kPrefetch * kStreamThreads;
+// The second form ("direct"): where a strip's runs are short - ten million points in four clusters: a strip of
+// 3968 rows references all 1220 partitions of its cluster, 290 entries each - staging 16 KB of positions per run
+// costs several times the entries themselves, and every run is a hand-over between the kernel's two roles.  The
+// entries then keep the same order (by partition, so that the workgroups, which walk their strips at about the
+// same pace, ask the caches for the same stretch of the position array at about the same time), but their
+// column is packed relative to a window of 2^19 points and the step kernel gathers every neighbour's position
+// from memory itself: no staging, no roles, no waits.  What bounds it then is the number of distinct cache lines
+// a wave's 64 position loads touch, so a strip's entries are sorted by column (a device radix sort by (strip,
+// column), once): 64 consecutive entries of a run of 470 over a partition's 128 lines of 16 positions meet
+// about 17 lines instead of 50.
+constexpr int kWindowBits = 19;
+constexpr int kWindowPoints = 1 << kWindowBits;
+constexpr int kMaxWindows = 32;     // 2^24 points
+constexpr unsigned int kDirectPiece = 128;  // consecutive entries of an item that one wave's lanes hold (two each)
+constexpr int kDirectStripMax = 6400;  // rows per strip of the direct form when the strips outnumber the compute
+                                       // units anyway: 150 KB of positions and accumulators, the whole LDS
+static_assert((kDirectStripMax - 1) >> (32 - kWindowBits) == 0, "row within strip and column within window share 32 bits");
 constexpr int kSpinLimit = 1 << 18; // polls of an LDS counter before a wave gives up waiting (about ten milliseconds;
                                     // a wait normally ends within a microsecond): every wave reaches the kernel's end.
                                     // TSNE_ATTRACTIVE_SPIN_LIMIT (read when the pattern is prepared) overrides it, so
@@ -249,6 +266,7 @@ __global__ void clear_pmax_kernel(float *p_max) {
 // stay in flight across them; measured cost: none); the counters only grow.
 // Every wait is a bounded poll.
 // ---------------------------------------------------------------------------
+template <int STRIP_MAX = kStripMax>
 __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int rl, float vx, float vy,
                                           double scale) {
     // magic + v * scale is a double in [2^52, 2^53), where doubles are the integers: its bit pattern is the
@@ -259,7 +277,7 @@ __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int 
     // x sums and y sums live in separate arrays: consecutive rows then fall
     // into consecutive 8-byte slots and the atomics of a wave spread over all banks.
     atomicAdd(&acc[rl], (unsigned long long)__double_as_longlong(tx));
-    atomicAdd(&acc[kStripMax + rl], (unsigned long long)__double_as_longlong(ty));
+    atomicAdd(&acc[STRIP_MAX + rl], (unsigned long long)__double_as_longlong(ty));
 }
 
 // Polls *counter until it reaches `need`; after kSpinLimit polls the wave sets *gave_up and goes on (the
@@ -462,6 +480,268 @@ __global__ __launch_bounds__(kBlock, 8) void attractive_blocked_kernel(const flo
     if (gave_up && tid == 0) atomicAdd(&scalars->wait_timeouts, 1u);
 }
 
+// How many (strip, partition) runs the pattern has: per strip the partitions it references, summed into *runs.
+__global__ __launch_bounds__(kBlock) void count_runs_kernel(const int *__restrict__ idx, int K,
+                                                            const int *__restrict__ strip_row0,
+                                                            unsigned long long *__restrict__ runs) {
+    __shared__ unsigned int seen[kMaxParts / 32];
+    __shared__ unsigned int total;
+    const int tid = threadIdx.x;
+    const int row0 = strip_row0[blockIdx.x];
+    const unsigned int count = (unsigned int)(strip_row0[blockIdx.x + 1] - row0) * (unsigned int)K;
+    const size_t base = (size_t)row0 * K;
+    for (int w = tid; w < kMaxParts / 32; w += kBlock) seen[w] = 0u;
+    if (tid == 0) total = 0u;
+    __syncthreads();
+    for (unsigned int e = tid; e < count; e += kBlock) {
+        const unsigned int part = (unsigned int)idx[base + e] / kPartPoints;
+        const unsigned int bit = 1u << (part & 31u);
+        if (!(seen[part >> 5] & bit)) atomicOr(&seen[part >> 5], bit);
+    }
+    __syncthreads();
+    unsigned int mine = 0u;
+    for (int w = tid; w < kMaxParts / 32; w += kBlock) mine += __popc(seen[w]);
+    mine = (unsigned int)group_sum<kWave>((float)mine);  // (at most 8192: exact in a float)
+    if ((tid & (kWave - 1)) == 0) atomicAdd(&total, mine);
+    __syncthreads();
+    if (tid == 0) atomicAdd(runs, (unsigned long long)total);
+}
+
+// ---------------------------------------------------------------------------
+// Preparation of the direct form.  Sort key of an entry: (row within strip) << 40 | strip << 24 | column; the
+// sort orders by the low 24 + strip bits, i.e. by (strip, column), and is stable.  A strip's entries then are the
+// rows * K sorted pairs from row0 * K on.  Every window's entries are padded to a multiple of kDirectPiece, so
+// that each piece of that many consecutive entries - what one wave of the step kernel takes at a time - lies in
+// one window; the padding entries name a row past the strip's last.  A strip's list: {first row, windows, rows,
+// entries with padding}, then the entry at which every window's entries start, the padded entry count, ~0, ~0.
+// ---------------------------------------------------------------------------
+typedef unsigned long long u64;
+constexpr int kDirectColBits = 24;
+static_assert(kMaxWindows * kWindowPoints == 1 << kDirectColBits, "columns of the direct form fit their key bits");
+
+// uniform_rows > 0: every strip has that many rows (the last one fewer); otherwise the boundaries are searched
+// (at most 1024 strips).
+__global__ __launch_bounds__(256) void direct_keys_kernel(const float *__restrict__ pij, const int *__restrict__ idx,
+                                                          long long nnz, int K, const int *__restrict__ strip_row0,
+                                                          int n_strips, int uniform_rows, u64 *__restrict__ keys,
+                                                          float *__restrict__ vals) {
+    __shared__ int bounds[1025];
+    if (!uniform_rows) {
+        for (int b = threadIdx.x; b <= n_strips; b += 256) bounds[b] = strip_row0[b];
+        __syncthreads();
+    }
+    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < nnz; e += (long long)gridDim.x * 256) {
+        const int i = (int)(e / K);
+        int strip, first;
+        if (uniform_rows) {
+            strip = i / uniform_rows;
+            first = strip * uniform_rows;
+        } else {
+            int lo = 0, hi = n_strips;  // the last boundary <= i
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (bounds[mid] <= i) lo = mid; else hi = mid;
+            }
+            strip = lo;
+            first = bounds[lo];
+        }
+        keys[e] = ((u64)(unsigned int)(i - first) << 40) | ((u64)(unsigned int)strip << kDirectColBits) |
+                  (u64)(unsigned int)idx[e];
+        vals[e] = pij[e];
+    }
+}
+
+// One workgroup of 128 threads per strip: where the strip's entries of every window start (a binary search in
+// its sorted keys), the padding ahead of every window (wpad: kMaxWindows + 1 words per strip), the strip's list,
+// and the padding entries themselves.
+__global__ __launch_bounds__(128) void direct_windows_kernel(const u64 *__restrict__ keys, int K,
+                                                             const int *__restrict__ strip_row0, int n_windows,
+                                                             unsigned int *__restrict__ wseg, int wseg_stride,
+                                                             unsigned int *__restrict__ wpad,
+                                                             float *__restrict__ ent_p) {
+    __shared__ unsigned int ustart[kMaxWindows + 1], pad[kMaxWindows + 1];
+    const int strip = blockIdx.x, tid = threadIdx.x;
+    const int row0 = strip_row0[strip], nrows = strip_row0[strip + 1] - row0;
+    const u64 *mine = keys + (size_t)row0 * K;
+    const unsigned int count = (unsigned int)nrows * (unsigned int)K;
+    if (tid <= n_windows) {
+        const unsigned int want = (unsigned int)tid << kWindowBits;  // first column of the window
+        unsigned int lo = 0u, hi = count;                           // first entry whose column is >= want
+        while (lo < hi) {
+            const unsigned int mid = (lo + hi) >> 1;
+            if ((unsigned int)(mine[mid] & ((1u << kDirectColBits) - 1u)) < want) lo = mid + 1u; else hi = mid;
+        }
+        ustart[tid] = tid == n_windows ? count : lo;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        unsigned int total = 0u;
+        for (int w = 0; w < n_windows; ++w) {
+            pad[w] = total;
+            const unsigned int len = ustart[w + 1] - ustart[w];
+            total += ((len + kDirectPiece - 1u) & ~(kDirectPiece - 1u)) - len;
+        }
+        pad[n_windows] = total;
+    }
+    __syncthreads();
+    unsigned int *whdr = wseg + (size_t)strip * wseg_stride;
+    if (tid <= n_windows) {
+        wpad[(size_t)strip * (kMaxWindows + 1) + tid] = pad[tid];
+        whdr[4 + tid] = ustart[tid] + pad[tid];
+    }
+    if (tid == 0) {
+        whdr[0] = (unsigned int)row0;
+        whdr[1] = (unsigned int)n_windows;
+        whdr[2] = (unsigned int)nrows;
+        whdr[3] = count + pad[n_windows];
+        whdr[4 + n_windows + 1] = ~0u;
+        whdr[4 + n_windows + 2] = ~0u;
+    }
+    for (int w = 0; w < n_windows; ++w) {
+        const unsigned int dummies = pad[w + 1] - pad[w];  // they follow the window's last entry
+        if ((unsigned int)tid < dummies)
+            reinterpret_cast<uint2 *>(ent_p)[entry_slot(ustart[w + 1] + pad[w] + tid, strip, (int)gridDim.x)] =
+                make_uint2(0u, ~0u);
+    }
+}
+
+__global__ __launch_bounds__(256) void direct_emit_kernel(const u64 *__restrict__ keys, const float *__restrict__ vals,
+                                                          long long nnz, int K, const int *__restrict__ strip_row0,
+                                                          int n_strips, const unsigned int *__restrict__ wpad,
+                                                          float *__restrict__ ent_p, float *__restrict__ p_max) {
+    float biggest = 0.0f;
+    for (long long q = (long long)blockIdx.x * 256 + threadIdx.x; q < nnz; q += (long long)gridDim.x * 256) {
+        const u64 key = keys[q];
+        const unsigned int col = (unsigned int)(key & ((1u << kDirectColBits) - 1u));
+        const int strip = (int)((key >> kDirectColBits) & 0xffffu);
+        const unsigned int row_local = (unsigned int)(key >> 40);
+        const unsigned int e = (unsigned int)(q - (long long)strip_row0[strip] * K);
+        const unsigned int pos = e + wpad[(size_t)strip * (kMaxWindows + 1) + (col >> kWindowBits)];
+        const float pv = vals[q];
+        biggest = fmaxf(biggest, fabsf(pv));
+        reinterpret_cast<uint2 *>(ent_p)[entry_slot(pos, strip, n_strips)] =
+            make_uint2(__float_as_uint(pv), (col & (kWindowPoints - 1u)) | (row_local << kWindowBits));
+    }
+    biggest = group_max<kWave>(biggest);
+    if ((threadIdx.x & (kWave - 1)) == 0) atomicMax(reinterpret_cast<unsigned int *>(p_max), __float_as_uint(biggest));
+}
+
+// ---------------------------------------------------------------------------
+// Direct form of the step kernel: one workgroup (twelve waves) per strip; LDS holds the strip's positions and
+// its force accumulators, the entries stream from memory as in the staged kernel (three rotating register sets,
+// two items in flight), and every entry's neighbour position is a load of its own, issued for all entries of
+// the item before the first is used.  Same arithmetic, same fixed-point sums.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kStreamThreads) void attractive_direct_kernel(const float *__restrict__ ent_p,
+                                                                        const unsigned int *__restrict__ wseg,
+                                                                        const float2 *__restrict__ yxy,
+                                                                        const LoopScalars *__restrict__ scalars,
+                                                                        float *__restrict__ attr, int N, int K,
+                                                                        int wseg_stride) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    float2 *yi = reinterpret_cast<float2 *>(lds_raw);
+    unsigned long long *acc = reinterpret_cast<unsigned long long *>(yi + kDirectStripMax);
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int strip = blockIdx.x;
+    typedef const __attribute__((address_space(4))) unsigned int *ConstWords;
+    ConstWords hdr = (ConstWords)(wseg + (size_t)strip * wseg_stride);
+    const int row0 = (int)hdr[0];
+    const int nrows = (int)hdr[2];
+    ConstWords window_start = hdr + 4;  // the count after the last window, then ~0
+    const float pm = scalars->vmax;
+    const double scale = pm > 0.0f ? 2251799813685248.0 / (double)pm : 1.0;  // 2^51 / p_max
+    const unsigned long long acc_start =
+        0ull - (unsigned long long)K * (unsigned long long)__double_as_longlong(kRoundMagic);
+    for (int r = tid; r < nrows; r += kStreamThreads) {
+        yi[r] = yxy[row0 + r];
+        acc[r] = acc_start;
+        acc[kDirectStripMax + r] = acc_start;
+    }
+    __syncthreads();
+
+    typedef unsigned int Entry __attribute__((ext_vector_type(2)));  // {probability bits, packed row / column}
+    typedef unsigned int EntryPair __attribute__((ext_vector_type(4)));
+    const unsigned int count = hdr[3];  // (with the windows' padding)
+    const unsigned int n_items = (count + kItemEntries - 1u) / kItemEntries;
+    struct PhaseRegs {
+        Entry en[kPrefetch];  // en[2 j + h]: entry 128 ((tid + j kStreamThreads) / 64) + 64 h + lane of the item
+    };
+    const EntryPair *pairs = reinterpret_cast<const EntryPair *>(ent_p) + (size_t)strip * (kItemEntries / 2) + tid;
+    const size_t item_pitch = (size_t)gridDim.x * (kItemEntries / 2);
+    auto issue = [&](PhaseRegs &R, unsigned int item) {
+        const EntryPair *src = pairs + (size_t)min(item, n_items - 1u) * item_pitch;
+#pragma unroll
+        for (int j = 0; j < kPrefetch / 2; ++j) {
+            const EntryPair v = __builtin_nontemporal_load(src + j * kStreamThreads);
+            R.en[2 * j] = Entry{v.x, v.y};
+            R.en[2 * j + 1] = Entry{v.z, v.w};
+        }
+    };
+    // A lane's four entries of an item are two pairs (t, t + 64), one pair in each of two pieces of kDirectPiece
+    // consecutive entries, and a piece lies in one window: the window of each of the wave's two pieces is tracked
+    // in scalar registers (windows are listed whether or not the strip has entries in them).
+    static_assert(kPrefetch == 4 && kDirectPiece == 2 * kWave, "two pieces of 128 entries per wave and item");
+    const unsigned int wave = (unsigned int)__builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n_windows = (int)hdr[1];
+    int win[2] = {0, 0};
+    unsigned int boundary[2] = {window_start[1], window_start[1]};  // where the window after win[j] starts
+    // Item R: every position load first, then the loads of the item two ahead (into Rn), then the arithmetic.
+    // Loads return in the order of issue as far as a wave's counters can tell: entry loads issued ahead of the
+    // position loads would have to land (from HBM) before the first position could be used.  Everything is
+    // unconditional - an item past the last one loads the last item again and none of its entries is in range -
+    // so that the outstanding-load counts the compiler works with are exact.
+    auto consume = [&](PhaseRegs &R, unsigned int item, PhaseRegs &Rn, unsigned int next_item) {
+        const unsigned int first = item * kItemEntries;
+        float2 yj[kPrefetch];
+        bool on[kPrefetch];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const unsigned int t0 = first + kDirectPiece * (wave + (unsigned int)j * kStreamWaves);
+            while (t0 >= boundary[j]) {  // (rare: a few dozen times per strip)
+                ++win[j];
+                boundary[j] = window_start[win[j] + 1];
+            }
+            const float2 *base = yxy + (size_t)min(win[j], n_windows - 1) * kWindowPoints;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int k = 2 * j + h;
+                const unsigned int t = t0 + 64u * (unsigned int)h + (unsigned int)lane;
+                on[k] = t < count && (R.en[k].y >> kWindowBits) < (unsigned int)nrows;
+                yj[k] = base[on[k] ? (R.en[k].y & (kWindowPoints - 1u)) : 0u];
+            }
+        }
+        issue(Rn, next_item);
+#pragma unroll
+        for (int k = 0; k < kPrefetch; ++k) {
+            if (on[k]) {
+                const unsigned int rl = R.en[k].y >> kWindowBits;
+                const float2 y0 = yi[rl];
+                const float dx = y0.x - yj[k].x, dy = y0.y - yj[k].y;
+                const float w = __uint_as_float(R.en[k].x) * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
+                add_force<kDirectStripMax>(acc, rl, w * dx, w * dy, scale);
+            }
+        }
+    };
+    PhaseRegs R0, R1, R2;
+    issue(R0, 0u);
+    issue(R1, 1u);
+    for (unsigned int p = 0; p < n_items; p += 3) {
+        consume(R0, p, R2, p + 2);
+        consume(R1, p + 1, R0, p + 3);
+        consume(R2, p + 2, R1, p + 4);
+    }
+    __syncthreads();
+    const double inv_scale = 1.0 / scale;
+    for (int r = tid; r < nrows; r += kStreamThreads) {
+        attr[row0 + r] = (float)((double)(long long)acc[r] * inv_scale);
+        attr[N + row0 + r] = (float)((double)(long long)acc[kDirectStripMax + r] * inv_scale);
+    }
+}
+
+constexpr size_t kDirectLds = sizeof(float2) * kDirectStripMax + sizeof(unsigned long long) * 2 * kDirectStripMax;
+static_assert(kDirectLds <= 160 * 1024, "one workgroup must fit the 160 KB of LDS");
+
 constexpr size_t kBlockedLds =
     sizeof(float2) * 2 * kPartPoints + sizeof(float2) * kStripMax + sizeof(unsigned long long) * 2 * kStripMax;
 static_assert(kBlockedLds <= 160 * 1024, "one workgroup must fit the 160 KB of LDS");
@@ -482,6 +762,7 @@ static_assert(kBlockedLds <= 160 * 1024, "one workgroup must fit the 160 KB of L
 namespace {
 
 constexpr int kMicroRows = 64;
+constexpr double kDirectRunEntries = 1000.0;  // mean entries per (strip, partition) run below which the direct form runs
 constexpr long long kPartCostEntries = 2000;
 
 __global__ __launch_bounds__(256) void micro_strip_parts_kernel(const int *__restrict__ idx, int N, int K, int words,
@@ -565,10 +846,55 @@ void release_blocked(tsne_hip_plan *p) {
     (void)hipFree(p->ent_p);
     (void)hipFree(p->seg);
     (void)hipFree(p->strip_row0);
+    (void)hipFree(p->wseg);
+    p->wseg = nullptr;
+    p->blocked_direct = false;
     p->ent_p = nullptr;
     p->seg = nullptr;
     p->strip_row0 = nullptr;
     p->blocked_ready = false;
+}
+
+// Fills ent_p and wseg of the direct form (both allocated, strip_row0 on the device, p_max cleared).
+static int prepare_direct(tsne_hip_plan *p, const float *pij, const int *indices, int uniform_rows, hipStream_t s) {
+    const int N = p->num_points, K = p->num_neighbors;
+    const long long nnz = (long long)N * K;
+    int strip_bits = 1;
+    while ((1 << strip_bits) < p->n_strips) ++strip_bits;
+    struct Scratch {
+        void *ptr = nullptr;
+        ~Scratch() {
+            if (ptr) (void)hipFree(ptr);
+        }
+    } keys, keys_alt, vals, vals_alt, hist, wpad;
+    const int sort_tiles = div_up(nnz, radix_sort_tile());
+    if (hipMalloc(&keys.ptr, sizeof(u64) * (size_t)nnz) != hipSuccess ||
+        hipMalloc(&keys_alt.ptr, sizeof(u64) * (size_t)nnz) != hipSuccess ||
+        hipMalloc(&vals.ptr, sizeof(float) * (size_t)nnz) != hipSuccess ||
+        hipMalloc(&vals_alt.ptr, sizeof(float) * (size_t)nnz) != hipSuccess ||
+        hipMalloc(&hist.ptr, sizeof(unsigned int) * 256 * ((size_t)sort_tiles + 1)) != hipSuccess ||
+        hipMalloc(&wpad.ptr, sizeof(unsigned int) * (size_t)p->n_strips * (kMaxWindows + 1)) != hipSuccess) {
+        set_error("attractive_prepare: out of device memory for sorting %lld entries", nnz);
+        return 1;
+    }
+    const int blocks = (int)std::min<long long>(div_up(nnz, 256), 65536);
+    direct_keys_kernel<<<blocks, 256, 0, s>>>(pij, indices, nnz, K, p->strip_row0, p->n_strips, uniform_rows,
+                                              static_cast<u64 *>(keys.ptr), static_cast<float *>(vals.ptr));
+    TSNE_LAUNCHED(s);
+    if (radix_sort_pairs(static_cast<u64 *>(keys.ptr), static_cast<float *>(vals.ptr), static_cast<u64 *>(keys_alt.ptr),
+                         static_cast<float *>(vals_alt.ptr), nnz, kDirectColBits + strip_bits,
+                         static_cast<unsigned int *>(hist.ptr), s))
+        return 1;
+    direct_windows_kernel<<<p->n_strips, 128, 0, s>>>(static_cast<u64 *>(keys.ptr), K, p->strip_row0, p->n_windows,
+                                                      p->wseg, p->wseg_stride, static_cast<unsigned int *>(wpad.ptr),
+                                                      p->ent_p);
+    TSNE_LAUNCHED(s);
+    direct_emit_kernel<<<blocks, 256, 0, s>>>(static_cast<u64 *>(keys.ptr), static_cast<float *>(vals.ptr), nnz, K,
+                                              p->strip_row0, p->n_strips, static_cast<unsigned int *>(wpad.ptr),
+                                              p->ent_p, &p->scalars->vmax);
+    TSNE_LAUNCHED(s);
+    TSNE_TRY(hipStreamSynchronize(s));  // the scratch arrays go out of scope
+    return 0;
 }
 
 int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s) {
@@ -609,13 +935,69 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     // A strip's list: the run starts (padded: the force kernel reads two past the last run) and the partitions.
     p->list_words = (n_parts + 4 + 3) & ~3;
     p->seg_stride = 4 + p->list_words + ((n_parts + 3) & ~3);
-    // Entries: whole items for every strip (the last item of a strip is padded; the padding is never consumed).
-    const size_t items_per_strip = ((size_t)strip_rows * K + kItemEntries - 1) / kItemEntries;
+    if (hipMalloc(&p->strip_row0, sizeof(int) * row0.size()) != hipSuccess ||
+        hipMemcpy(p->strip_row0, row0.data(), sizeof(int) * row0.size(), hipMemcpyHostToDevice) != hipSuccess) {
+        release_blocked(p);
+        set_error("attractive_prepare: out of device memory for the strip boundaries");
+        return 1;
+    }
+    // Which form: the direct one where the runs are short.  (TSNE_ATTRACTIVE_FORM=staged / direct overrides.)
+    {
+        unsigned long long *d_runs = nullptr, runs = 0;
+        hipError_t e = hipMalloc(&d_runs, sizeof(runs));
+        if (e == hipSuccess) e = hipMemsetAsync(d_runs, 0, sizeof(runs), s);
+        if (e == hipSuccess) {
+            count_runs_kernel<<<p->n_strips, kBlock, 0, s>>>(indices, K, p->strip_row0, d_runs);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipMemcpyAsync(&runs, d_runs, sizeof(runs), hipMemcpyDeviceToHost, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        (void)hipFree(d_runs);
+        if (e != hipSuccess) {
+            release_blocked(p);
+            TSNE_TRY(e);
+        }
+        const double run_entries = (double)N * K / (double)std::max<unsigned long long>(runs, 1ull);
+        // (measured: ten million points in four clusters, 290 entries per run: 2.6 ms per launch against 6.0 ms
+        // staged; fits of 50000 to 60000 points, 350 to 700 entries per run, whose strips all run at once: 2 % slower)
+        p->blocked_direct = run_entries < kDirectRunEntries && p->n_strips > cus;
+        if (const char *v = std::getenv("TSNE_ATTRACTIVE_FORM")) p->blocked_direct = v[0] == 'd';
+        // (the direct form's keys hold 24 bits of column and 16 of strip; its sort counts in 31 bits)
+        // (strips that are not all of one length are at most as many as the compute units)
+        if (div_up(N, kWindowPoints) > kMaxWindows || (int64_t)N * K >= ((int64_t)1 << 31) || cus > 1024)
+            p->blocked_direct = false;
+    }
+    int direct_uniform_rows = 0;
+    if (p->blocked_direct && p->n_strips > cus) {
+        direct_uniform_rows = kDirectStripMax;
+        // More strips than compute units whatever their size: the direct form then takes strips as long as the
+        // LDS holds (every strip walks the positions of all the columns it references once).
+        row0.clear();
+        for (int r = 0; r < N; r += kDirectStripMax) row0.push_back(r);
+        row0.push_back(N);
+        p->n_strips = (int)row0.size() - 1;
+        p->strip_rows = strip_rows = std::min(N, kDirectStripMax);
+        (void)hipFree(p->strip_row0);
+        p->strip_row0 = nullptr;
+        if (hipMalloc(&p->strip_row0, sizeof(int) * row0.size()) != hipSuccess ||
+            hipMemcpy(p->strip_row0, row0.data(), sizeof(int) * row0.size(), hipMemcpyHostToDevice) != hipSuccess) {
+            release_blocked(p);
+            set_error("attractive_prepare: out of device memory for the strip boundaries");
+            return 1;
+        }
+    }
+    p->n_windows = p->blocked_direct ? div_up(N, kWindowPoints) : 0;
+    p->wseg_stride = (4 + p->n_windows + 3 + 3) & ~3;
+    // Entries: whole items for every strip (the last item of a strip is padded; the padding is never consumed);
+    // the direct form pads every window's entries to whole pieces.
+    const size_t strip_entries = (size_t)strip_rows * K + (size_t)kDirectPiece * p->n_windows;
+    const size_t items_per_strip = (strip_entries + kItemEntries - 1) / kItemEntries;
     const size_t nnz = items_per_strip * p->n_strips * kItemEntries;
     bool ok = hipMalloc(&p->ent_p, 2 * sizeof(float) * nnz) == hipSuccess &&
-              hipMalloc(&p->seg, sizeof(unsigned int) * (size_t)p->n_strips * p->seg_stride) == hipSuccess &&
-              hipMalloc(&p->strip_row0, sizeof(int) * row0.size()) == hipSuccess &&
-              hipMemcpy(p->strip_row0, row0.data(), sizeof(int) * row0.size(), hipMemcpyHostToDevice) == hipSuccess;
+              hipMalloc(&p->seg, p->blocked_direct ? sizeof(unsigned int)
+                                                   : sizeof(unsigned int) * (size_t)p->n_strips * p->seg_stride) == hipSuccess &&
+              (!p->blocked_direct ||
+               hipMalloc(&p->wseg, sizeof(unsigned int) * (size_t)p->n_strips * p->wseg_stride) == hipSuccess);
     if (!ok) {
         release_blocked(p);
         set_error("attractive_prepare: out of device memory for the re-blocked pattern (%zu bytes)", nnz * 8);
@@ -623,12 +1005,20 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     }
     clear_pmax_kernel<<<1, 64, 0, s>>>(&p->scalars->vmax);
     TSNE_LAUNCHED(s);
-    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(reblock_kernel),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kReblockLds));
-    reblock_kernel<<<p->n_strips, kBlock, kReblockLds, s>>>(pij, indices, N, K, p->strip_row0, p->list_words, p->seg_stride, p->ent_p,
-                                                  p->seg,
-                                                  &p->scalars->vmax);
-    TSNE_LAUNCHED(s);
+    if (p->blocked_direct) {
+        if (const int rc = prepare_direct(p, pij, indices, direct_uniform_rows, s)) {
+            release_blocked(p);
+            return rc;
+        }
+    } else {
+        TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(reblock_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kReblockLds));
+        reblock_kernel<<<p->n_strips, kBlock, kReblockLds, s>>>(pij, indices, N, K, p->strip_row0, p->list_words,
+                                                                p->seg_stride, p->ent_p, p->seg, &p->scalars->vmax);
+        TSNE_LAUNCHED(s);
+    }
+    TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attractive_direct_kernel),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDirectLds));
     TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attractive_blocked_kernel<false>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBlockedLds));
     TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attractive_blocked_kernel<true>),
@@ -646,6 +1036,12 @@ int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s) {
         return 1;
     }
     if (profile_mark(p, kKernelAttractive, s)) return 1;
+    if (p->blocked_direct) {
+        attractive_direct_kernel<<<p->n_strips, kStreamThreads, kDirectLds, s>>>(
+            p->ent_p, p->wseg, p->yxy, p->scalars, attr, p->num_points, p->num_neighbors, p->wseg_stride);
+        TSNE_LAUNCHED(s);
+        return 0;
+    }
     const auto kernel = p->spin_limit == kSpinLimit ? attractive_blocked_kernel<false> : attractive_blocked_kernel<true>;
     kernel<<<p->n_strips, kBlock, kBlockedLds, s>>>(p->ent_p, p->seg, p->yxy, p->scalars, attr, p->num_points,
                                                     p->num_neighbors, p->list_words, p->seg_stride,

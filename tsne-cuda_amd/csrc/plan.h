@@ -98,6 +98,12 @@ struct tsne_hip_plan {
     unsigned int *seg = nullptr;    // per strip seg_stride words: counts, run starts, partitions in opening order
     int strip_rows = 0, n_strips = 0, n_parts = 0, list_words = 0, seg_stride = 0;  // strip_rows: of the longest strip
     int *strip_row0 = nullptr;      // n_strips + 1: first row of every strip
+    // Second form of the re-blocked pattern, for strips whose runs are short (see attractive_blocked.hip): the
+    // column of an entry is packed relative to a window of 2^19 points, wseg lists per strip where each
+    // window's entries start, and the step kernel gathers the neighbours' positions from memory.
+    bool blocked_direct = false;
+    unsigned int *wseg = nullptr;
+    int wseg_stride = 0, n_windows = 0;
     int spin_limit = 0;             // polls before a wave of the attractive kernel gives up a wait
     bool blocked_ready = false;
     // Optional CSR pattern (borrowed pointers; tsne_hip_plan_set_csr_pattern): when set, steps without an explicit
