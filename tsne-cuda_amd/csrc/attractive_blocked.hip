@@ -66,6 +66,9 @@ constexpr unsigned int kItemEntries = kPrefetch * kStreamThreads;
 constexpr int kWindowBits = 19;
 constexpr int kWindowPoints = 1 << kWindowBits;
 constexpr int kMaxWindows = 32;     // 2^24 points
+constexpr int kDirectThreads = 1024;  // sixteen waves, all of them streaming
+constexpr int kDirectWaves = kDirectThreads / kWave;
+constexpr unsigned int kDirectItem = kPrefetch * kDirectThreads;  // entries per item of the direct form
 constexpr unsigned int kDirectPiece = 128;  // consecutive entries of an item that one wave's lanes hold (two each)
 constexpr int kDirectStripMax = 6400;  // rows per strip of the direct form when the strips outnumber the compute
                                        // units anyway: 150 KB of positions and accumulators, the whole LDS
@@ -118,11 +121,12 @@ __device__ __forceinline__ unsigned int scan_slots(const unsigned int (&value)[k
 // Inside an item, every 128 entries are stored as 64 pairs (j, j + 64): a lane of the force kernel loads a pair
 // at a time, and the 64 lanes of a wave then hold 64 consecutive entries in each half of their registers
 // (consecutive entries belong to consecutive rows, whose accumulators lie in different LDS banks).
+template <unsigned int ITEM = kItemEntries>
 __device__ __forceinline__ size_t entry_slot(unsigned int pos, int strip, int n_strips) {
-    const unsigned int item = pos / kItemEntries;
-    const unsigned int in_item = pos - item * kItemEntries;
+    const unsigned int item = pos / ITEM;
+    const unsigned int in_item = pos - item * ITEM;
     const unsigned int j = in_item & 127u;
-    return ((size_t)item * n_strips + strip) * kItemEntries + (in_item - j) + 2u * (j & 63u) + (j >> 6);
+    return ((size_t)item * n_strips + strip) * ITEM + (in_item - j) + 2u * (j & 63u) + (j >> 6);
 }
 static_assert(kItemEntries % 128 == 0, "items hold whole groups of 64 entry pairs");
 
@@ -600,7 +604,7 @@ __global__ __launch_bounds__(128) void direct_windows_kernel(const u64 *__restri
     for (int w = 0; w < n_windows; ++w) {
         const unsigned int dummies = pad[w + 1] - pad[w];  // they follow the window's last entry
         if ((unsigned int)tid < dummies)
-            reinterpret_cast<uint2 *>(ent_p)[entry_slot(ustart[w + 1] + pad[w] + tid, strip, (int)gridDim.x)] =
+            reinterpret_cast<uint2 *>(ent_p)[entry_slot<kDirectItem>(ustart[w + 1] + pad[w] + tid, strip, (int)gridDim.x)] =
                 make_uint2(0u, ~0u);
     }
 }
@@ -619,7 +623,7 @@ __global__ __launch_bounds__(256) void direct_emit_kernel(const u64 *__restrict_
         const unsigned int pos = e + wpad[(size_t)strip * (kMaxWindows + 1) + (col >> kWindowBits)];
         const float pv = vals[q];
         biggest = fmaxf(biggest, fabsf(pv));
-        reinterpret_cast<uint2 *>(ent_p)[entry_slot(pos, strip, n_strips)] =
+        reinterpret_cast<uint2 *>(ent_p)[entry_slot<kDirectItem>(pos, strip, n_strips)] =
             make_uint2(__float_as_uint(pv), (col & (kWindowPoints - 1u)) | (row_local << kWindowBits));
     }
     biggest = group_max<kWave>(biggest);
@@ -627,12 +631,12 @@ __global__ __launch_bounds__(256) void direct_emit_kernel(const u64 *__restrict_
 }
 
 // ---------------------------------------------------------------------------
-// Direct form of the step kernel: one workgroup (twelve waves) per strip; LDS holds the strip's positions and
+// Direct form of the step kernel: one workgroup (sixteen waves) per strip; LDS holds the strip's positions and
 // its force accumulators, the entries stream from memory as in the staged kernel (three rotating register sets,
 // two items in flight), and every entry's neighbour position is a load of its own, issued for all entries of
 // the item before the first is used.  Same arithmetic, same fixed-point sums.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kStreamThreads) void attractive_direct_kernel(const float *__restrict__ ent_p,
+__global__ __launch_bounds__(kDirectThreads) void attractive_direct_kernel(const float *__restrict__ ent_p,
                                                                         const unsigned int *__restrict__ wseg,
                                                                         const float2 *__restrict__ yxy,
                                                                         const LoopScalars *__restrict__ scalars,
@@ -653,7 +657,7 @@ __global__ __launch_bounds__(kStreamThreads) void attractive_direct_kernel(const
     const double scale = pm > 0.0f ? 2251799813685248.0 / (double)pm : 1.0;  // 2^51 / p_max
     const unsigned long long acc_start =
         0ull - (unsigned long long)K * (unsigned long long)__double_as_longlong(kRoundMagic);
-    for (int r = tid; r < nrows; r += kStreamThreads) {
+    for (int r = tid; r < nrows; r += kDirectThreads) {
         yi[r] = yxy[row0 + r];
         acc[r] = acc_start;
         acc[kDirectStripMax + r] = acc_start;
@@ -663,17 +667,17 @@ __global__ __launch_bounds__(kStreamThreads) void attractive_direct_kernel(const
     typedef unsigned int Entry __attribute__((ext_vector_type(2)));  // {probability bits, packed row / column}
     typedef unsigned int EntryPair __attribute__((ext_vector_type(4)));
     const unsigned int count = hdr[3];  // (with the windows' padding)
-    const unsigned int n_items = (count + kItemEntries - 1u) / kItemEntries;
+    const unsigned int n_items = (count + kDirectItem - 1u) / kDirectItem;
     struct PhaseRegs {
-        Entry en[kPrefetch];  // en[2 j + h]: entry 128 ((tid + j kStreamThreads) / 64) + 64 h + lane of the item
+        Entry en[kPrefetch];  // en[2 j + h]: entry 128 ((tid + j kDirectThreads) / 64) + 64 h + lane of the item
     };
-    const EntryPair *pairs = reinterpret_cast<const EntryPair *>(ent_p) + (size_t)strip * (kItemEntries / 2) + tid;
-    const size_t item_pitch = (size_t)gridDim.x * (kItemEntries / 2);
+    const EntryPair *pairs = reinterpret_cast<const EntryPair *>(ent_p) + (size_t)strip * (kDirectItem / 2) + tid;
+    const size_t item_pitch = (size_t)gridDim.x * (kDirectItem / 2);
     auto issue = [&](PhaseRegs &R, unsigned int item) {
         const EntryPair *src = pairs + (size_t)min(item, n_items - 1u) * item_pitch;
 #pragma unroll
         for (int j = 0; j < kPrefetch / 2; ++j) {
-            const EntryPair v = __builtin_nontemporal_load(src + j * kStreamThreads);
+            const EntryPair v = __builtin_nontemporal_load(src + j * kDirectThreads);
             R.en[2 * j] = Entry{v.x, v.y};
             R.en[2 * j + 1] = Entry{v.z, v.w};
         }
@@ -692,12 +696,12 @@ __global__ __launch_bounds__(kStreamThreads) void attractive_direct_kernel(const
     // unconditional - an item past the last one loads the last item again and none of its entries is in range -
     // so that the outstanding-load counts the compiler works with are exact.
     auto consume = [&](PhaseRegs &R, unsigned int item, PhaseRegs &Rn, unsigned int next_item) {
-        const unsigned int first = item * kItemEntries;
+        const unsigned int first = item * kDirectItem;
         float2 yj[kPrefetch];
         bool on[kPrefetch];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const unsigned int t0 = first + kDirectPiece * (wave + (unsigned int)j * kStreamWaves);
+            const unsigned int t0 = first + kDirectPiece * (wave + (unsigned int)j * kDirectWaves);
             while (t0 >= boundary[j]) {  // (rare: a few dozen times per strip)
                 ++win[j];
                 boundary[j] = window_start[win[j] + 1];
@@ -733,7 +737,7 @@ __global__ __launch_bounds__(kStreamThreads) void attractive_direct_kernel(const
     }
     __syncthreads();
     const double inv_scale = 1.0 / scale;
-    for (int r = tid; r < nrows; r += kStreamThreads) {
+    for (int r = tid; r < nrows; r += kDirectThreads) {
         attr[row0 + r] = (float)((double)(long long)acc[r] * inv_scale);
         attr[N + row0 + r] = (float)((double)(long long)acc[kDirectStripMax + r] * inv_scale);
     }
@@ -991,8 +995,9 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     // Entries: whole items for every strip (the last item of a strip is padded; the padding is never consumed);
     // the direct form pads every window's entries to whole pieces.
     const size_t strip_entries = (size_t)strip_rows * K + (size_t)kDirectPiece * p->n_windows;
-    const size_t items_per_strip = (strip_entries + kItemEntries - 1) / kItemEntries;
-    const size_t nnz = items_per_strip * p->n_strips * kItemEntries;
+    const size_t item_entries = p->blocked_direct ? kDirectItem : kItemEntries;
+    const size_t items_per_strip = (strip_entries + item_entries - 1) / item_entries;
+    const size_t nnz = items_per_strip * p->n_strips * item_entries;
     bool ok = hipMalloc(&p->ent_p, 2 * sizeof(float) * nnz) == hipSuccess &&
               hipMalloc(&p->seg, p->blocked_direct ? sizeof(unsigned int)
                                                    : sizeof(unsigned int) * (size_t)p->n_strips * p->seg_stride) == hipSuccess &&
@@ -1037,7 +1042,7 @@ int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s) {
     }
     if (profile_mark(p, kKernelAttractive, s)) return 1;
     if (p->blocked_direct) {
-        attractive_direct_kernel<<<p->n_strips, kStreamThreads, kDirectLds, s>>>(
+        attractive_direct_kernel<<<p->n_strips, kDirectThreads, kDirectLds, s>>>(
             p->ent_p, p->wseg, p->yxy, p->scalars, attr, p->num_points, p->num_neighbors, p->wseg_stride);
         TSNE_LAUNCHED(s);
         return 0;
