@@ -954,7 +954,7 @@ def test_knn_few_failed_queries_are_redone_by_candidate_range(stages, sweep):
 def test_iterate_graph_replay_matches_eager(stages, c0_problem, monkeypatch):
     """Steps on one stream or two, launched one by one or as replays of a captured graph of two
     steps, with eager work and synchronisations between the calls, give what the plain loop gives
-    (to the repeatability of the loop itself: its float atomics are unordered)."""
+    (bit for bit: the loop's sums are integer sums)."""
     c = c0_problem
     n = c["P"].shape[0]
     dP, di = dev(c["P"]), dev(c["idx"])
