@@ -124,6 +124,49 @@ def test_symmetrize(stages, c0_problem):
     np.testing.assert_allclose(P, c["P"], rtol=1e-6, atol=0)
 
 
+@pytest.mark.parametrize("n,k,duplicates", [(5000, 90, False), (4096, 7, False), (30000, 24, True), (5000, 600, False)])
+def test_symmetrize_hashed_and_scanning_forms(stages, c0_problem, monkeypatch, n, k, duplicates):
+    """The symmetrisation looks a row's number up in a per-row hash table of the row it points to (the default
+    from 4096 points up) or scans that row (small problems, thousands of neighbours): the same values,
+    bit for bit; where a row names a column twice the hashed form notices and hands over to the scan, which adds
+    such values up.  Against the oracle either way."""
+    if (n, k) == (5000, 90):
+        p, idx = c0_problem["p"], c0_problem["idx"]
+    else:
+        rng = np.random.default_rng(n + k)
+        if duplicates:
+            idx = rng.integers(0, n, (n, k)).astype(np.int32)
+            idx[:, 0] = np.arange(n)
+            idx[::3, 5] = idx[::3, 2]   # columns named twice and three times in a row
+            idx[::7, 9] = idx[::7, 2]
+        else:
+            # row i names the columns i + o for k distinct offsets o (one of five offset sets): many mutual pairs
+            sets = np.stack([np.concatenate([[0], 1 + rng.choice(n - 1, size=k - 1, replace=False)]) for _ in range(5)])
+            sets[1, 1:] = (n - sets[0, 1:]) % n   # set 1 mirrors set 0: rows of those two sets name each other
+            idx = ((np.arange(n)[:, None] + sets[np.arange(n) % 5]) % n).astype(np.int32)
+        p = rng.random(idx.shape).astype(np.float32)
+        p[:, 0] = 0.0
+        p /= p.sum(1, keepdims=True)
+    want = oracle.symmetrize(p, idx)
+    got = {}
+    for form in ("hashed", "scan"):
+        if form == "scan":
+            monkeypatch.setenv("TSNE_SYMMETRIZE_SCAN", "1")
+        else:
+            monkeypatch.delenv("TSNE_SYMMETRIZE_SCAN", raising=False)
+        got[form] = stages.symmetrize(dev(p), dev(idx)).cpu().numpy()
+        np.testing.assert_allclose(got[form], want, rtol=2e-6, atol=0)
+    if not duplicates and k != 7:
+        assert (want > p / (2.0 * n) * (1.0 + 1e-3)).mean() > 0.005   # the case has pairs in both directions
+    assert np.array_equal(got["hashed"].view(np.uint32), got["scan"].view(np.uint32))
+    # a column that names no point is refused by the form that would address a table with it
+    monkeypatch.delenv("TSNE_SYMMETRIZE_SCAN", raising=False)
+    bad = idx.copy()
+    bad[n // 2, k // 2] = n
+    with pytest.raises(RuntimeError, match="outside"):
+        stages.symmetrize(dev(p), dev(bad))
+
+
 @pytest.mark.parametrize("n,k", [(2, 2), (7, 3), (300, 300), (5000, 90), (70000, 20), (20000, 1)])
 def test_symmetrize_full_csr(stages, c0_problem, n, k):
     """(A + A^T) / 2N with the union pattern: the device radix sort + segmented reduce against the oracle's
