@@ -70,8 +70,8 @@ constexpr int kDirectThreads = 1024;  // sixteen waves, all of them streaming
 constexpr int kDirectWaves = kDirectThreads / kWave;
 constexpr unsigned int kDirectItem = kPrefetch * kDirectThreads;  // entries per item of the direct form
 constexpr unsigned int kDirectPiece = 128;  // consecutive entries of an item that one wave's lanes hold (two each)
-constexpr int kDirectStripMax = 6400;  // rows per strip of the direct form when the strips outnumber the compute
-                                       // units anyway: 150 KB of positions and accumulators, the whole LDS
+constexpr int kDirectStripMax = 6784;  // rows per strip of the direct form when the strips outnumber the compute
+                                       // units anyway: 159 KB of positions and accumulators, the whole LDS
 static_assert((kDirectStripMax - 1) >> (32 - kWindowBits) == 0, "row within strip and column within window share 32 bits");
 constexpr int kSpinLimit = 1 << 18; // polls of an LDS counter before a wave gives up waiting (about ten milliseconds;
                                     // a wait normally ends within a microsecond): every wave reaches the kernel's end.
@@ -973,14 +973,17 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
     }
     int direct_uniform_rows = 0;
     if (p->blocked_direct && p->n_strips > cus) {
-        direct_uniform_rows = kDirectStripMax;
+        // As few rounds of strips over the compute units as the longest strips allow, and the strips of those
+        // rounds of equal length (a multiple of the wave).
+        const int rounds = div_up(N, (int64_t)cus * kDirectStripMax);
+        direct_uniform_rows = std::min(kDirectStripMax, div_up(div_up(N, (int64_t)cus * rounds), kWave) * kWave);
         // More strips than compute units whatever their size: the direct form then takes strips as long as the
         // LDS holds (every strip walks the positions of all the columns it references once).
         row0.clear();
-        for (int r = 0; r < N; r += kDirectStripMax) row0.push_back(r);
+        for (int r = 0; r < N; r += direct_uniform_rows) row0.push_back(r);
         row0.push_back(N);
         p->n_strips = (int)row0.size() - 1;
-        p->strip_rows = strip_rows = std::min(N, kDirectStripMax);
+        p->strip_rows = strip_rows = std::min(N, direct_uniform_rows);
         (void)hipFree(p->strip_row0);
         p->strip_row0 = nullptr;
         if (hipMalloc(&p->strip_row0, sizeof(int) * row0.size()) != hipSuccess ||
