@@ -199,14 +199,14 @@ def main():
 
     # ---- every phase against its roofline -----------------------------------
     # Algorithmic bytes per launch of the loop's kernels (G = 390 interpolation nodes per side, four charge
-    # planes; the transposed spectra are 2 plane pairs x 1024 x 512 complex).
-    G2, spectra = 390.0 * 390.0, 2 * 1024 * 512 * 8.0
+    # planes; the transposed spectra are 2 plane pairs x 1024 x 512 complex; 21 fixed-point moments per box).
+    G2, spectra, moments = 390.0 * 390.0, 2 * 1024 * 512 * 8.0, 21 * 130 * 130 * 8.0
     loop_bytes = {
         "tile_count_kernel": 12.0 * n,                      # positions in, (tile, rank) codes out
         "tile_scatter_kernel": 20.0 * n,                    # positions and codes in, positions grouped by tile out
-        "spread_kernel": 8.0 * n + 16.0 * G2,               # grouped positions in, node charges out
-        "conv_rows_forward_kernel": 16.0 * G2 + spectra,    # node charges in, row spectra out
-        "conv_columns_kernel": 2.0 * spectra,               # row spectra in, convolved columns out
+        "spread_kernel": 8.0 * n + moments,                 # grouped positions in, box moments out
+        "conv_rows_forward_kernel": moments + spectra,      # box moments in (-> node charges), row spectra out
+        "conv_columns_kernel": 2.0 * spectra + moments,     # row spectra in, convolved columns out, box moments cleared
         "conv_rows_inverse_kernel": spectra + 16.0 * G2,    # in, node potentials out
         "gather_forces_kernel": 16.0 * n + 16.0 * G2,       # positions and node potentials in, forces out
         "attractive_kernel": attr_bytes,
