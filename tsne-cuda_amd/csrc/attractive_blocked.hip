@@ -270,9 +270,8 @@ __global__ void clear_pmax_kernel(float *p_max) {
 // stay in flight across them; measured cost: none); the counters only grow.
 // Every wait is a bounded poll.
 // ---------------------------------------------------------------------------
-template <int STRIP_MAX = kStripMax>
 __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int rl, float vx, float vy,
-                                          double scale) {
+                                          double scale, int y_offset = kStripMax) {
     // magic + v * scale is a double in [2^52, 2^53), where doubles are the integers: its bit pattern is the
     // magic's plus round(v * scale).  The patterns themselves are summed; every row has exactly K entries, so
     // its accumulators start at -K times the magic's pattern (mod 2^64) and end at the sum of the integers.
@@ -281,7 +280,7 @@ __device__ __forceinline__ void add_force(unsigned long long *acc, unsigned int 
     // x sums and y sums live in separate arrays: consecutive rows then fall
     // into consecutive 8-byte slots and the atomics of a wave spread over all banks.
     atomicAdd(&acc[rl], (unsigned long long)__double_as_longlong(tx));
-    atomicAdd(&acc[STRIP_MAX + rl], (unsigned long long)__double_as_longlong(ty));
+    atomicAdd(&acc[y_offset + rl], (unsigned long long)__double_as_longlong(ty));
 }
 
 // Polls *counter until it reaches `need`; after kSpinLimit polls the wave sets *gave_up and goes on (the
@@ -641,10 +640,10 @@ __global__ __launch_bounds__(kDirectThreads) void attractive_direct_kernel(const
                                                                         const float2 *__restrict__ yxy,
                                                                         const LoopScalars *__restrict__ scalars,
                                                                         float *__restrict__ attr, int N, int K,
-                                                                        int wseg_stride) {
+                                                                        int wseg_stride, int rows_cap) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     float2 *yi = reinterpret_cast<float2 *>(lds_raw);
-    unsigned long long *acc = reinterpret_cast<unsigned long long *>(yi + kDirectStripMax);
+    unsigned long long *acc = reinterpret_cast<unsigned long long *>(yi + rows_cap);
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int strip = blockIdx.x;
@@ -660,7 +659,7 @@ __global__ __launch_bounds__(kDirectThreads) void attractive_direct_kernel(const
     for (int r = tid; r < nrows; r += kDirectThreads) {
         yi[r] = yxy[row0 + r];
         acc[r] = acc_start;
-        acc[kDirectStripMax + r] = acc_start;
+        acc[rows_cap + r] = acc_start;
     }
     __syncthreads();
 
@@ -723,7 +722,7 @@ __global__ __launch_bounds__(kDirectThreads) void attractive_direct_kernel(const
                 const float2 y0 = yi[rl];
                 const float dx = y0.x - yj[k].x, dy = y0.y - yj[k].y;
                 const float w = __uint_as_float(R.en[k].x) * __builtin_amdgcn_rcpf(1.0f + dx * dx + dy * dy);
-                add_force<kDirectStripMax>(acc, rl, w * dx, w * dy, scale);
+                add_force(acc, rl, w * dx, w * dy, scale, rows_cap);
             }
         }
     };
@@ -739,7 +738,7 @@ __global__ __launch_bounds__(kDirectThreads) void attractive_direct_kernel(const
     const double inv_scale = 1.0 / scale;
     for (int r = tid; r < nrows; r += kDirectThreads) {
         attr[row0 + r] = (float)((double)(long long)acc[r] * inv_scale);
-        attr[N + row0 + r] = (float)((double)(long long)acc[kDirectStripMax + r] * inv_scale);
+        attr[N + row0 + r] = (float)((double)(long long)acc[rows_cap + r] * inv_scale);
     }
 }
 
@@ -1045,8 +1044,10 @@ int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s) {
     }
     if (profile_mark(p, kKernelAttractive, s)) return 1;
     if (p->blocked_direct) {
-        attractive_direct_kernel<<<p->n_strips, kDirectThreads, kDirectLds, s>>>(
-            p->ent_p, p->wseg, p->yxy, p->scalars, attr, p->num_points, p->num_neighbors, p->wseg_stride);
+        // (LDS for the longest strip only: what is left of a compute unit's 160 KB hosts the repulsive chain's kernels)
+        const int rows_cap = (p->strip_rows + kWave - 1) / kWave * kWave;
+        attractive_direct_kernel<<<p->n_strips, kDirectThreads, (size_t)24 * rows_cap, s>>>(
+            p->ent_p, p->wseg, p->yxy, p->scalars, attr, p->num_points, p->num_neighbors, p->wseg_stride, rows_cap);
         TSNE_LAUNCHED(s);
         return 0;
     }
