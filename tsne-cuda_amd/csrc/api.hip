@@ -584,23 +584,16 @@ int tsne_hip_iterate(tsne_hip_plan *plan, const float *pij, const int *indices, 
     if (launch_bounds(plan, embedding, slot, s, !continues)) return 1;
     if (plan->recenter && launch_centre_sums(plan, embedding, slot, s)) return 1;
     if (launch_pack_xy(plan, embedding, s)) return 1;
-    // Schedule of src/fit_tsne.cu:416-420: two stretches of constant parameters; the step that reports the
-    // normalisation runs by itself.
-    const int last = normalization ? step_end - 1 : step_end;
-    const int switch_at = std::min(std::max(force_magnify_iters, step_begin), last);
+    // Schedule of src/fit_tsne.cu:416-420: two stretches of constant parameters.  The normalisation of the last
+    // step is read afterwards: its partial sums stay in the loop scalars until the next step's chain clears them.
+    const int switch_at = std::min(std::max(force_magnify_iters, step_begin), step_end);
     if (launch_steps(plan, pij, indices, embedding, gains, old_forces, eta, pre_exaggeration_momentum,
                      early_exaggeration, switch_at - step_begin, slot, s))
         return 1;
     if (launch_steps(plan, pij, indices, embedding, gains, old_forces, eta, post_exaggeration_momentum, 1.0f,
-                     last - switch_at, slot, s))
+                     step_end - switch_at, slot, s))
         return 1;
-    if (normalization) {
-        const bool late = last >= force_magnify_iters;
-        if (launch_step(plan, pij, indices, embedding, gains, old_forces, eta,
-                        late ? post_exaggeration_momentum : pre_exaggeration_momentum,
-                        late ? 1.0f : early_exaggeration, slot, normalization, s))
-            return 1;
-    }
+    if (normalization && launch_finish_z(plan, normalization, s)) return 1;
     if (profile_mark(plan, -1, s)) return 1;
     TSNE_TRY(hipEventRecord(plan->leave_event, s));
     TSNE_TRY(hipStreamWaitEvent(caller, plan->leave_event, 0));

@@ -299,7 +299,7 @@ class Plan(object):
 
     def iterate_(self, pij, idx, embedding, gains, old_forces, step_begin, step_end, force_magnify_iters=250,
                  eta=200.0, pre_momentum=0.5, post_momentum=0.8, early_exaggeration=12.0):
-        z = torch.zeros(1, dtype=torch.float32, device=self.device)
+        z = torch.empty(1, dtype=torch.float32, device=self.device)  # written by the call
         _check(lib().tsne_hip_iterate(self._h, _ptr(None if pij is None else _f32(pij)), _ptr(idx),
                                       _ptr(_f32(embedding)),
                                       _ptr(_f32(gains)), _ptr(_f32(old_forces)), step_begin, step_end,
