@@ -435,7 +435,13 @@ def test_grid_size_changes_between_steps(stages, c0_problem):
         rep_o, z_o, w_o, yt_o, phi_o = oracle.repulsive(y, nb=nb, details=True)
         assert w.shape == w_o.shape
         assert rel_l2(rep.cpu().numpy(), rep_o) <= 1e-4, nb
-        assert abs(float(z) - z_o) <= 1e-5 * abs(z_o), nb
+        # At this spread z_i = (1 + r^2) phi_1 - 2 (x phi_2 + y phi_3) + phi_4 cancels some forty-fold, and the fp32
+        # transforms leave 1e-7 (phi_1..3) to 1e-6 (phi_4) of a plane's norm against the oracle's double-precision
+        # convolution: Z lands 1e-6 to 2e-5 from the oracle's, whichever transform length the grid gets (it enters
+        # the repulsive gradient, whose bar is 1e-4, as a factor).
+        assert abs(float(z) - z_o) <= 3e-5 * abs(z_o), nb
+        assert max(np.abs(yt.cpu().numpy().reshape(-1, 4)[:, t] - np.asarray(yt_o).reshape(-1, 4)[:, t]).max() /
+                   np.abs(np.asarray(yt_o).reshape(-1, 4)[:, t]).max() for t in range(4)) <= 5e-6, nb
     dP, di = dev(c["P"]), dev(c["idx"])
     plan.prepare_attractive(dP, di)
     y0 = c["y0"]

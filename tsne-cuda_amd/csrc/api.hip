@@ -387,6 +387,7 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     (void)hipFree(p->col_results);
     (void)hipFree(p->kernel_rows);
     (void)hipFree(p->twiddles);
+    (void)hipFree(p->twiddles_short);
     (void)hipFree(p->scalars);
     (void)hipFree(p->attr);
     (void)hipFree(p->rep);
@@ -462,16 +463,23 @@ int tsne_hip_plan_create(tsne_hip_plan **plan, int num_points, int num_neighbors
               hipMalloc(&p->col_results, sizeof(float2) * spec) == hipSuccess &&
               hipMalloc(&p->kernel_rows, sizeof(float) * (size_t)(kFft / 2 + 1) * kNodePad) == hipSuccess &&
               hipMalloc(&p->twiddles, sizeof(float2) * kFft) == hipSuccess &&
+              hipMalloc(&p->twiddles_short, sizeof(float2) * kFftShort) == hipSuccess &&
               hipMalloc(&p->scalars, sizeof(LoopScalars)) == hipSuccess &&
               hipMalloc(&p->attr, sizeof(float) * 2 * N) == hipSuccess &&
               hipMalloc(&p->rep, sizeof(float) * 2 * N) == hipSuccess;
     if (ok) {
-        std::vector<float2> tw(kFft);
+        std::vector<float2> tw(kFft), tws(kFftShort);
         for (int k = 0; k < kFft; ++k) {
             const double ang = -2.0 * M_PI * (double)k / (double)kFft;
             tw[k] = make_float2((float)std::cos(ang), (float)std::sin(ang));
         }
+        for (int k = 0; k < kFftShort; ++k) {
+            const double ang = -2.0 * M_PI * (double)k / (double)kFftShort;
+            tws[k] = make_float2((float)std::cos(ang), (float)std::sin(ang));
+        }
         ok = hipMemcpy(p->twiddles, tw.data(), sizeof(float2) * kFft, hipMemcpyHostToDevice) == hipSuccess &&
+             hipMemcpy(p->twiddles_short, tws.data(), sizeof(float2) * kFftShort, hipMemcpyHostToDevice) ==
+                 hipSuccess &&
              hipMemset(p->yxy, 0, sizeof(float2) * (N + 2)) == hipSuccess &&
              hipMemset(p->box_moments, 0, moment_bytes) == hipSuccess &&
              hipMemset(p->centre_parts, 0, sizeof(double2) * 2 * kMaxCentreParts) == hipSuccess &&

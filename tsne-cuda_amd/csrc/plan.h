@@ -11,6 +11,7 @@ namespace tsnehip {
 constexpr int kInterp = 3;        // interpolation nodes per box and dimension (src/fit_tsne.cu:248)
 constexpr int kTerms = 4;         // charges per point (src/fit_tsne.cu:254)
 constexpr int kFft = 1024;        // padded transform length, >= 2 * 3 * n_boxes - 1
+constexpr int kFftShort = 800;    // ... and the one used where it is enough: up to 133 boxes (400 nodes) per side
 constexpr int kNodePad = 512;     // leading dimension of the transposed spectra (>= nodes per dim)
 constexpr int kMaxBoxes = 170;    // 3 * 170 = 510 nodes <= kNodePad
 constexpr int kTileBoxes = 5;     // boxes per side of a spreading tile (25 boxes x 21 moments x 8 B = 4.2 KB of LDS;
@@ -87,6 +88,7 @@ struct tsne_hip_plan {
     float2 *col_results = nullptr;      // same shape
     float *kernel_rows = nullptr;       // (kFft/2+1) x kNodePad: row spectra of the Cauchy kernel
     float2 *twiddles = nullptr;         // kFft roots of unity
+    float2 *twiddles_short = nullptr;   // kFftShort roots of unity
     tsnehip::LoopScalars *scalars = nullptr;
     float *attr = nullptr;  // 2N, used by tsne_hip_iterate
     float *rep = nullptr;   // 2N

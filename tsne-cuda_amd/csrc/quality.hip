@@ -49,7 +49,7 @@ struct DeviceArray {
 };
 
 constexpr int kTrustThreads = 256;
-constexpr int kTrustMaxSample = 8192;  // two float arrays of that many entries in LDS
+constexpr int kTrustMaxSample = 8192;  // two 8-byte arrays of that many entries in LDS
 
 // Block-wide reductions over kTrustThreads threads (red: kTrustThreads / kWave slots of LDS).
 __device__ __forceinline__ unsigned long long block_min_key(unsigned long long v, unsigned long long *red) {
@@ -78,58 +78,62 @@ __device__ __forceinline__ int block_sum_int(int v, int *red) {
     return r;
 }
 
-// Non-negative floats order like their bit patterns: (distance, index) as one 64-bit key.
-__device__ __forceinline__ unsigned long long dist_key(float d, int j) {
-    return ((unsigned long long)__float_as_uint(d) << 32) | (unsigned int)j;
+// Non-negative doubles order like their bit patterns; ties go to the lower index.
+__device__ __forceinline__ bool key_less(unsigned long long da, int ja, unsigned long long db, int jb) {
+    return da < db || (da == db && ja < jb);
 }
 
 // One workgroup per sampled point i.  xt: the sample's points, dimension-major (D x M); emb: the sample's
 // embedding, M xs then M ys.  For each of the n_neighbors nearest points of i in the embedding (by
 // (distance, index), i excluded) the rank of that point among i's input-space neighbours (1 = nearest) minus
 // n_neighbors, where positive, goes into *penalty: the sum in the definition of trustworthiness
-// (Venna & Kaski; scikit-learn's sklearn.manifold.trustworthiness computes the same sum).
+// (Venna & Kaski; scikit-learn's sklearn.manifold.trustworthiness computes the same sum).  Squared distances
+// are taken in double on the float coordinates (differences and their squares are then exact, the sums rounded
+// at 1e-16), so that which point is the n-th neighbour does not hang on fp32 rounding: one point more or less
+// among the nearest moves the sum by its whole rank.
 __global__ __launch_bounds__(kTrustThreads) void trustworthiness_kernel(const float *__restrict__ xt,
                                                                         const float *__restrict__ emb, int M, int D,
                                                                         int n_neighbors,
                                                                         unsigned long long *__restrict__ penalty) {
 #pragma clang fp contract(off)
-    extern __shared__ float lds[];
-    float *d_in = lds, *d_emb = lds + M;
+    extern __shared__ unsigned long long lds[];
+    unsigned long long *d_in = lds, *d_emb = lds + M;  // bit patterns of the squared distances
     __shared__ unsigned long long red_key[kTrustThreads / kWave];
     __shared__ int red_int[kTrustThreads / kWave];
     const int i = blockIdx.x;
-    const float ex = emb[i], ey = emb[M + i];
+    const double ex = emb[i], ey = emb[M + i];
     for (int j = threadIdx.x; j < M; j += kTrustThreads) {
-        float acc = 0.0f;
+        double acc = 0.0;
         for (int d = 0; d < D; ++d) {
-            const float df = xt[(size_t)d * M + i] - xt[(size_t)d * M + j];
-            acc = fmaf(df, df, acc);
+            const double df = (double)xt[(size_t)d * M + i] - (double)xt[(size_t)d * M + j];
+            acc += df * df;
         }
-        d_in[j] = acc;
-        const float dx = ex - emb[j], dy = ey - emb[M + j];
-        d_emb[j] = dx * dx + dy * dy;
+        d_in[j] = (unsigned long long)__double_as_longlong(acc);
+        const double dx = ex - (double)emb[j], dy = ey - (double)emb[M + j];
+        d_emb[j] = (unsigned long long)__double_as_longlong(dx * dx + dy * dy);
     }
     __syncthreads();
-    unsigned long long last = 0ull;  // keys are > 0 for every j != i that matters (index part breaks ties)
-    bool first = true;
+    unsigned long long last_d = 0ull;
+    int last_j = -1;  // nothing taken yet: every (distance, index) lies above (0, -1)
     unsigned long long total = 0ull;
     for (int round = 0; round < n_neighbors; ++round) {
-        // the smallest embedding key above the one taken last
+        // the smallest embedding (distance, index) above the one taken last: the distance, then the index
         unsigned long long best = ~0ull;
-        for (int j = threadIdx.x; j < M; j += kTrustThreads) {
-            if (j == i) continue;
-            const unsigned long long key = dist_key(d_emb[j], j);
-            if ((first || key > last) && key < best) best = key;
-        }
+        for (int j = threadIdx.x; j < M; j += kTrustThreads)
+            if (j != i && key_less(last_d, last_j, d_emb[j], j) && d_emb[j] < best) best = d_emb[j];
         best = block_min_key(best, red_key);
         if (best == ~0ull) break;
-        last = best;
-        first = false;
-        const int j = (int)(unsigned int)(best & 0xffffffffull);
-        const unsigned long long in_key = dist_key(d_in[j], j);
+        unsigned long long best_j = ~0ull;
+        for (int j = threadIdx.x; j < M; j += kTrustThreads)
+            if (j != i && d_emb[j] == best && key_less(last_d, last_j, best, j) && (unsigned long long)j < best_j)
+                best_j = (unsigned long long)j;
+        const int j = (int)block_min_key(best_j, red_key);
+        last_d = best;
+        last_j = j;
+        const unsigned long long in_d = d_in[j];
         int closer = 0;
         for (int l = threadIdx.x; l < M; l += kTrustThreads)
-            if (l != i && dist_key(d_in[l], l) < in_key) closer += 1;
+            if (l != i && key_less(d_in[l], l, in_d, j)) closer += 1;
         const int rank = block_sum_int(closer, red_int) + 1;
         if (rank > n_neighbors) total += (unsigned long long)(rank - n_neighbors);
     }
@@ -285,7 +289,7 @@ extern "C" int tsnecuda_trustworthiness(const float *points, const float *embedd
     TSNE_TRY(hipMemcpy(d_xt.ptr, xt.data(), sizeof(float) * xt.size(), hipMemcpyHostToDevice));
     TSNE_TRY(hipMemcpy(d_emb.ptr, emb.data(), sizeof(float) * emb.size(), hipMemcpyHostToDevice));
     TSNE_TRY(hipMemset(d_pen.ptr, 0, sizeof(unsigned long long)));
-    const size_t lds = sizeof(float) * 2 * (size_t)M;
+    const size_t lds = sizeof(unsigned long long) * 2 * (size_t)M;
     TSNE_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(trustworthiness_kernel),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     trustworthiness_kernel<<<M, kTrustThreads, lds, nullptr>>>(d_xt.as<float>(), d_emb.as<float>(), M, num_dims,

@@ -124,20 +124,161 @@ __device__ __forceinline__ void radix4_pass(float2 *s, int nfft, int log2L, cons
     }
 }
 
-__device__ __forceinline__ void fft_forward(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+// Grids of up to 400 nodes per side (133 boxes; the default 130 gives 390) need 799 points of padding, and get
+// transforms of 800 = 8 * 10 * 10 points: 0.61 of the 1024 x 1024 transform's points, in three in-place passes
+// (forwards: radix 8 over the whole transform, radix 10 over its eight parts of 100, radix 10 over the tens);
+// position p = 100 j1 + 10 j2 + j3 then holds frequency j1 + 8 j2 + 80 j3, and the inverse runs the same passes
+// backwards.  Plain layout, no swizzle.
+template <int R, bool INVERSE>
+__device__ __forceinline__ void small_dft(float2 (&x)[R]) {
+    if constexpr (R == 2) {
+        const float2 a = x[0], b = x[1];
+        x[0] = cadd(a, b);
+        x[1] = csub(a, b);
+    } else if constexpr (R == 4) {
+        const float2 t0 = cadd(x[0], x[2]), t1 = csub(x[0], x[2]), t2 = cadd(x[1], x[3]), t3 = csub(x[1], x[3]);
+        x[0] = cadd(t0, t2);
+        x[2] = csub(t0, t2);
+        if (!INVERSE) {
+            x[1] = make_float2(t1.x + t3.y, t1.y - t3.x);
+            x[3] = make_float2(t1.x - t3.y, t1.y + t3.x);
+        } else {
+            x[1] = make_float2(t1.x - t3.y, t1.y + t3.x);
+            x[3] = make_float2(t1.x + t3.y, t1.y - t3.x);
+        }
+    } else if constexpr (R == 8) {
+        // Even and odd elements as two transforms of four, then w8^k = exp(-+ i pi k / 4) on the odd half.
+        float2 e[4] = {x[0], x[2], x[4], x[6]}, o[4] = {x[1], x[3], x[5], x[7]};
+        small_dft<4, INVERSE>(e);
+        small_dft<4, INVERSE>(o);
+        constexpr float h = 0.70710678118654752f;
+        const float sg = INVERSE ? -1.0f : 1.0f;  // forwards: w8 = (1 - i) / sqrt 2
+        const float2 o1 = make_float2(h * (o[1].x + sg * o[1].y), h * (o[1].y - sg * o[1].x));
+        const float2 o2 = make_float2(sg * o[2].y, -sg * o[2].x);
+        const float2 o3 = make_float2(h * (-o[3].x + sg * o[3].y), h * (-o[3].y - sg * o[3].x));
+        x[0] = cadd(e[0], o[0]);
+        x[4] = csub(e[0], o[0]);
+        x[1] = cadd(e[1], o1);
+        x[5] = csub(e[1], o1);
+        x[2] = cadd(e[2], o2);
+        x[6] = csub(e[2], o2);
+        x[3] = cadd(e[3], o3);
+        x[7] = csub(e[3], o3);
+    } else if constexpr (R == 10) {
+        // Even and odd elements as two transforms of five, then w10^k = exp(-+ i pi k / 5) on the odd half.
+        float2 e[5] = {x[0], x[2], x[4], x[6], x[8]}, o[5] = {x[1], x[3], x[5], x[7], x[9]};
+        small_dft<5, INVERSE>(e);
+        small_dft<5, INVERSE>(o);
+        constexpr float wr[5] = {1.0f, 0.80901699437494745f, 0.30901699437494745f, -0.30901699437494745f,
+                                 -0.80901699437494745f};
+        constexpr float wi[5] = {0.0f, 0.58778525229247314f, 0.95105651629515353f, 0.95105651629515353f,
+                                 0.58778525229247314f};  // -Im w10^k forwards
 #pragma unroll
-    for (int l = kLog2Fft; l >= 2; l -= 2) {
-        radix4_pass<false>(s, nfft, l, tw, tid, nthreads);
-        __syncthreads();
+        for (int k = 0; k < 5; ++k) {
+            const float2 w = make_float2(wr[k], INVERSE ? wi[k] : -wi[k]);
+            const float2 t = k == 0 ? o[0] : cmul(o[k], w);
+            x[k] = cadd(e[k], t);
+            x[k + 5] = csub(e[k], t);
+        }
+    } else {
+        static_assert(R == 5, "radix");
+        // cos(2 pi / 5) and cos(4 pi / 5) are -1/4 +- sqrt(5)/4: written so, the part of an output that cancels for
+        // smooth data carries exact coefficients, and the rounded constant meets a difference only.
+        constexpr float r5 = 0.55901699437494742f;                               // sqrt(5) / 4
+        constexpr float s1 = 0.95105651629515353f, s2 = 0.58778525229247314f;   // sin(2 pi / 5), sin(4 pi / 5)
+        const float2 t1 = cadd(x[1], x[4]), t2 = cadd(x[2], x[3]), t3 = csub(x[1], x[4]), t4 = csub(x[2], x[3]);
+        const float2 t5 = cadd(t1, t2);
+        const float2 m0 = make_float2(x[0].x - 0.25f * t5.x, x[0].y - 0.25f * t5.y);
+        const float2 t6 = make_float2(r5 * (t1.x - t2.x), r5 * (t1.y - t2.y));
+        const float2 a1 = cadd(m0, t6), a2 = csub(m0, t6);
+        float2 b1 = make_float2(s1 * t3.x + s2 * t4.x, s1 * t3.y + s2 * t4.y);
+        float2 b2 = make_float2(s2 * t3.x - s1 * t4.x, s2 * t3.y - s1 * t4.y);
+        if (INVERSE) {
+            b1 = make_float2(-b1.x, -b1.y);
+            b2 = make_float2(-b2.x, -b2.y);
+        }
+        x[0] = cadd(x[0], t5);
+        x[1] = make_float2(a1.x + b1.y, a1.y - b1.x);  // a1 - i b1
+        x[4] = make_float2(a1.x - b1.y, a1.y + b1.x);
+        x[2] = make_float2(a2.x + b2.y, a2.y - b2.x);
+        x[3] = make_float2(a2.x - b2.y, a2.y + b2.x);
     }
 }
-__device__ __forceinline__ void fft_inverse(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+
+// One pass of radix R over the sub-transforms of length L of `nfft` transforms of N points, N slots apart:
+// decimation in frequency forwards (twiddles after the sums), decimation in time for the inverse.
+template <int N, int L, int R, bool INVERSE>
+__device__ __forceinline__ void mixed_pass(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+    constexpr int Q = L / R, B = N / R, STRIDE = N / L;
+    for (int id = tid; id < nfft * B; id += nthreads) {
+        const int f = id / B, q = id - f * B;
+        const int b = q / Q, k = q - b * Q;
+        float2 *base = s + f * N + b * L + k;
+        float2 x[R];
 #pragma unroll
-    for (int l = 2; l <= kLog2Fft; l += 2) {
-        radix4_pass<true>(s, nfft, l, tw, tid, nthreads);
-        __syncthreads();
+        for (int j = 0; j < R; ++j) x[j] = base[j * Q];
+        if constexpr (INVERSE && Q > 1) {
+#pragma unroll
+            for (int j = 1; j < R; ++j) x[j] = cmul_conj(x[j], tw[j * k * STRIDE]);
+        }
+        small_dft<R, INVERSE>(x);
+        if constexpr (!INVERSE && Q > 1) {
+#pragma unroll
+            for (int j = 1; j < R; ++j) x[j] = cmul(x[j], tw[j * k * STRIDE]);
+        }
+#pragma unroll
+        for (int j = 0; j < R; ++j) base[j * Q] = x[j];
     }
+    __syncthreads();
 }
+
+// What the convolution's kernels need of a transform length: the slot of element i within a transform's N LDS
+// slots, the frequency held at a position of the forward transform's output, and the transforms themselves
+// (every pass ends with a barrier).
+template <int N>
+struct Transform;
+
+template <>
+struct Transform<kFft> {
+    static __device__ __forceinline__ int slot(int i) { return pad(i); }
+    static __device__ __forceinline__ int frequency(int pos) { return rev4(pos); }
+    static __device__ __forceinline__ void forward(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+#pragma unroll
+        for (int l = kLog2Fft; l >= 2; l -= 2) {
+            radix4_pass<false>(s, nfft, l, tw, tid, nthreads);
+            __syncthreads();
+        }
+    }
+    static __device__ __forceinline__ void inverse(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+#pragma unroll
+        for (int l = 2; l <= kLog2Fft; l += 2) {
+            radix4_pass<true>(s, nfft, l, tw, tid, nthreads);
+            __syncthreads();
+        }
+    }
+};
+
+template <>
+struct Transform<kFftShort> {
+    static constexpr int N = kFftShort;
+    static_assert(N == 800, "the passes below factor 800");
+    static __device__ __forceinline__ int slot(int i) { return i; }
+    static __device__ __forceinline__ int frequency(int pos) {
+        const int j1 = pos / 100, r1 = pos - j1 * 100;
+        const int j2 = r1 / 10, j3 = r1 - j2 * 10;
+        return j1 + 8 * j2 + 80 * j3;
+    }
+    static __device__ __forceinline__ void forward(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+        mixed_pass<N, 800, 8, false>(s, nfft, tw, tid, nthreads);
+        mixed_pass<N, 100, 10, false>(s, nfft, tw, tid, nthreads);
+        mixed_pass<N, 10, 10, false>(s, nfft, tw, tid, nthreads);
+    }
+    static __device__ __forceinline__ void inverse(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+        mixed_pass<N, 10, 10, true>(s, nfft, tw, tid, nthreads);
+        mixed_pass<N, 100, 10, true>(s, nfft, tw, tid, nthreads);
+        mixed_pass<N, 800, 8, true>(s, nfft, tw, tid, nthreads);
+    }
+};
 
 struct Bounds {
     float lo, box_width, h;
@@ -663,34 +804,35 @@ __device__ __forceinline__ float kernel_value(float lo, float h, int a, int b) {
 }
 
 // Kernel values of 4 * PAIRS rows of the grid (two rows packed into one complex transform) and their transforms.
-template <int THREADS, int PAIRS>
+template <int THREADS, int PAIRS, int NFFT>
 __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *sc, int slot, int n_boxes,
                                                   const float2 *__restrict__ tw, float *__restrict__ kernel_rows,
-                                                  float2 (*s)[kFftPad]) {
+                                                  float2 (*s)[NFFT]) {
+    using T = Transform<NFFT>;
     constexpr int kTransforms = 2 * PAIRS;
     const int tid = threadIdx.x;
     const int G = n_boxes * kInterp;
     const Bounds bd = load_bounds(sc, slot, n_boxes);
     const int a0 = block * 2 * kTransforms;
-    for (int e = tid; e < kTransforms * kFft; e += THREADS) {
-        const int f = e >> kLog2Fft, m = e & (kFft - 1);
-        const int b = m < kFft / 2 ? m : kFft - m;
+    for (int e = tid; e < kTransforms * NFFT; e += THREADS) {
+        const int f = e / NFFT, m = e - f * NFFT;
+        const int b = m < NFFT / 2 ? m : NFFT - m;
         const int ra = a0 + 2 * f;
         float2 v = make_float2(0.f, 0.f);
         if (b < G) {
             if (ra < G) v.x = kernel_value(bd.lo, bd.h, ra, b);
             if (ra + 1 < G) v.y = kernel_value(bd.lo, bd.h, ra + 1, b);
         }
-        s[f][pad(m)] = v;
+        s[f][T::slot(m)] = v;
     }
     __syncthreads();
-    fft_forward(&s[0][0], kTransforms, tw, tid, THREADS);
-    for (int e = tid; e < kTransforms * kFft; e += THREADS) {
-        const int f = e >> kLog2Fft, pos = e & (kFft - 1);
-        const int v = rev4(pos);
+    T::forward(&s[0][0], kTransforms, tw, tid, THREADS);
+    for (int e = tid; e < kTransforms * NFFT; e += THREADS) {
+        const int f = e / NFFT, pos = e - f * NFFT;
+        const int v = T::frequency(pos);
         const int ra = a0 + 2 * f;
-        if (v <= kFft / 2 && ra < kNodePad) {
-            const float2 val = s[f][pad(pos)];
+        if (v <= NFFT / 2 && ra < kNodePad) {
+            const float2 val = s[f][T::slot(pos)];
             *reinterpret_cast<float2 *>(kernel_rows + (size_t)v * kNodePad + ra) = val;
         }
     }
@@ -709,7 +851,7 @@ __device__ __forceinline__ void kernel_rows_block(int block, const LoopScalars *
 // provided those are in one piece (the loop enqueues the attractive kernel first for that reason).  One row per
 // workgroup (256 threads, 16 KB) measured 21 us against 17 us alone and 2 % fewer iterations per second.
 // ---------------------------------------------------------------------------
-template <int ROWS>
+template <int ROWS, int NFFT>
 __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(const unsigned long long *__restrict__ moments,
                                                                        double from_fixed, LagrangeMonomials mono,
                                                                        float4 *__restrict__ charges_out, int G,
@@ -717,8 +859,9 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(const uns
                                                                        const float2 *__restrict__ twiddles,
                                                                        float2 *__restrict__ row_spectra,
                                                                        float *__restrict__ kernel_rows) {
+    using T = Transform<NFFT>;
     constexpr int kThreads = 256 * ROWS;
-    __shared__ float2 s[2 * ROWS][kFftPad];  // [row * 2 + pair]
+    __shared__ float2 s[2 * ROWS][NFFT];  // [row * 2 + pair]
     const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     // The workgroups past the rows produce the kernel's row spectra (needed by the column
@@ -726,7 +869,7 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(const uns
     const int row_blocks = (G + ROWS - 1) / ROWS;
     const int launched = kXcds * ((row_blocks + kXcds - 1) / kXcds);
     if ((int)blockIdx.x >= launched) {
-        kernel_rows_block<kThreads, ROWS>(blockIdx.x - launched, sc, slot, n_boxes, tw, kernel_rows, s);
+        kernel_rows_block<kThreads, ROWS, NFFT>(blockIdx.x - launched, sc, slot, n_boxes, tw, kernel_rows, s);
         return;
     }
     const int row_block = xcd_row_block(blockIdx.x, row_blocks);
@@ -734,8 +877,8 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(const uns
     const int m0 = row_block * ROWS;
     const float s3 = r2_plane_scale(sc, slot);
     const Bounds bd = load_bounds(sc, slot, n_boxes);
-    for (int e = tid; e < ROWS * kFft; e += kThreads) {
-        const int r = e >> kLog2Fft, n = e & (kFft - 1);
+    for (int e = tid; e < ROWS * NFFT; e += kThreads) {
+        const int r = e / NFFT, n = e - r * NFFT;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (n < G && m0 + r < G) {
             const int gx = m0 + r;
@@ -772,19 +915,19 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(const uns
             }
             if (charges_out) charges_out[(size_t)gx * G + n] = v;
         }
-        s[r * 2 + 0][pad(n)] = make_float2(v.x, v.w * s3);  // planes 1 and r^2 / m^2
-        s[r * 2 + 1][pad(n)] = make_float2(v.y, v.z);       // planes x and y
+        s[r * 2 + 0][T::slot(n)] = make_float2(v.x, v.w * s3);  // planes 1 and r^2 / m^2
+        s[r * 2 + 1][T::slot(n)] = make_float2(v.y, v.z);       // planes x and y
     }
     __syncthreads();
-    fft_forward(&s[0][0], 2 * ROWS, tw, tid, kThreads);
-    for (int e = tid; e < 2 * kFft; e += kThreads) {
-        const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
-        float2 *dst = row_spectra + ((size_t)pair * kFft + pos) * kNodePad + m0;
+    T::forward(&s[0][0], 2 * ROWS, tw, tid, kThreads);
+    for (int e = tid; e < 2 * NFFT; e += kThreads) {
+        const int pair = e / NFFT, pos = e - pair * NFFT;
+        float2 *dst = row_spectra + ((size_t)pair * NFFT + pos) * kNodePad + m0;
         if (ROWS == 2) {
-            const float2 r0 = s[0 + pair][pad(pos)], r1 = s[2 + pair][pad(pos)];
+            const float2 r0 = s[0 + pair][T::slot(pos)], r1 = s[2 + pair][T::slot(pos)];
             *reinterpret_cast<float4 *>(dst) = make_float4(r0.x, r0.y, r1.x, r1.y);
         } else {
-            *dst = s[pair][pad(pos)];
+            *dst = s[pair][T::slot(pos)];
         }
     }
 }
@@ -803,7 +946,7 @@ __global__ __launch_bounds__(256 * ROWS) void conv_rows_forward_kernel(const uns
 // the same two positions of every transform), so the workgroup holds four transforms: 32 KB, the 26 allocation
 // units of LDS that fit beside a workgroup of the attractive kernel (27 free), where 40 KB do not.  The extra pass
 // has work for half the threads and costs 1.5 us alone.
-template <bool SLIM>
+template <bool SLIM, int NFFT>
 __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restrict__ row_spectra, int G,
                                                            const float *__restrict__ kernel_rows,
                                                            const float2 *__restrict__ twiddles,
@@ -816,58 +959,62 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
     constexpr int kPairsInFlight = 2;
     constexpr int kData = 2 * kPairsInFlight;  // transforms of data per round
     constexpr int kKernelSlot = SLIM ? 0 : kData;
-    __shared__ float2 s[SLIM ? kData : kData + 1][kFftPad];
+    using T = Transform<NFFT>;
+    static_assert(!SLIM || NFFT == 2 * 512, "the slim form keeps positions tid and tid + 512 of the kernel's spectrum");
+    __shared__ float2 s[SLIM ? kData : kData + 1][NFFT];
     const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int c0 = blockIdx.x * 2;
     {
-        int v0 = rev4(c0), v1 = rev4(c0 + 1);
-        v0 = min(v0, kFft - v0);
-        v1 = min(v1, kFft - v1);
-        for (int m = tid; m < kFft; m += 512) {
-            const int a = m < kFft / 2 ? m : kFft - m;
+        int v0 = T::frequency(c0), v1 = T::frequency(c0 + 1);
+        v0 = min(v0, NFFT - v0);
+        v1 = min(v1, NFFT - v1);
+        for (int m = tid; m < NFFT; m += 512) {
+            const int a = m < NFFT / 2 ? m : NFFT - m;
             float2 v = make_float2(0.f, 0.f);
             if (a < G) {
                 v.x = kernel_rows[(size_t)v0 * kNodePad + a];
                 v.y = kernel_rows[(size_t)v1 * kNodePad + a];
             }
-            s[kKernelSlot][pad(m)] = v;
+            s[kKernelSlot][T::slot(m)] = v;
         }
     }
     float2 kk_reg[2] = {make_float2(0.f, 0.f), make_float2(0.f, 0.f)};  // SLIM: the kernel's spectrum at tid, tid + 512
-    if (SLIM) {
+    if constexpr (SLIM) {
         __syncthreads();
-        fft_forward(&s[0][0], 1, tw, tid, 512);
-        kk_reg[0] = s[0][pad(tid)];
-        kk_reg[1] = s[0][pad(tid + 512)];
+        T::forward(&s[0][0], 1, tw, tid, 512);
+        kk_reg[0] = s[0][T::slot(tid)];
+        kk_reg[1] = s[0][T::slot(tid + 512)];
         __syncthreads();
     }
     for (int pair0 = 0; pair0 < 2; pair0 += kPairsInFlight) {
-        for (int e = tid; e < kData * kFft; e += 512) {
-            const int t = e >> kLog2Fft, m = e & (kFft - 1);  // t = pair in flight * 2 + col
+        for (int e = tid; e < kData * NFFT; e += 512) {
+            const int t = e / NFFT, m = e - t * NFFT;  // t = pair in flight * 2 + col
             float2 v = make_float2(0.f, 0.f);
-            if (m < G) v = row_spectra[((size_t)(pair0 + (t >> 1)) * kFft + c0 + (t & 1)) * kNodePad + m];
-            s[t][pad(m)] = v;
+            if (m < G) v = row_spectra[((size_t)(pair0 + (t >> 1)) * NFFT + c0 + (t & 1)) * kNodePad + m];
+            s[t][T::slot(m)] = v;
         }
         __syncthreads();
         // (SLIM = false: the kernel columns are transformed with the first round)
-        fft_forward(&s[0][0], !SLIM && pair0 == 0 ? kData + 1 : kData, tw, tid, 512);
+        T::forward(&s[0][0], !SLIM && pair0 == 0 ? kData + 1 : kData, tw, tid, 512);
 #pragma unroll
-        for (int r = 0; r < kData * kFft / 512; ++r) {
+        for (int r = 0; r < (kData * NFFT + 511) / 512; ++r) {
             const int e = tid + r * 512;
-            const int t = e >> kLog2Fft, m = e & (kFft - 1);  // (m = tid + 512 (r & 1))
-            const float2 kk = SLIM ? kk_reg[r & 1] : s[kKernelSlot][pad(m)];
+            if (kData * NFFT % 512 != 0 && e >= kData * NFFT) break;
+            const int t = e / NFFT, m = e - t * NFFT;  // (1024 points: m = tid + 512 (r & 1))
+            const float2 kk = SLIM ? kk_reg[r & 1] : s[kKernelSlot][T::slot(m)];
             const float kv = (t & 1) ? kk.y : kk.x;
-            float2 v = s[t][pad(m)];
+            float2 v = s[t][T::slot(m)];
             v.x *= kv;
             v.y *= kv;
-            s[t][pad(m)] = v;
+            s[t][T::slot(m)] = v;
         }
         __syncthreads();
-        fft_inverse(&s[0][0], kData, tw, tid, 512);
-        for (int e = tid; e < kData * kFft; e += 512) {
-            const int t = e >> kLog2Fft, m = e & (kFft - 1);
-            if (m < G) col_results[((size_t)(pair0 + (t >> 1)) * kFft + c0 + (t & 1)) * kNodePad + m] = s[t][pad(m)];
+        T::inverse(&s[0][0], kData, tw, tid, 512);
+        for (int e = tid; e < kData * NFFT; e += 512) {
+            const int t = e / NFFT, m = e - t * NFFT;
+            if (m < G)
+                col_results[((size_t)(pair0 + (t >> 1)) * NFFT + c0 + (t & 1)) * kNodePad + m] = s[t][T::slot(m)];
         }
         __syncthreads();
     }
@@ -877,31 +1024,33 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
 // Inverse row pass for x nodes m0, m0+1: consumes digit-reversed positions,
 // produces node potentials in natural order, scaled by 1/1024^2.
 // ---------------------------------------------------------------------------
+template <int NFFT>
 __global__ __launch_bounds__(kRowThreads) void conv_rows_inverse_kernel(const float2 *__restrict__ col_results, int G,
                                                                 const LoopScalars *sc, int slot,
                                                                 const float2 *__restrict__ twiddles,
                                                                 float4 *__restrict__ node_potentials) {
-    __shared__ float2 s[4][kFftPad];  // [row * 2 + pair]
+    using T = Transform<NFFT>;
+    __shared__ float2 s[4][NFFT];  // [row * 2 + pair]
     const float2 *tw = twiddles;
     const int tid = threadIdx.x;
     const int row_block = xcd_row_block(blockIdx.x, (G + 1) / 2);
     if (row_block < 0) return;
     const int m0 = row_block * 2;
-    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
-        const int pair = e >> kLog2Fft, pos = e & (kFft - 1);
+    for (int e = tid; e < 2 * NFFT; e += kRowThreads) {
+        const int pair = e / NFFT, pos = e - pair * NFFT;
         const float4 v =
-            *reinterpret_cast<const float4 *>(col_results + ((size_t)pair * kFft + pos) * kNodePad + m0);
-        s[0 + pair][pad(pos)] = make_float2(v.x, v.y);
-        s[2 + pair][pad(pos)] = make_float2(v.z, v.w);
+            *reinterpret_cast<const float4 *>(col_results + ((size_t)pair * NFFT + pos) * kNodePad + m0);
+        s[0 + pair][T::slot(pos)] = make_float2(v.x, v.y);
+        s[2 + pair][T::slot(pos)] = make_float2(v.z, v.w);
     }
     __syncthreads();
-    fft_inverse(&s[0][0], 4, tw, tid, kRowThreads);
-    const float scale = 1.0f / ((float)kFft * (float)kFft);
+    T::inverse(&s[0][0], 4, tw, tid, kRowThreads);
+    const float scale = 1.0f / ((float)NFFT * (float)NFFT);
     const float scale3 = scale / r2_plane_scale(sc, slot);
-    for (int e = tid; e < 2 * kFft; e += kRowThreads) {
-        const int r = e >> kLog2Fft, n = e & (kFft - 1);
+    for (int e = tid; e < 2 * NFFT; e += kRowThreads) {
+        const int r = e / NFFT, n = e - r * NFFT;
         if (n < G && m0 + r < G) {
-            const float2 p0 = s[r * 2 + 0][pad(n)], p1 = s[r * 2 + 1][pad(n)];
+            const float2 p0 = s[r * 2 + 0][T::slot(n)], p1 = s[r * 2 + 1][T::slot(n)];
             node_potentials[(size_t)(m0 + r) * G + n] =
                 make_float4(p0.x * scale, p1.x * scale, p1.y * scale, p0.y * scale3);
         }
@@ -1040,24 +1189,43 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
                                                            p->num_chunks, p->scalars, slot, slot ^ 1, nb,
                                                            p->moment_scale, p->box_moments, keep);
     TSNE_LAUNCHED(s);
+    // Transform length: 800 points where the padded grid (2 G - 1) fits, else 1024 (TSNE_FFT=1024 forces the latter).
+    static const bool long_only = getenv("TSNE_FFT") && atoi(getenv("TSNE_FFT")) == kFft;
+    const bool short_fft = 2 * G - 1 <= kFftShort && !long_only;
+    const int row_grid = xcd_launch_blocks(div_up(G, 2));
+    const double from_fixed = 1.0 / p->moment_scale;
+    float4 *charges4 = reinterpret_cast<float4 *>(charges_out);
     if (profile_mark(p, kKernelConvRowsForward, s)) return 1;
-    conv_rows_forward_kernel<2><<<xcd_launch_blocks(div_up(G, 2)) + div_up(G, 8), 512, 0, s>>>(
-        p->box_moments, 1.0 / p->moment_scale, p->monomials, reinterpret_cast<float4 *>(charges_out), G, nb, p->scalars,
-        slot, p->twiddles, p->row_spectra, p->kernel_rows);
+    if (short_fft)
+        conv_rows_forward_kernel<2, kFftShort><<<row_grid + div_up(G, 8), 512, 0, s>>>(
+            p->box_moments, from_fixed, p->monomials, charges4, G, nb, p->scalars, slot, p->twiddles_short,
+            p->row_spectra, p->kernel_rows);
+    else
+        conv_rows_forward_kernel<2, kFft><<<row_grid + div_up(G, 8), 512, 0, s>>>(
+            p->box_moments, from_fixed, p->monomials, charges4, G, nb, p->scalars, slot, p->twiddles, p->row_spectra,
+            p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
     static const int slim_mode = getenv("TSNE_SLIM_COLUMNS") ? atoi(getenv("TSNE_SLIM_COLUMNS")) : -1;
     const bool slim = slim_mode < 0 ? (p->blocked_ready && p->strip_rows >= 1024) : slim_mode == 1;
-    if (slim)
-        conv_columns_kernel<true><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results,
-                                                           p->box_moments, kMoments * nb * nb);
+    const int moment_words = kMoments * nb * nb;
+    if (short_fft)  // (five transforms of 800 points are the 32 KB the slim form exists for)
+        conv_columns_kernel<false, kFftShort><<<kFftShort / 2, 512, 0, s>>>(
+            p->row_spectra, G, p->kernel_rows, p->twiddles_short, p->col_results, p->box_moments, moment_words);
+    else if (slim)
+        conv_columns_kernel<true, kFft><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
+                                                                 p->col_results, p->box_moments, moment_words);
     else
-        conv_columns_kernel<false><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles, p->col_results,
-                                                            p->box_moments, kMoments * nb * nb);
+        conv_columns_kernel<false, kFft><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
+                                                                  p->col_results, p->box_moments, moment_words);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvRowsInverse, s)) return 1;
-    conv_rows_inverse_kernel<<<xcd_launch_blocks(div_up(G, 2)), kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot, p->twiddles,
-                                                          p->node_potentials);
+    if (short_fft)
+        conv_rows_inverse_kernel<kFftShort><<<row_grid, kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot,
+                                                                            p->twiddles_short, p->node_potentials);
+    else
+        conv_rows_inverse_kernel<kFft><<<row_grid, kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot,
+                                                                       p->twiddles, p->node_potentials);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelGather, s)) return 1;
     gather_forces_kernel<<<std::min(div_up(N, 256), 1024), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
