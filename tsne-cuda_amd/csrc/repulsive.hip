@@ -207,16 +207,19 @@ __device__ __forceinline__ void small_dft(float2 (&x)[R]) {
 
 // One pass of radix R over the sub-transforms of length L of `nfft` transforms of N points, N slots apart:
 // decimation in frequency forwards (twiddles after the sums), decimation in time for the inverse.
-template <int N, int L, int R, bool INVERSE>
-__device__ __forceinline__ void mixed_pass(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+// load(f, i) delivers element i of transform f, store(f, i, v) takes it back: the LDS in the middle of a transform,
+// memory at either end of it where a kernel fuses its loads and stores into the first and last pass.
+template <int N, int L, int R, bool INVERSE, class Load, class Store>
+__device__ __forceinline__ void mixed_pass_io(int nfft, const float2 *tw, int tid, int nthreads, Load load,
+                                              Store store) {
     constexpr int Q = L / R, B = N / R, STRIDE = N / L;
     for (int id = tid; id < nfft * B; id += nthreads) {
         const int f = id / B, q = id - f * B;
         const int b = q / Q, k = q - b * Q;
-        float2 *base = s + f * N + b * L + k;
+        const int i0 = b * L + k;
         float2 x[R];
 #pragma unroll
-        for (int j = 0; j < R; ++j) x[j] = base[j * Q];
+        for (int j = 0; j < R; ++j) x[j] = load(f, i0 + j * Q);
         if constexpr (INVERSE && Q > 1) {
 #pragma unroll
             for (int j = 1; j < R; ++j) x[j] = cmul_conj(x[j], tw[j * k * STRIDE]);
@@ -227,8 +230,14 @@ __device__ __forceinline__ void mixed_pass(float2 *s, int nfft, const float2 *tw
             for (int j = 1; j < R; ++j) x[j] = cmul(x[j], tw[j * k * STRIDE]);
         }
 #pragma unroll
-        for (int j = 0; j < R; ++j) base[j * Q] = x[j];
+        for (int j = 0; j < R; ++j) store(f, i0 + j * Q, x[j]);
     }
+}
+template <int N, int L, int R, bool INVERSE>
+__device__ __forceinline__ void mixed_pass(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
+    mixed_pass_io<N, L, R, INVERSE>(
+        nfft, tw, tid, nthreads, [s](int f, int i) { return s[f * N + i]; },
+        [s](int f, int i, float2 v) { s[f * N + i] = v; });
     __syncthreads();
 }
 
@@ -1020,6 +1029,59 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
     }
 }
 
+// The column pass on 800-point transforms, with the ends of the transforms in memory: the first forward pass takes
+// its elements straight from the row spectra (and the kernel's column, the fifth transform, from kernel_rows), the
+// first inverse pass multiplies by the kernel's spectrum as it loads, and the last inverse pass stores the G rows
+// that are wanted: five trips through the LDS per element instead of eight, three barriers fewer.
+__global__ __launch_bounds__(512) void conv_columns_short_kernel(const float2 *__restrict__ row_spectra, int G,
+                                                                 const float *__restrict__ kernel_rows,
+                                                                 const float2 *__restrict__ tw,
+                                                                 float2 *__restrict__ col_results,
+                                                                 unsigned long long *__restrict__ moments,
+                                                                 int moment_words) {
+    constexpr int N = kFftShort;
+    using T = Transform<N>;
+    for (int e = blockIdx.x * 512 + threadIdx.x; e < moment_words; e += gridDim.x * 512) moments[e] = 0ull;
+    __shared__ float2 s[5][N];  // [pair * 2 + col], then the kernel's two columns as one complex transform
+    const int tid = threadIdx.x;
+    const int c0 = blockIdx.x * 2;
+    int v0 = T::frequency(c0), v1 = T::frequency(c0 + 1);
+    v0 = min(v0, N - v0);
+    v1 = min(v1, N - v1);
+    const float *k0 = kernel_rows + (size_t)v0 * kNodePad, *k1 = kernel_rows + (size_t)v1 * kNodePad;
+    auto lds_load = [&](int f, int i) { return s[f][i]; };
+    auto lds_store = [&](int f, int i, float2 v) { s[f][i] = v; };
+    mixed_pass_io<N, 800, 8, false>(
+        5, tw, tid, 512,
+        [&](int f, int m) {
+            float2 v = make_float2(0.f, 0.f);
+            if (f < 4) {
+                if (m < G) v = row_spectra[((size_t)(f >> 1) * N + c0 + (f & 1)) * kNodePad + m];
+            } else {
+                const int a = m < N / 2 ? m : N - m;
+                if (a < G) v = make_float2(k0[a], k1[a]);
+            }
+            return v;
+        },
+        lds_store);
+    __syncthreads();
+    mixed_pass<N, 100, 10, false>(&s[0][0], 5, tw, tid, 512);
+    mixed_pass<N, 10, 10, false>(&s[0][0], 5, tw, tid, 512);
+    mixed_pass_io<N, 10, 10, true>(
+        4, tw, tid, 512,
+        [&](int f, int i) {
+            const float2 kk = s[4][i], v = s[f][i];
+            const float kv = (f & 1) ? kk.y : kk.x;
+            return make_float2(v.x * kv, v.y * kv);
+        },
+        lds_store);
+    __syncthreads();
+    mixed_pass<N, 100, 10, true>(&s[0][0], 4, tw, tid, 512);
+    mixed_pass_io<N, 800, 8, true>(4, tw, tid, 512, lds_load, [&](int f, int m, float2 v) {
+        if (m < G) col_results[((size_t)(f >> 1) * N + c0 + (f & 1)) * kNodePad + m] = v;
+    });
+}
+
 // ---------------------------------------------------------------------------
 // Inverse row pass for x nodes m0, m0+1: consumes digit-reversed positions,
 // produces node potentials in natural order, scaled by 1/1024^2.
@@ -1210,8 +1272,8 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     const bool slim = slim_mode < 0 ? (p->blocked_ready && p->strip_rows >= 1024) : slim_mode == 1;
     const int moment_words = kMoments * nb * nb;
     if (short_fft)  // (five transforms of 800 points are the 32 KB the slim form exists for)
-        conv_columns_kernel<false, kFftShort><<<kFftShort / 2, 512, 0, s>>>(
-            p->row_spectra, G, p->kernel_rows, p->twiddles_short, p->col_results, p->box_moments, moment_words);
+        conv_columns_short_kernel<<<kFftShort / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles_short,
+                                                                p->col_results, p->box_moments, moment_words);
     else if (slim)
         conv_columns_kernel<true, kFft><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
                                                                  p->col_results, p->box_moments, moment_words);
