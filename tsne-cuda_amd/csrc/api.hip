@@ -160,6 +160,7 @@ static bool overlap_active(const tsne_hip_plan *p) {
 // attractive kernel, and lose by the chain's later start (measured: 3-10 % slower from 5000 to 60000 points,
 // even at 200000, 1 % faster at 400000, 4 % at 800000).
 static bool attractive_is_critical(const tsne_hip_plan *p, const float *pij) {
+    if (const char *v = std::getenv("TSNE_ATTRACTIVE_CRITICAL")) return v[0] != '0';
     return !pij && !p->csr_row_ptr && p->blocked_ready && p->strip_rows >= 1024;
 }
 

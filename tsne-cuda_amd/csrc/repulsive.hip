@@ -207,8 +207,9 @@ __device__ __forceinline__ void small_dft(float2 (&x)[R]) {
 
 // One pass of radix R over the sub-transforms of length L of `nfft` transforms of N points, N slots apart:
 // decimation in frequency forwards (twiddles after the sums), decimation in time for the inverse.
-// load(f, i) delivers element i of transform f, store(f, i, v) takes it back: the LDS in the middle of a transform,
-// memory at either end of it where a kernel fuses its loads and stores into the first and last pass.
+// load(f, i, j) delivers element i of transform f (the j-th of its butterfly, a compile-time number once the loop
+// is unrolled), store(f, i, j, v) takes it back: the LDS in the middle of a transform, memory at either end of it
+// where a kernel fuses its loads and stores into the first and last pass.
 template <int N, int L, int R, bool INVERSE, class Load, class Store>
 __device__ __forceinline__ void mixed_pass_io(int nfft, const float2 *tw, int tid, int nthreads, Load load,
                                               Store store) {
@@ -219,7 +220,7 @@ __device__ __forceinline__ void mixed_pass_io(int nfft, const float2 *tw, int ti
         const int i0 = b * L + k;
         float2 x[R];
 #pragma unroll
-        for (int j = 0; j < R; ++j) x[j] = load(f, i0 + j * Q);
+        for (int j = 0; j < R; ++j) x[j] = load(f, i0 + j * Q, j);
         if constexpr (INVERSE && Q > 1) {
 #pragma unroll
             for (int j = 1; j < R; ++j) x[j] = cmul_conj(x[j], tw[j * k * STRIDE]);
@@ -230,14 +231,14 @@ __device__ __forceinline__ void mixed_pass_io(int nfft, const float2 *tw, int ti
             for (int j = 1; j < R; ++j) x[j] = cmul(x[j], tw[j * k * STRIDE]);
         }
 #pragma unroll
-        for (int j = 0; j < R; ++j) store(f, i0 + j * Q, x[j]);
+        for (int j = 0; j < R; ++j) store(f, i0 + j * Q, j, x[j]);
     }
 }
 template <int N, int L, int R, bool INVERSE>
 __device__ __forceinline__ void mixed_pass(float2 *s, int nfft, const float2 *tw, int tid, int nthreads) {
     mixed_pass_io<N, L, R, INVERSE>(
-        nfft, tw, tid, nthreads, [s](int f, int i) { return s[f * N + i]; },
-        [s](int f, int i, float2 v) { s[f * N + i] = v; });
+        nfft, tw, tid, nthreads, [s](int f, int i, int) { return s[f * N + i]; },
+        [s](int f, int i, int, float2 v) { s[f * N + i] = v; });
     __syncthreads();
 }
 
@@ -1030,9 +1031,15 @@ __global__ __launch_bounds__(512) void conv_columns_kernel(const float2 *__restr
 }
 
 // The column pass on 800-point transforms, with the ends of the transforms in memory: the first forward pass takes
-// its elements straight from the row spectra (and the kernel's column, the fifth transform, from kernel_rows), the
-// first inverse pass multiplies by the kernel's spectrum as it loads, and the last inverse pass stores the G rows
-// that are wanted: five trips through the LDS per element instead of eight, three barriers fewer.
+// its elements straight from the row spectra (and the kernel's column from kernel_rows), the first inverse pass
+// multiplies by the kernel's spectrum as it loads, and the last inverse pass stores the G rows that are wanted:
+// five trips through the LDS per element instead of eight, three barriers fewer.
+// SLIM = false: the kernel's two columns ride along as a fifth transform (32000 bytes of LDS).
+// SLIM = true: they are transformed first, alone, and every thread keeps the ten values its butterfly of the
+// first inverse pass multiplies by: four transforms, 25600 bytes, like the row passes - the 20 allocation units
+// of 1280 bytes that are left in one piece on a compute unit that holds a workgroup of the attractive kernel
+// (101 units) and one of the spreading kernel (7), whichever of the two was placed first.
+template <bool SLIM>
 __global__ __launch_bounds__(512) void conv_columns_short_kernel(const float2 *__restrict__ row_spectra, int G,
                                                                  const float *__restrict__ kernel_rows,
                                                                  const float2 *__restrict__ tw,
@@ -1042,42 +1049,65 @@ __global__ __launch_bounds__(512) void conv_columns_short_kernel(const float2 *_
     constexpr int N = kFftShort;
     using T = Transform<N>;
     for (int e = blockIdx.x * 512 + threadIdx.x; e < moment_words; e += gridDim.x * 512) moments[e] = 0ull;
-    __shared__ float2 s[5][N];  // [pair * 2 + col], then the kernel's two columns as one complex transform
+    constexpr int kKernelSlot = SLIM ? 0 : 4;
+    __shared__ float2 s[SLIM ? 4 : 5][N];  // [pair * 2 + col]; SLIM = false: then the kernel's two columns
     const int tid = threadIdx.x;
     const int c0 = blockIdx.x * 2;
     int v0 = T::frequency(c0), v1 = T::frequency(c0 + 1);
     v0 = min(v0, N - v0);
     v1 = min(v1, N - v1);
     const float *k0 = kernel_rows + (size_t)v0 * kNodePad, *k1 = kernel_rows + (size_t)v1 * kNodePad;
-    auto lds_load = [&](int f, int i) { return s[f][i]; };
-    auto lds_store = [&](int f, int i, float2 v) { s[f][i] = v; };
-    mixed_pass_io<N, 800, 8, false>(
-        5, tw, tid, 512,
-        [&](int f, int m) {
-            float2 v = make_float2(0.f, 0.f);
-            if (f < 4) {
-                if (m < G) v = row_spectra[((size_t)(f >> 1) * N + c0 + (f & 1)) * kNodePad + m];
-            } else {
-                const int a = m < N / 2 ? m : N - m;
-                if (a < G) v = make_float2(k0[a], k1[a]);
+    auto lds_load = [&](int f, int i, int) { return s[f][i]; };
+    auto lds_store = [&](int f, int i, int, float2 v) { s[f][i] = v; };
+    auto kernel_column = [&](int m) {
+        const int a = m < N / 2 ? m : N - m;
+        return a < G ? make_float2(k0[a], k1[a]) : make_float2(0.f, 0.f);
+    };
+    auto data_column = [&](int f, int m) {
+        return m < G ? row_spectra[((size_t)(f >> 1) * N + c0 + (f & 1)) * kNodePad + m] : make_float2(0.f, 0.f);
+    };
+    float kreg[10] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if constexpr (SLIM) {
+        mixed_pass_io<N, 800, 8, false>(1, tw, tid, 512, [&](int, int m, int) { return kernel_column(m); }, lds_store);
+        __syncthreads();
+        mixed_pass<N, 100, 10, false>(&s[0][0], 1, tw, tid, 512);
+        mixed_pass<N, 10, 10, false>(&s[0][0], 1, tw, tid, 512);
+        if (tid < 4 * (N / 10)) {  // the thread's butterfly of the first inverse pass: transform tid / 80, tens tid % 80
+            const int f = tid / (N / 10), b = tid - f * (N / 10);
+#pragma unroll
+            for (int j = 0; j < 10; ++j) {
+                const float2 kk = s[0][10 * b + j];
+                kreg[j] = (f & 1) ? kk.y : kk.x;
             }
-            return v;
-        },
-        lds_store);
+        }
+        __syncthreads();
+        mixed_pass_io<N, 800, 8, false>(4, tw, tid, 512, [&](int f, int m, int) { return data_column(f, m); },
+                                        lds_store);
+    } else {
+        mixed_pass_io<N, 800, 8, false>(
+            5, tw, tid, 512, [&](int f, int m, int) { return f < 4 ? data_column(f, m) : kernel_column(m); },
+            lds_store);
+    }
     __syncthreads();
-    mixed_pass<N, 100, 10, false>(&s[0][0], 5, tw, tid, 512);
-    mixed_pass<N, 10, 10, false>(&s[0][0], 5, tw, tid, 512);
+    mixed_pass<N, 100, 10, false>(&s[0][0], SLIM ? 4 : 5, tw, tid, 512);
+    mixed_pass<N, 10, 10, false>(&s[0][0], SLIM ? 4 : 5, tw, tid, 512);
     mixed_pass_io<N, 10, 10, true>(
         4, tw, tid, 512,
-        [&](int f, int i) {
-            const float2 kk = s[4][i], v = s[f][i];
-            const float kv = (f & 1) ? kk.y : kk.x;
+        [&](int f, int i, int j) {
+            const float2 v = s[f][i];
+            float kv;
+            if constexpr (SLIM) {
+                kv = kreg[j];
+            } else {
+                const float2 kk = s[kKernelSlot][i];
+                kv = (f & 1) ? kk.y : kk.x;
+            }
             return make_float2(v.x * kv, v.y * kv);
         },
         lds_store);
     __syncthreads();
     mixed_pass<N, 100, 10, true>(&s[0][0], 4, tw, tid, 512);
-    mixed_pass_io<N, 800, 8, true>(4, tw, tid, 512, lds_load, [&](int f, int m, float2 v) {
+    mixed_pass_io<N, 800, 8, true>(4, tw, tid, 512, lds_load, [&](int f, int m, int, float2 v) {
         if (m < G) col_results[((size_t)(f >> 1) * N + c0 + (f & 1)) * kNodePad + m] = v;
     });
 }
@@ -1271,9 +1301,12 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     static const int slim_mode = getenv("TSNE_SLIM_COLUMNS") ? atoi(getenv("TSNE_SLIM_COLUMNS")) : -1;
     const bool slim = slim_mode < 0 ? (p->blocked_ready && p->strip_rows >= 1024) : slim_mode == 1;
     const int moment_words = kMoments * nb * nb;
-    if (short_fft)  // (five transforms of 800 points are the 32 KB the slim form exists for)
-        conv_columns_short_kernel<<<kFftShort / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles_short,
-                                                                p->col_results, p->box_moments, moment_words);
+    if (short_fft && slim)
+        conv_columns_short_kernel<true><<<kFftShort / 2, 512, 0, s>>>(
+            p->row_spectra, G, p->kernel_rows, p->twiddles_short, p->col_results, p->box_moments, moment_words);
+    else if (short_fft)
+        conv_columns_short_kernel<false><<<kFftShort / 2, 512, 0, s>>>(
+            p->row_spectra, G, p->kernel_rows, p->twiddles_short, p->col_results, p->box_moments, moment_words);
     else if (slim)
         conv_columns_kernel<true, kFft><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
                                                                  p->col_results, p->box_moments, moment_words);
