@@ -199,8 +199,8 @@ def main():
 
     # ---- every phase against its roofline -----------------------------------
     # Algorithmic bytes per launch of the loop's kernels (G = 390 interpolation nodes per side, four charge
-    # planes; the transposed spectra are 2 plane pairs x 1024 x 512 complex; 21 fixed-point moments per box).
-    G2, spectra, moments = 390.0 * 390.0, 2 * 1024 * 512 * 8.0, 21 * 130 * 130 * 8.0
+    # planes; the transposed spectra are 2 plane pairs x 800 x 512 complex; 21 fixed-point moments per box).
+    G2, spectra, moments = 390.0 * 390.0, 2 * 800 * 512 * 8.0, 21 * 130 * 130 * 8.0
     loop_bytes = {
         "tile_count_kernel": 12.0 * n,                      # positions in, (tile, rank) codes out
         "tile_scatter_kernel": 20.0 * n,                    # positions and codes in, positions grouped by tile out
