@@ -103,7 +103,13 @@ constexpr int kSingleStreamPoints = 65536;
 // TSNE_OVERLAP: 0 never, 1 always, unset: by the size of the problem.
 static bool overlap_enabled(const tsne_hip_plan *p) {
     const char *v = std::getenv("TSNE_OVERLAP");  // read on every call, like TSNE_GRAPH
-    return v ? v[0] != '0' : p->num_points > kSingleStreamPoints;
+    // (the direct form of the attractive kernel gathers its positions from memory, as the chain's spreading and
+    // gathering kernels do theirs, and from about seven million points on each of them slows the others down by
+    // more than the overlap hides: ms per step on two streams / on one - 4 M points 1.01 / 1.03, 6 M 1.58 / 1.61,
+    // 8 M 2.54 / 2.44, 10 M 3.70 / 3.37)
+    constexpr int kDirectOverlapPoints = 7000000;
+    return v ? v[0] != '0'
+             : (p->num_points > kSingleStreamPoints && !(p->blocked_direct && p->num_points > kDirectOverlapPoints));
 }
 
 // Overlapped form: a step's repulsive chain and its attractive kernel run on two streams, the update behind the
