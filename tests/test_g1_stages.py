@@ -462,6 +462,38 @@ def test_grid_size_changes_between_steps(stages, c0_problem):
                                                  float("nan"))] == [130, 130, 130, 130, 140, 140, 150, 170, 170, 130]
 
 
+def test_convolution_forms(stages, c0_problem, monkeypatch):
+    """The repulsive convolution runs on 800-point transforms where the padded grid fits (up to 133 boxes) and on
+    1024-point ones otherwise, and its column pass keeps the kernel's columns in LDS beside the data or in
+    registers: the two column passes give the same bits at either length, the two lengths the same node
+    potentials to fp32 round-off, and every form follows the oracle."""
+    c = c0_problem
+    n = c["X"].shape[0]
+    rng = np.random.default_rng(77)
+    y = (rng.standard_normal(2 * n) * 6).astype(np.float32)
+    rep_o, z_o, _, yt_o, _ = oracle.repulsive(y, nb=130, details=True)
+    yt_o = np.asarray(yt_o).reshape(-1, 4)
+    plan = stages.Plan(n, c["K"])
+    got = {}
+    for fft in ("800", "1024"):
+        for slim in ("0", "1"):
+            monkeypatch.setenv("TSNE_FFT", fft)
+            monkeypatch.setenv("TSNE_SLIM_COLUMNS", slim)
+            rep, z, _, yt, _ = plan.repulsive(dev(y), details=True)
+            got[fft, slim] = (rep.cpu().numpy(), float(z), yt.cpu().numpy().reshape(-1, 4))
+            assert rel_l2(got[fft, slim][0], rep_o) <= 1e-4, (fft, slim)
+            assert abs(got[fft, slim][1] - z_o) <= 1e-5 * abs(z_o), (fft, slim)
+    for fft in ("800", "1024"):
+        assert same_bits(got[fft, "0"][0], got[fft, "1"][0]) and got[fft, "0"][1] == got[fft, "1"][1], fft
+        assert same_bits(got[fft, "0"][2], got[fft, "1"][2]), fft
+    assert not same_bits(got["800", "0"][2], got["1024", "0"][2])   # (the switch did switch)
+    for t in range(4):
+        scale = np.abs(yt_o[:, t]).max()
+        assert np.abs(got["800", "0"][2][:, t] - got["1024", "0"][2][:, t]).max() <= 4e-6 * scale, t
+        assert np.abs(got["800", "0"][2][:, t] - yt_o[:, t]).max() <= 4e-6 * scale, t
+    plan.close()
+
+
 @pytest.mark.parametrize("n,d,k,perp", [
     (2, 2, 2, 1.5),         # smallest problem: self plus one neighbour
     (50, 3, 50, 10.0),      # K == N, fewer points than one candidate tile

@@ -1282,7 +1282,8 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
                                                            p->moment_scale, p->box_moments, keep);
     TSNE_LAUNCHED(s);
     // Transform length: 800 points where the padded grid (2 G - 1) fits, else 1024 (TSNE_FFT=1024 forces the latter).
-    static const bool long_only = getenv("TSNE_FFT") && atoi(getenv("TSNE_FFT")) == kFft;
+    const char *fft_env = getenv("TSNE_FFT");  // (read on every call, like the column pass's switch below)
+    const bool long_only = fft_env && atoi(fft_env) == kFft;
     const bool short_fft = 2 * G - 1 <= kFftShort && !long_only;
     const int row_grid = xcd_launch_blocks(div_up(G, 2));
     const double from_fixed = 1.0 / p->moment_scale;
@@ -1298,7 +1299,8 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
             p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
-    static const int slim_mode = getenv("TSNE_SLIM_COLUMNS") ? atoi(getenv("TSNE_SLIM_COLUMNS")) : -1;
+    const char *slim_env = getenv("TSNE_SLIM_COLUMNS");
+    const int slim_mode = slim_env ? atoi(slim_env) : -1;
     const bool slim = slim_mode < 0 ? (p->blocked_ready && p->strip_rows >= 1024) : slim_mode == 1;
     const int moment_words = kMoments * nb * nb;
     if (short_fft && slim)
