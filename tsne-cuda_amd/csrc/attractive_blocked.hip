@@ -483,33 +483,6 @@ __global__ __launch_bounds__(kBlock, 8) void attractive_blocked_kernel(const flo
     if (gave_up && tid == 0) atomicAdd(&scalars->wait_timeouts, 1u);
 }
 
-// How many (strip, partition) runs the pattern has: per strip the partitions it references, summed into *runs.
-__global__ __launch_bounds__(kBlock) void count_runs_kernel(const int *__restrict__ idx, int K,
-                                                            const int *__restrict__ strip_row0,
-                                                            unsigned long long *__restrict__ runs) {
-    __shared__ unsigned int seen[kMaxParts / 32];
-    __shared__ unsigned int total;
-    const int tid = threadIdx.x;
-    const int row0 = strip_row0[blockIdx.x];
-    const unsigned int count = (unsigned int)(strip_row0[blockIdx.x + 1] - row0) * (unsigned int)K;
-    const size_t base = (size_t)row0 * K;
-    for (int w = tid; w < kMaxParts / 32; w += kBlock) seen[w] = 0u;
-    if (tid == 0) total = 0u;
-    __syncthreads();
-    for (unsigned int e = tid; e < count; e += kBlock) {
-        const unsigned int part = (unsigned int)idx[base + e] / kPartPoints;
-        const unsigned int bit = 1u << (part & 31u);
-        if (!(seen[part >> 5] & bit)) atomicOr(&seen[part >> 5], bit);
-    }
-    __syncthreads();
-    unsigned int mine = 0u;
-    for (int w = tid; w < kMaxParts / 32; w += kBlock) mine += __popc(seen[w]);
-    mine = (unsigned int)group_sum<kWave>((float)mine);  // (at most 8192: exact in a float)
-    if ((tid & (kWave - 1)) == 0) atomicAdd(&total, mine);
-    __syncthreads();
-    if (tid == 0) atomicAdd(runs, (unsigned long long)total);
-}
-
 // ---------------------------------------------------------------------------
 // Preparation of the direct form.  Sort key of an entry: (row within strip) << 40 | strip << 24 | column; the
 // sort orders by the low 24 + strip bits, i.e. by (strip, column), and is stable.  A strip's entries then are the
@@ -765,7 +738,6 @@ static_assert(kBlockedLds <= 160 * 1024, "one workgroup must fit the 160 KB of L
 namespace {
 
 constexpr int kMicroRows = 64;
-constexpr double kDirectRunEntries = 1000.0;  // mean entries per (strip, partition) run below which the direct form runs
 constexpr long long kPartCostEntries = 2000;
 
 __global__ __launch_bounds__(256) void micro_strip_parts_kernel(const int *__restrict__ idx, int N, int K, int words,
@@ -944,26 +916,14 @@ int prepare_blocked(tsne_hip_plan *p, const float *pij, const int *indices, hipS
         set_error("attractive_prepare: out of device memory for the strip boundaries");
         return 1;
     }
-    // Which form: the direct one where the runs are short.  (TSNE_ATTRACTIVE_FORM=staged / direct overrides.)
+    // Which form: the direct one where the strips outnumber the compute units, so that the staged form would run
+    // them in rounds.  (TSNE_ATTRACTIVE_FORM=staged / direct overrides.)  Measured, ms per step staged / direct,
+    // four clusters of 50 dimensions, K = 90: 1.00 M points (252 strips) 0.214 / 0.235; 1.05 M 0.318 / 0.258;
+    // 1.2 M 0.341 / 0.283; 1.5 M 0.458 / 0.336; 2 M 0.554 / 0.475; 3 M 0.945 / 0.705; 10 M 6.4 / 3.4 (there a
+    // strip's runs are 290 entries long, and staging 16 KB for each is seven times the entries' own traffic).
+    // Fits of 50000 to 60000 points, whose strips all run at once, were 2 % slower in the direct form.
     {
-        unsigned long long *d_runs = nullptr, runs = 0;
-        hipError_t e = hipMalloc(&d_runs, sizeof(runs));
-        if (e == hipSuccess) e = hipMemsetAsync(d_runs, 0, sizeof(runs), s);
-        if (e == hipSuccess) {
-            count_runs_kernel<<<p->n_strips, kBlock, 0, s>>>(indices, K, p->strip_row0, d_runs);
-            e = hipGetLastError();
-        }
-        if (e == hipSuccess) e = hipMemcpyAsync(&runs, d_runs, sizeof(runs), hipMemcpyDeviceToHost, s);
-        if (e == hipSuccess) e = hipStreamSynchronize(s);
-        (void)hipFree(d_runs);
-        if (e != hipSuccess) {
-            release_blocked(p);
-            TSNE_TRY(e);
-        }
-        const double run_entries = (double)N * K / (double)std::max<unsigned long long>(runs, 1ull);
-        // (measured: ten million points in four clusters, 290 entries per run: 2.6 ms per launch against 6.0 ms
-        // staged; fits of 50000 to 60000 points, 350 to 700 entries per run, whose strips all run at once: 2 % slower)
-        p->blocked_direct = run_entries < kDirectRunEntries && p->n_strips > cus;
+        p->blocked_direct = p->n_strips > cus;
         if (const char *v = std::getenv("TSNE_ATTRACTIVE_FORM")) p->blocked_direct = v[0] == 'd';
         // (the direct form's keys hold 24 bits of column and 16 of strip; its sort counts in 31 bits)
         // (strips that are not all of one length are at most as many as the compute units)
