@@ -12,9 +12,10 @@
 //   * charges, box indices and Lagrange weights are recomputed in registers
 //     instead of being stored (src/kernels/nbodyfft.cu:43-105,
 //     src/kernels/rep_forces.cu:57-76);
-//   * the convolution zero-pads to 1024 and runs as in-place radix-4 FFTs in
-//     LDS: a decimation-in-frequency forward transform leaves its output in
-//     base-4 digit-reversed order, the decimation-in-time inverse consumes that
+//   * the convolution zero-pads to 800 points (grids of up to 133 boxes per
+//     side) or 1024 and runs as in-place mixed-radix FFTs in LDS: a
+//     decimation-in-frequency forward transform leaves its output in
+//     digit-reversed order, the decimation-in-time inverse consumes that
 //     order, so nothing is ever permuted.  Two real charge planes ride in one
 //     complex transform; the kernel is real and even, so its spectrum is real
 //     and the planes never mix.  fp32 round-off does leak between the two
@@ -30,7 +31,7 @@ namespace tsnehip {
 namespace {
 
 constexpr int kLog2Fft = 10;
-constexpr int kRowThreads = 512;  // threads of a row-pass workgroup (four transforms of 1024 points)
+constexpr int kRowThreads = 512;  // threads of a row-pass workgroup (four transforms)
 
 __device__ __forceinline__ int rev4(int x) {
     // Reverse the five base-4 digits of a 10-bit index.
@@ -800,7 +801,7 @@ __global__ __launch_bounds__(kSpreadThreads, 4) void spread_kernel(const float2 
 // Kernel rows: for node offsets a in [0, G) transform the even sequence
 // b -> k(a, |b|) = (1 + (a h)^2 + (b h)^2)^-2 (src/kernels/nbodyfft.cu:175-203)
 // along b.  Two rows share one complex transform (both spectra are real).
-// Output kernel_rows[v][a] for frequencies v in [0, 512].
+// Output kernel_rows[v][a] for frequencies v in [0, n / 2], n the transform length.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float kernel_value(float lo, float h, int a, int b) {
 #pragma clang fp contract(off)
@@ -1114,7 +1115,7 @@ __global__ __launch_bounds__(512) void conv_columns_short_kernel(const float2 *_
 
 // ---------------------------------------------------------------------------
 // Inverse row pass for x nodes m0, m0+1: consumes digit-reversed positions,
-// produces node potentials in natural order, scaled by 1/1024^2.
+// produces node potentials in natural order, scaled by 1 / (transform length)^2.
 // ---------------------------------------------------------------------------
 template <int NFFT>
 __global__ __launch_bounds__(kRowThreads) void conv_rows_inverse_kernel(const float2 *__restrict__ col_results, int G,
