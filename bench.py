@@ -166,8 +166,8 @@ def main():
     ms_per_step = loop_s * 1e3 / args.steps
     iters_per_s = args.steps / loop_s
 
-    # ---- per-kernel durations: HIP events on the loop's stream, recorded by
-    # the library around every kernel of a further stretch of the same loop ----
+    # ---- per-kernel durations: a pair of HIP events per launch (the kernel's own start and end), handed to
+    # every kernel of a further stretch of the same loop by the library ----
     prof_steps = min(args.steps, 200)
     plan.profile_begin()
     plan.iterate_(None, None, y, gains, old, done, done + prof_steps, eta=eta)
@@ -193,7 +193,7 @@ def main():
         late_runs.append(run_s)
         done += args.steps
     late_s = sorted(late_runs)[len(late_runs) // 2]
-    attr_ms = kernels_us["attractive_kernel"] * 1e-3  # profiling slot of whichever attractive kernel ran
+    attr_ms = kernels_us["attractive_kernel"] * 1e-3  # start-to-end events of whichever attractive kernel ran
     attr_bytes = 8.0 * n * k + 16.0 * n  # P and index streams; read positions, write forces
     achieved = attr_bytes / (attr_ms * 1e-3) / 1e9
 

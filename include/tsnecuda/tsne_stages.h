@@ -295,15 +295,17 @@ int tsne_hip_sum_squares(tsne_hip_plan *plan, const float *values, int64_t n, fl
 /* Per-kernel timing of tsne_hip_iterate with HIP events on the loop's own
  * stream (the measured counterpart of the reference's _time_* phase timers,
  * src/fit_tsne.cu:8-14,586-601).  Between profile_begin and profile_end every
- * kernel launch of tsne_hip_iterate is bracketed by events; profile_end waits
- * for them and fills total_ms[k] / launches[k] for k < tsne_hip_profile_kernel_count(). */
+ * kernel launch of tsne_hip_iterate carries a pair of events that receive the
+ * kernel's own start and end (the gaps between launches are not counted);
+ * profile_end waits for them and fills total_ms[k] / launches[k] for
+ * k < tsne_hip_profile_kernel_count(). */
 int tsne_hip_profile_kernel_count(void);
 const char *tsne_hip_profile_kernel_name(int id);
 int tsne_hip_profile_begin(tsne_hip_plan *plan);
 int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches);
 /* The same for the attractive kernel alone while the loop runs as it does unprofiled (its kernels on two
- * streams, the repulsive chain beside the attractive kernel): a pair of events around that one kernel on the
- * stream it is launched on; *total_ms / *launches give its duration beside the chain (no reference counterpart:
+ * streams, the repulsive chain beside the attractive kernel): that one kernel's launches carry the pair of
+ * events; *total_ms / *launches give its duration beside the chain (no reference counterpart:
  * the reference runs its phases one after the other). */
 int tsne_hip_profile_attractive_begin(tsne_hip_plan *plan);
 int tsne_hip_profile_attractive_end(tsne_hip_plan *plan, double *total_ms, int *launches);

@@ -33,17 +33,25 @@ bool sync_kernels_enabled() {
     return enabled;
 }
 
-int profile_mark(tsne_hip_plan *p, int id, hipStream_t s) {
-    if (!p->profiling) return 0;
-    if (p->events_used == p->events.size()) {
+int profile_mark(tsne_hip_plan *p, int id, hipStream_t) {
+    if (p->profiling || (p->profiling_attractive && id == kKernelAttractive)) p->pending_kernel = id;
+    return 0;
+}
+
+int profile_events(tsne_hip_plan *p, hipEvent_t *start, hipEvent_t *stop) {
+    *start = *stop = nullptr;
+    if (!(p->profiling || p->profiling_attractive) || p->pending_kernel < 0) return 0;
+    while (p->events.size() < p->events_used + 2) {
         hipEvent_t e;
         TSNE_TRY(hipEventCreate(&e));
         p->events.push_back(e);
     }
-    TSNE_TRY(hipEventRecord(p->events[p->events_used], s));
-    if (p->event_kernel.size() <= p->events_used) p->event_kernel.resize(p->events_used + 1);
-    p->event_kernel[p->events_used] = id;
-    p->events_used += 1;
+    *start = p->events[p->events_used];
+    *stop = p->events[p->events_used + 1];
+    p->event_kernel.resize(p->events_used / 2 + 1);
+    p->event_kernel[p->events_used / 2] = p->pending_kernel;
+    p->events_used += 2;
+    p->pending_kernel = -1;
     return 0;
 }
 
@@ -129,27 +137,10 @@ static bool overlap_enabled(const tsne_hip_plan *p) {
 // dependencies whichever stream they were recorded on and runs as before.)
 // Attractive forces of a step: the explicit N x K pattern if given, else the plan's CSR pattern if one is set,
 // else the re-blocked pattern.
-static int attractive_mark(tsne_hip_plan *p, hipStream_t s) {
-    if (!p->profiling_attractive) return 0;
-    if (p->attractive_events_used == p->attractive_events.size()) {
-        hipEvent_t e;
-        TSNE_TRY(hipEventCreate(&e));
-        p->attractive_events.push_back(e);
-    }
-    TSNE_TRY(hipEventRecord(p->attractive_events[p->attractive_events_used++], s));
-    return 0;
-}
-
 static int launch_step_attractive(tsne_hip_plan *p, const float *pij, const int *indices, hipStream_t s) {
-    if (attractive_mark(p, s)) return 1;
-    int rc;
-    if (pij)
-        rc = launch_attractive(p, pij, indices, p->attr, s);
-    else if (p->csr_row_ptr)
-        rc = launch_attractive_csr(p, p->csr_row_ptr, p->csr_col_idx, p->csr_values, p->attr, s);
-    else
-        rc = launch_attractive_blocked(p, p->attr, s);
-    return rc || attractive_mark(p, s);
+    if (pij) return launch_attractive(p, pij, indices, p->attr, s);
+    if (p->csr_row_ptr) return launch_attractive_csr(p, p->csr_row_ptr, p->csr_col_idx, p->csr_values, p->attr, s);
+    return launch_attractive_blocked(p, p->attr, s);
 }
 
 static bool overlap_active(const tsne_hip_plan *p) {
@@ -368,7 +359,6 @@ void tsne_hip_plan_destroy(tsne_hip_plan *p) {
     if (p->side_stream) (void)hipStreamSynchronize(p->side_stream);
     (void)hipDeviceSynchronize();
     for (hipEvent_t e : p->events) (void)hipEventDestroy(e);
-    for (hipEvent_t e : p->attractive_events) (void)hipEventDestroy(e);
     if (p->fork_event) (void)hipEventDestroy(p->fork_event);
     if (p->join_event) (void)hipEventDestroy(p->join_event);
     for (auto &g : p->step_graphs) (void)hipGraphExecDestroy(g.exec);
@@ -625,6 +615,7 @@ int tsne_hip_profile_begin(tsne_hip_plan *plan) {
     if (check_plan(plan, "profile_begin")) return 1;
     plan->profiling = true;
     plan->events_used = 0;
+    plan->pending_kernel = -1;
     return 0;
 }
 
@@ -637,10 +628,10 @@ int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches) {
         launches[k] = 0;
     }
     if (plan->events_used == 0) return 0;
+    // (the loop's stream is in order and the last timed kernel is its last: when that one has ended, all have)
     TSNE_TRY(hipEventSynchronize(plan->events[plan->events_used - 1]));
-    for (size_t e = 0; e + 1 < plan->events_used; ++e) {
-        const int id = plan->event_kernel[e];
-        if (id < 0) continue;
+    for (size_t e = 0; e + 1 < plan->events_used; e += 2) {
+        const int id = plan->event_kernel[e / 2];
         float ms = 0.0f;
         TSNE_TRY(hipEventElapsedTime(&ms, plan->events[e], plan->events[e + 1]));
         total_ms[id] += ms;
@@ -653,7 +644,8 @@ int tsne_hip_profile_end(tsne_hip_plan *plan, double *total_ms, int *launches) {
 int tsne_hip_profile_attractive_begin(tsne_hip_plan *plan) {
     if (check_plan(plan, "profile_attractive_begin")) return 1;
     plan->profiling_attractive = true;
-    plan->attractive_events_used = 0;
+    plan->events_used = 0;
+    plan->pending_kernel = -1;
     return 0;
 }
 
@@ -663,13 +655,14 @@ int tsne_hip_profile_attractive_end(tsne_hip_plan *plan, double *total_ms, int *
     plan->profiling_attractive = false;
     *total_ms = 0.0;
     *launches = 0;
-    const size_t used = plan->attractive_events_used;
-    plan->attractive_events_used = 0;
+    const size_t used = plan->events_used;
+    plan->events_used = 0;
     if (used < 2) return 0;
-    TSNE_TRY(hipEventSynchronize(plan->attractive_events[used - 1]));
+    // (every attractive kernel ends before the update of its step starts, and the updates are in sequence)
+    TSNE_TRY(hipEventSynchronize(plan->events[used - 1]));
     for (size_t e = 0; e + 1 < used; e += 2) {
         float ms = 0.0f;
-        TSNE_TRY(hipEventElapsedTime(&ms, plan->attractive_events[e], plan->attractive_events[e + 1]));
+        TSNE_TRY(hipEventElapsedTime(&ms, plan->events[e], plan->events[e + 1]));
         *total_ms += ms;
         *launches += 1;
     }

@@ -123,8 +123,8 @@ int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, fl
     const int N = p->num_points, K = p->num_neighbors;
     if (profile_mark(p, kKernelAttractive, s)) return 1;
 #define TSNE_ATTR(LANES, SLOTS, ROWS)                                                              \
-    attractive_kernel<LANES, SLOTS, ROWS><<<div_up(N, (256 / LANES) * ROWS), 256, 0, s>>>(pij, indices, p->yxy, \
-                                                                                          attr, N, K)
+    TSNE_LOOP_KERNEL(p, (attractive_kernel<LANES, SLOTS, ROWS>), div_up(N, (256 / LANES) * ROWS), 256, 0, s, pij,  \
+                     indices, p->yxy, attr, N, K)
     if (K <= 16) {
         TSNE_ATTR(16, 1, 8);
     } else if (K <= 32) {
@@ -138,7 +138,7 @@ int launch_attractive(tsne_hip_plan *p, const float *pij, const int *indices, fl
     } else if (K <= 256) {
         TSNE_ATTR(64, 4, 2);
     } else {
-        attractive_generic_kernel<64><<<div_up(N, 256 / 64), 256, 0, s>>>(pij, indices, p->yxy, attr, N, K);
+        TSNE_LOOP_KERNEL(p, (attractive_generic_kernel<64>), div_up(N, 256 / 64), 256, 0, s, pij, indices, p->yxy, attr, N, K);
     }
 #undef TSNE_ATTR
     TSNE_LAUNCHED(s);

@@ -1006,13 +1006,12 @@ int launch_attractive_blocked(tsne_hip_plan *p, float *attr, hipStream_t s) {
     if (p->blocked_direct) {
         // (LDS for the longest strip only: what is left of a compute unit's 160 KB hosts the repulsive chain's kernels)
         const int rows_cap = (p->strip_rows + kWave - 1) / kWave * kWave;
-        attractive_direct_kernel<<<p->n_strips, kDirectThreads, (size_t)24 * rows_cap, s>>>(
-            p->ent_p, p->wseg, p->yxy, p->scalars, attr, p->num_points, p->num_neighbors, p->wseg_stride, rows_cap);
+        TSNE_LOOP_KERNEL(p, (attractive_direct_kernel), p->n_strips, kDirectThreads, (size_t)24 * rows_cap, s, p->ent_p, p->wseg, p->yxy, p->scalars, attr, p->num_points, p->num_neighbors, p->wseg_stride, rows_cap);
         TSNE_LAUNCHED(s);
         return 0;
     }
     const auto kernel = p->spin_limit == kSpinLimit ? attractive_blocked_kernel<false> : attractive_blocked_kernel<true>;
-    kernel<<<p->n_strips, kBlock, kBlockedLds, s>>>(p->ent_p, p->seg, p->yxy, p->scalars, attr, p->num_points,
+    TSNE_LOOP_KERNEL(p, (kernel), p->n_strips, kBlock, kBlockedLds, s, p->ent_p, p->seg, p->yxy, p->scalars, attr, p->num_points,
                                                     p->num_neighbors, p->list_words, p->seg_stride,
                                                     p->spin_limit);
     TSNE_LAUNCHED(s);

@@ -4,6 +4,8 @@
 
 #include <vector>
 
+#include <hip/hip_ext.h>
+
 #include "common.h"
 
 namespace tsnehip {
@@ -135,24 +137,40 @@ struct tsne_hip_plan {
     };
     std::vector<StepGraph> step_graphs;
 
-    // Optional per-kernel timing: an event is recorded before every kernel of
-    // the loop and one after the last; a kernel's time is the gap to the next
-    // event on the same in-order stream.
+    // Optional per-kernel timing: every kernel of the loop is launched with a pair of events of its own that
+    // receive its start and its end (hipExtLaunchKernelGGL), so a kernel's time is its own duration, without the
+    // gaps between launches.  profile_mark names the kernel that the next launch belongs to.
     bool profiling = false;
-    std::vector<hipEvent_t> events;
-    std::vector<int> event_kernel;  // kernel id per recorded event, -1 = end marker
-    size_t events_used = 0;
+    std::vector<hipEvent_t> events;  // pairs: start, stop
+    std::vector<int> event_kernel;   // kernel id per pair
+    size_t events_used = 0;          // events handed out (two per timed launch)
+    int pending_kernel = -1;         // set by profile_mark, consumed by the next launch
     // The other mode: the loop runs as it does unprofiled (two streams), and only the attractive kernel is
-    // bracketed by a pair of events on the stream it is launched on (its duration beside the repulsive chain).
+    // launched with a pair of events (its duration beside the repulsive chain).
     bool profiling_attractive = false;
-    std::vector<hipEvent_t> attractive_events;
-    size_t attractive_events_used = 0;
 };
 
 namespace tsnehip {
 
-// Records a profiling event for kernel `id` (no-op unless profiling is on).
+// Names the kernel (`id`, or -1 for none) that the next TSNE_LOOP_KERNEL launch is timed as (no-op unless
+// profiling is on).
 int profile_mark(tsne_hip_plan *p, int id, hipStream_t s);
+// The pair of events for the launch that follows a profile_mark (both null when that launch is not timed).
+int profile_events(tsne_hip_plan *p, hipEvent_t *start, hipEvent_t *stop);
+
+// Launch of one of the loop's kernels from a function that returns an int status and has the plan at hand.
+#define TSNE_LOOP_KERNEL(plan_, kernel_, grid_, block_, lds_, stream_, ...)                                       \
+    do {                                                                                                         \
+        hipEvent_t start_ = nullptr, stop_ = nullptr;                                                            \
+        if (((plan_)->profiling || (plan_)->profiling_attractive) &&                                             \
+            ::tsnehip::profile_events(plan_, &start_, &stop_))                                                   \
+            return 1;                                                                                            \
+        if (start_)                                                                                              \
+            hipExtLaunchKernelGGL(kernel_, dim3(grid_), dim3(block_), (std::uint32_t)(lds_), stream_, start_,     \
+                                  stop_, 0, __VA_ARGS__);                                                        \
+        else                                                                                                     \
+            hipLaunchKernelGGL(kernel_, dim3(grid_), dim3(block_), (std::uint32_t)(lds_), stream_, __VA_ARGS__);  \
+    } while (0)
 
 // Stage launchers shared between the stage-level ABI and the fused loop.
 // `slot` selects which pair of bounds in LoopScalars the launch reads.

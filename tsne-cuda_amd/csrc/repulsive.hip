@@ -1264,12 +1264,12 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     // (one point per thread until that many workgroups are in use)
     const int sort_blocks = std::min(div_up(N, 1024), kSortBlocks);
     if (profile_mark(p, kKernelTileCount, s)) return 1;
-    tile_count_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, p->scalars, slot, slot ^ 1, nb, p->tile_count,
+    TSNE_LOOP_KERNEL(p, (tile_count_kernel), sort_blocks, 1024, 0, s, embedding, N, p->scalars, slot, slot ^ 1, nb, p->tile_count,
                                                    p->tile_cursor, p->chunks, p->num_chunks, p->num_chunks + 1,
                                                    p->point_code, p->wg_tile_base, keep);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelTileScatter, s)) return 1;
-    tile_scatter_kernel<<<sort_blocks, 1024, 0, s>>>(embedding, N, tiles_per_dim * tiles_per_dim, p->tile_cursor,
+    TSNE_LOOP_KERNEL(p, (tile_scatter_kernel), sort_blocks, 1024, 0, s, embedding, N, tiles_per_dim * tiles_per_dim, p->tile_cursor,
                                                      p->point_code, p->wg_tile_base, p->tile_xy, p->tile_perm,
                                                      p->scalars, keep);
     TSNE_LAUNCHED(s);
@@ -1278,7 +1278,7 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     // than workgroups the surplus ones exit at once).
     const int spread_blocks =
         xcd_launch_blocks(std::min(N / kChunkPoints + tiles_per_dim * tiles_per_dim + 1, p->spread_grid));
-    spread_kernel<<<spread_blocks, kSpreadThreads, 0, s>>>(p->tile_xy, p->tile_perm, p->yxy, p->chunks,
+    TSNE_LOOP_KERNEL(p, (spread_kernel), spread_blocks, kSpreadThreads, 0, s, p->tile_xy, p->tile_perm, p->yxy, p->chunks,
                                                            p->num_chunks, p->scalars, slot, slot ^ 1, nb,
                                                            p->moment_scale, p->box_moments, keep);
     TSNE_LAUNCHED(s);
@@ -1291,12 +1291,10 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     float4 *charges4 = reinterpret_cast<float4 *>(charges_out);
     if (profile_mark(p, kKernelConvRowsForward, s)) return 1;
     if (short_fft)
-        conv_rows_forward_kernel<2, kFftShort><<<row_grid + div_up(G, 8), 512, 0, s>>>(
-            p->box_moments, from_fixed, p->monomials, charges4, G, nb, p->scalars, slot, p->twiddles_short,
+        TSNE_LOOP_KERNEL(p, (conv_rows_forward_kernel<2, kFftShort>), row_grid + div_up(G, 8), 512, 0, s, p->box_moments, from_fixed, p->monomials, charges4, G, nb, p->scalars, slot, p->twiddles_short,
             p->row_spectra, p->kernel_rows);
     else
-        conv_rows_forward_kernel<2, kFft><<<row_grid + div_up(G, 8), 512, 0, s>>>(
-            p->box_moments, from_fixed, p->monomials, charges4, G, nb, p->scalars, slot, p->twiddles, p->row_spectra,
+        TSNE_LOOP_KERNEL(p, (conv_rows_forward_kernel<2, kFft>), row_grid + div_up(G, 8), 512, 0, s, p->box_moments, from_fixed, p->monomials, charges4, G, nb, p->scalars, slot, p->twiddles, p->row_spectra,
             p->kernel_rows);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvColumns, s)) return 1;
@@ -1305,28 +1303,26 @@ int launch_repulsive(tsne_hip_plan *p, const float *embedding, int slot, float *
     const bool slim = slim_mode < 0 ? (p->blocked_ready && p->strip_rows >= 1024) : slim_mode == 1;
     const int moment_words = kMoments * nb * nb;
     if (short_fft && slim)
-        conv_columns_short_kernel<true><<<kFftShort / 2, 512, 0, s>>>(
-            p->row_spectra, G, p->kernel_rows, p->twiddles_short, p->col_results, p->box_moments, moment_words);
+        TSNE_LOOP_KERNEL(p, (conv_columns_short_kernel<true>), kFftShort / 2, 512, 0, s, p->row_spectra, G, p->kernel_rows, p->twiddles_short, p->col_results, p->box_moments, moment_words);
     else if (short_fft)
-        conv_columns_short_kernel<false><<<kFftShort / 2, 512, 0, s>>>(
-            p->row_spectra, G, p->kernel_rows, p->twiddles_short, p->col_results, p->box_moments, moment_words);
+        TSNE_LOOP_KERNEL(p, (conv_columns_short_kernel<false>), kFftShort / 2, 512, 0, s, p->row_spectra, G, p->kernel_rows, p->twiddles_short, p->col_results, p->box_moments, moment_words);
     else if (slim)
-        conv_columns_kernel<true, kFft><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
+        TSNE_LOOP_KERNEL(p, (conv_columns_kernel<true, kFft>), kFft / 2, 512, 0, s, p->row_spectra, G, p->kernel_rows, p->twiddles,
                                                                  p->col_results, p->box_moments, moment_words);
     else
-        conv_columns_kernel<false, kFft><<<kFft / 2, 512, 0, s>>>(p->row_spectra, G, p->kernel_rows, p->twiddles,
+        TSNE_LOOP_KERNEL(p, (conv_columns_kernel<false, kFft>), kFft / 2, 512, 0, s, p->row_spectra, G, p->kernel_rows, p->twiddles,
                                                                   p->col_results, p->box_moments, moment_words);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelConvRowsInverse, s)) return 1;
     if (short_fft)
-        conv_rows_inverse_kernel<kFftShort><<<row_grid, kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot,
+        TSNE_LOOP_KERNEL(p, (conv_rows_inverse_kernel<kFftShort>), row_grid, kRowThreads, 0, s, p->col_results, G, p->scalars, slot,
                                                                             p->twiddles_short, p->node_potentials);
     else
-        conv_rows_inverse_kernel<kFft><<<row_grid, kRowThreads, 0, s>>>(p->col_results, G, p->scalars, slot,
+        TSNE_LOOP_KERNEL(p, (conv_rows_inverse_kernel<kFft>), row_grid, kRowThreads, 0, s, p->col_results, G, p->scalars, slot,
                                                                        p->twiddles, p->node_potentials);
     TSNE_LAUNCHED(s);
     if (profile_mark(p, kKernelGather, s)) return 1;
-    gather_forces_kernel<<<std::min(div_up(N, 256), 1024), 256, 0, s>>>(embedding, N, p->scalars, slot, nb, p->lagrange,
+    TSNE_LOOP_KERNEL(p, (gather_forces_kernel), std::min(div_up(N, 256), 1024), 256, 0, s, embedding, N, p->scalars, slot, nb, p->lagrange,
                                                         p->node_potentials, rep, point_potentials, p->scalars, keep,
                                                         p->z_scale);
     TSNE_LAUNCHED(s);

@@ -484,7 +484,7 @@ int symmetrize_full(const float *p, const int *idx, int N, int K, int *row_ptr, 
 int launch_attractive_csr(tsne_hip_plan *p, const int *row_ptr, const int *col_idx, const float *values, float *attr,
                           hipStream_t s) {
     if (profile_mark(p, kKernelAttractive, s)) return 1;
-    attractive_csr_kernel<<<div_up(p->num_points, 256 / kWave), 256, 0, s>>>(row_ptr, col_idx, values, p->yxy,
+    TSNE_LOOP_KERNEL(p, (attractive_csr_kernel), div_up(p->num_points, 256 / kWave), 256, 0, s, row_ptr, col_idx, values, p->yxy,
                                                                              p->num_points, attr);
     TSNE_LAUNCHED(s);
     return 0;

@@ -300,11 +300,11 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
         // 512 25 us, one item per thread (977 workgroups) 39 us.
         const int blocks = std::min(std::min(div_up(N / 4, 256), p->stream_grid), kMaxCentreParts);
         if (next_slot >= 0) {
-            update_vec4_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
+            TSNE_LOOP_KERNEL(p, (update_vec4_kernel<true>), blocks, 256, 0, s, embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
                                                             momentum, exaggeration, p->yxy, p->scalars,
                                                             p->centre_parts, next_slot, p->recenter ? 1 : 0);
         } else {
-            update_vec4_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
+            TSNE_LOOP_KERNEL(p, (update_vec4_kernel<false>), blocks, 256, 0, s, embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
                                                              momentum, exaggeration, nullptr, p->scalars, nullptr, 0, 0);
         }
         TSNE_LAUNCHED(s);
@@ -312,11 +312,11 @@ int launch_update(tsne_hip_plan *p, float *embedding, float *attr, float *rep, f
     }
     const int blocks = std::min(std::min(div_up(N, 256), 4 * p->stream_grid), kMaxCentreParts);  // 4-byte accesses: the same window
     if (next_slot >= 0) {
-        update_kernel<true><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
+        TSNE_LOOP_KERNEL(p, (update_kernel<true>), blocks, 256, 0, s, embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
                                                    momentum, exaggeration, p->yxy, p->scalars, p->centre_parts, next_slot,
                                                    p->recenter ? 1 : 0);
     } else {
-        update_kernel<false><<<blocks, 256, 0, s>>>(embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
+        TSNE_LOOP_KERNEL(p, (update_kernel<false>), blocks, 256, 0, s, embedding, attr, rep, gains, old_forces, N, eta, z_ptr, z_inv,
                                                     momentum, exaggeration, nullptr, p->scalars, nullptr, 0, 0);
     }
     TSNE_LAUNCHED(s);
